@@ -1,0 +1,143 @@
+/*
+ * ll_nvfp4.h — C ABI of the MI355X (gfx950) NVFP4 inference hot path.
+ *
+ * Every entry point takes raw device pointers, sizes and a HIP stream (as void*),
+ * launches on that stream, allocates nothing and returns 0 on success or a negative
+ * LL_E* code; ll_last_error() gives the message for the calling thread.  All tensors
+ * are row-major.  "bf16" means the 16-bit bit pattern.  Pointers must be valid on
+ * the current HIP device.
+ *
+ * NVFP4 tensor format (what the reference's QuantizedTensor carries):
+ *   values  u8 [Mp, Kp/2]     byte j of a row = code[2j] | code[2j+1] << 4  (e2m1 codes)
+ *   scales  u8 [Mp * Kp/16]   e4m3fn block scales in the 128x4 "blocked" order:
+ *                             off(r, c) = ((r/128 * (Kp/64) + c/4) * 32 + r%32) * 16 + (r%128)/32 * 4 + c%4
+ *   amax    f32[1]            tensor-wide max |x|
+ *   Mp = M rounded up to 128, Kp = K rounded up to 64.
+ *
+ * Scale-rule ids are the reference's (fouroversix/src/fouroversix/utils.py:113-122).
+ */
+#ifndef LL_NVFP4_H
+#define LL_NVFP4_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  LL_OK = 0,
+  LL_EINVAL = -1,   /* bad shape / pointer / option */
+  LL_ELAUNCH = -2,  /* HIP reported an error at launch */
+  LL_ENOSUP = -3    /* valid request this build does not implement */
+};
+
+enum { LL_RULE_STATIC_6 = 0, LL_RULE_STATIC_4 = 1, LL_RULE_MAE = 2, LL_RULE_MSE = 3, LL_RULE_ABS_MAX = 4 };
+enum { LL_DTYPE_BF16 = 0, LL_DTYPE_F16 = 1, LL_DTYPE_F32 = 2 }; /* utils/kernel/kv_dequant.py:18-25 */
+
+const char* ll_last_error(void);
+int ll_version(void);
+
+/* Number of floats of scratch ll_nvfp4_quantize needs when it computes amax itself. */
+size_t ll_nvfp4_quantize_workspace_floats(void);
+
+/*
+ * Replaces torch.ops.fouroversix.quantize_to_fp4 (fouroversix/src/fouroversix/csrc/bindings.cpp:28,
+ * csrc/quantize/fp4_quant.cu:99-239) for is_nvfp4, round-to-nearest, no RHT / 2-D / transpose, with
+ * the arithmetic of the PyTorch backend (quantize/pytorch/reference.py:242-368, backend.py:36-112).
+ *   x        bf16 [M, K], row stride ldx elements
+ *   values   u8 [Mp, Kp/2]      every byte written (padding rows/cols quantize zeros)
+ *   scales   u8 [Mp*Kp/16]      every byte written
+ *   amax     f32[1]             written unless amax_given != 0, in which case it is read
+ *   workspace  f32[ll_nvfp4_quantize_workspace_floats()], may be NULL when amax_given != 0
+ */
+int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ldx, int rule,
+                      uint8_t* values, uint8_t* scales, float* amax, int amax_given,
+                      float* workspace, void* stream);
+
+/*
+ * Replaces QuantizedTensor.dequantize (fouroversix/src/fouroversix/quantize/quantized_tensor.py:184-214):
+ * out[r, c] = cast(((e2m1 * e4m3) * amax) / (e2m1_max * e4m3_max)) for r < M, c < K; ldo in elements.
+ */
+int ll_nvfp4_dequantize(const uint8_t* values, const uint8_t* scales, const float* amax, int rule,
+                        int64_t Mp, int64_t Kp, int64_t M, int64_t K,
+                        void* out, int out_dtype, int64_t ldo, void* stream);
+
+/*
+ * Replaces torch.ops.fouroversix.gemm_nvfp4nvfp4_accum_fp32_out_bf16_tnt
+ * (fouroversix/src/fouroversix/csrc/bindings.cpp:31, csrc/fp4_gemm.cu:40-186):
+ *   D[m, n] = bf16(alpha * sum_k deq(A)[m, k] * deq(B)[n, k])  (+ bias[n], added in bf16 like linear.py:73-74)
+ *   A_values u8 [Mp, Kp/2], A_scales blocked [Mp*Kp/16]; B_values u8 [Np, Kp/2], B_scales blocked.
+ *   alpha: device f32[1], or NULL to use (*amax_a * *amax_b) / (denom_a * denom_b) as
+ *          matmul/cutlass/backend.py:81-90 computes it (denom = e2m1_max * e4m3_max of each rule).
+ *   D bf16 [M, N], row stride ldd; only rows < M and columns < N are written (M <= Mp, N <= Np).
+ *   bias bf16 [N] or NULL.
+ */
+int ll_nvfp4_gemm_tnt(const uint8_t* A_values, const uint8_t* A_scales, const uint8_t* B_values,
+                      const uint8_t* B_scales, const float* alpha, const float* amax_a, const float* amax_b,
+                      float denom_a, float denom_b, int64_t M, int64_t N, int64_t Mp, int64_t Np, int64_t Kp,
+                      void* D, int64_t ldd, const void* bias, void* stream);
+
+/*
+ * Replaces torch.ops.longlive_kernels.dequantize_kv_cache_fp4 (utils/kernel/kv_dequant.cpp:14,
+ * utils/kernel/kv_dequant_cuda.cu:59-239) and the Triton fp4_dequantize it falls back to
+ * (utils/nvfp4_kernel.py:40-176): n_blocks cache slots, each NVFP4 [rows_padded, 128] holding
+ * block_token_size*num_heads logical rows, are dequantized to out[1, n_blocks*block_token_size, num_heads, 128]
+ * as f32(e2m1) * f32(scale) * (amax / (e2m1_max*e4m3_max)).
+ *   values_ptrs / scales_ptrs / amax_ptrs: DEVICE arrays of n_blocks device pointers.
+ */
+int ll_kv_dequantize_blocks(const uint64_t* values_ptrs, const uint64_t* scales_ptrs, const uint64_t* amax_ptrs,
+                            int n_blocks, int num_heads, int block_token_size, int out_dtype,
+                            float e2m1_max, float e4m3_max, void* out, void* stream);
+
+/*
+ * FP4 KV-cache attention for one chunk; replaces dequantize_kv_cache + slice copies + flash attention
+ * (wan_5b/modules/causal_model.py:557-567, 628-671, 673-724, 781; wan_5b/modules/attention.py:84-306):
+ *   out[t, h, :] = softmax_j(q[t, h, :] . k_j[h, :] * scale) v_j   over the key list
+ *       [ n_cached tokens read from the NVFP4 slots (slot = j / block_token_size) | n_new bf16 tokens ]
+ *   q bf16 [Lq, H, 128]; k_new, v_new bf16 [n_new, H, 128] (the caller passes the smoothed K of the
+ *   current chunk, utils/quant.py:797-798); out bf16 [Lq, H, 128].  No mask (causal_model.py:781).
+ *   k_* / v_* pointer arrays: DEVICE arrays of device pointers, one per slot, slot layout as above
+ *   (rows = token*H + head, 128 columns).  n_cached must be a multiple of 64; n_new may be 0.
+ */
+int ll_kv_attention(const void* q, int64_t Lq, int num_heads,
+                    const uint64_t* k_values_ptrs, const uint64_t* k_scales_ptrs, const uint64_t* k_amax_ptrs,
+                    const uint64_t* v_values_ptrs, const uint64_t* v_scales_ptrs, const uint64_t* v_amax_ptrs,
+                    int64_t n_cached, int block_token_size, float e2m1_max, float e4m3_max,
+                    const void* k_new, const void* v_new, int64_t n_new,
+                    float softmax_scale, void* out, void* stream);
+
+/* Plain bf16 attention (cross-attention to the text context; wan_5b/modules/causal_model.py:197-262):
+ * q [Lq,H,128], k/v [Lk,H,128], out [Lq,H,128], no mask. */
+int ll_attention_bf16(const void* q, const void* k, const void* v, int64_t Lq, int64_t Lk, int num_heads,
+                      float softmax_scale, void* out, void* stream);
+
+/*
+ * Replaces rope_apply_triton (utils/rope_triton.py:36-135): x bf16 [S, N, D] (strides in elements, last
+ * dim contiguous), cos/sin f32 [seq_len, D/2]; rows < seq_len are rotated in fp32, the rest copied.
+ */
+int ll_rope_apply(const void* x, int64_t S, int N, int D, int64_t x_stride_s, int64_t x_stride_n,
+                  const float* cos, const float* sin, int64_t seq_len, void* out, void* stream);
+
+/*
+ * Replaces adaln_modulate_triton (utils/adaln_triton.py:36-126): x bf16 [B, L, C] contiguous,
+ * scale/shift bf16 indexed [b, l / frame_seqlen, :] with the given strides (elements);
+ * y = bf16(bf16(LN(x)) * bf16(1 + scale)) + shift.
+ */
+int ll_adaln_modulate(const void* x, int64_t B, int64_t L, int C, const void* scale, const void* shift,
+                      int64_t scale_stride_b, int64_t scale_stride_f, int64_t shift_stride_b, int64_t shift_stride_f,
+                      int64_t frame_seqlen, float eps, int add_one_to_scale, void* out, void* stream);
+
+/* WanRMSNorm (wan_5b/modules/model.py:82-98): y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) over the
+ * last dim C of x bf16 [rows, C]; w bf16 [C]. */
+int ll_rms_norm(const void* x, int64_t rows, int C, const void* weight, float eps, void* out, void* stream);
+
+/* Test hooks: hardware fp32->e4m3 / fp32->e2m1 conversions applied to n floats (used by the GPU tests to
+ * check the instructions the fast paths rely on against the software codecs). mode 0: e4m3, 1: e2m1. */
+int ll_debug_convert(const float* in, int64_t n, int mode, uint8_t* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LL_NVFP4_H */

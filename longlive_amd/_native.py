@@ -1,0 +1,280 @@
+"""ctypes binding of ``libll_nvfp4.so`` (the C ABI declared in ``include/ll_nvfp4.h``).
+
+The library is the only implementation of the hot path: if it is missing, every
+call raises.  Nothing here falls back to PyTorch arithmetic.  PyTorch is used
+for device memory and the current HIP stream only.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import re
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libll_nvfp4.so")
+HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "ll_nvfp4.h")
+
+RULE_IDS = {"static_6": 0, "static_4": 1, "mae": 2, "mse": 3, "abs_max": 4}
+DTYPE_CODES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+
+_lib = None
+
+_SIGNATURES = {
+    "ll_last_error": (c_char_p, []),
+    "ll_version": (c_int, []),
+    "ll_nvfp4_quantize_workspace_floats": (c_size_t, []),
+    "ll_nvfp4_quantize": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                  c_void_p, c_void_p]),
+    "ll_nvfp4_dequantize": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,
+                                    c_void_p, c_int, c_int64, c_void_p]),
+    "ll_nvfp4_gemm_tnt": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                  c_float, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p,
+                                  c_void_p]),
+    "ll_kv_dequantize_blocks": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float,
+                                        c_void_p, c_void_p]),
+    "ll_kv_attention": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                c_int64, c_int, c_float, c_float, c_void_p, c_void_p, c_int64, c_float, c_void_p,
+                                c_void_p]),
+    "ll_attention_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_float, c_void_p, c_void_p]),
+    "ll_rope_apply": (c_int, [c_void_p, c_int64, c_int, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int64,
+                              c_void_p, c_void_p]),
+    "ll_adaln_modulate": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                  c_int64, c_int64, c_float, c_int, c_void_p, c_void_p]),
+    "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
+    "ll_debug_convert": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
+}
+
+
+def declared_symbols() -> list[str]:
+    """Entry points declared in include/ll_nvfp4.h."""
+    with open(HEADER_PATH) as f:
+        text = f.read()
+    return sorted(set(re.findall(r"\b(ll_[a-z0-9_]+)\s*\(", text)))
+
+
+def load():
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -c 'import __graft_entry__ as g; g.build()'` "
+            "(or `make -C longlive_amd/csrc`). There is no fallback implementation."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def _check(code: int, what: str) -> None:
+    if code != 0:
+        msg = load().ll_last_error().decode()
+        if code == -1:
+            raise ValueError(msg or what)
+        raise RuntimeError(msg or what)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _require_cuda(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if t is not None and t.device.type != "cuda":
+            raise ValueError("the NVFP4 kernels run on the GPU only; got a tensor on " + str(t.device))
+
+
+_workspaces: dict[tuple[int, int], torch.Tensor] = {}
+
+
+def _workspace(device: torch.device) -> torch.Tensor:
+    key = (device.index if device.index is not None else torch.cuda.current_device(), _stream())
+    ws = _workspaces.get(key)
+    if ws is None:
+        ws = torch.empty(load().ll_nvfp4_quantize_workspace_floats(), dtype=torch.float32, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def padded_shape(shape: tuple[int, int]) -> tuple[int, int]:
+    return (-(-shape[0] // 128) * 128, -(-shape[1] // 64) * 64)
+
+
+# --------------------------------------------------------------------------- quantize / dequantize
+def quantize(x: torch.Tensor, rule: str, amax: torch.Tensor | None = None, out=None):
+    """x bf16 [M, K] -> (values u8 [Mp, Kp/2], scales float8_e4m3fn [Mp*Kp/16] blocked, amax f32[1]).
+    ``out`` = (values, scale_factors, amax) buffers of exactly those shapes to write into (KV slots)."""
+    _require_cuda(x, amax)
+    if x.ndim != 2:
+        raise ValueError("quantize expects a 2-D tensor")
+    if x.dtype != torch.bfloat16:
+        raise ValueError(f"the NVFP4 quantizer takes bfloat16 input, got {x.dtype}")
+    if x.stride(1) != 1:
+        x = x.contiguous()
+    M, K = x.shape
+    Mp, Kp = padded_shape((M, K))
+    given = amax is not None
+    if out is not None:
+        values, scales, amax_t = out
+        if (values.shape != (Mp, Kp // 2) or values.dtype != torch.uint8 or scales.numel() != Mp * Kp // 16
+                or scales.element_size() != 1 or amax_t.numel() != 1 or amax_t.dtype != torch.float32
+                or not (values.is_contiguous() and scales.is_contiguous())):
+            raise ValueError("out buffers do not match the padded NVFP4 shape of x")
+        if given:
+            amax_t.copy_(amax.reshape(amax_t.shape))
+    else:
+        values = torch.empty((Mp, Kp // 2), dtype=torch.uint8, device=x.device)
+        scales = torch.empty(Mp * Kp // 16, dtype=torch.uint8, device=x.device)
+        amax_t = amax.reshape(1).to(torch.float32).contiguous() if given else torch.empty(
+            1, dtype=torch.float32, device=x.device)
+    ws = None if given else _workspace(x.device)
+    with torch.cuda.device(x.device):
+        code = load().ll_nvfp4_quantize(x.data_ptr(), M, K, x.stride(0), RULE_IDS[rule], values.data_ptr(),
+                                        scales.data_ptr(), amax_t.data_ptr(), int(given), _ptr(ws), _stream())
+    _check(code, "ll_nvfp4_quantize")
+    if out is not None:
+        return out
+    return values, scales.view(torch.float8_e4m3fn), amax_t
+
+
+def dequantize(values, scales, amax, rule: str, padded, original, dtype: torch.dtype) -> torch.Tensor:
+    _require_cuda(values, scales, amax)
+    out = torch.empty(original, dtype=dtype, device=values.device)
+    with torch.cuda.device(values.device):
+        code = load().ll_nvfp4_dequantize(values.data_ptr(), scales.data_ptr(), amax.data_ptr(), RULE_IDS[rule],
+                                          padded[0], padded[1], original[0], original[1], out.data_ptr(),
+                                          DTYPE_CODES[dtype], out.stride(0), _stream())
+    _check(code, "ll_nvfp4_dequantize")
+    return out
+
+
+# --------------------------------------------------------------------------- GEMM
+def gemm(a_values, a_scales, b_values, b_scales, M: int, N: int, *, alpha=None, amax_a=None, amax_b=None,
+         denom_a: float = 1536.0, denom_b: float = 1536.0, bias=None, out=None) -> torch.Tensor:
+    _require_cuda(a_values, a_scales, b_values, b_scales, alpha, amax_a, amax_b, bias)
+    Mp, Kb = a_values.shape
+    Np, Kb2 = b_values.shape
+    if Kb != Kb2:
+        raise ValueError(f"inner dimensions differ: {Kb * 2} vs {Kb2 * 2}")
+    if out is None:
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=a_values.device)
+    if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous bfloat16 vector of length N")
+    with torch.cuda.device(a_values.device):
+        code = load().ll_nvfp4_gemm_tnt(a_values.data_ptr(), a_scales.data_ptr(), b_values.data_ptr(),
+                                        b_scales.data_ptr(), _ptr(alpha), _ptr(amax_a), _ptr(amax_b), denom_a, denom_b,
+                                        M, N, Mp, Np, Kb * 2, out.data_ptr(), out.stride(0), _ptr(bias), _stream())
+    _check(code, "ll_nvfp4_gemm_tnt")
+    return out
+
+
+# --------------------------------------------------------------------------- KV cache
+def kv_dequantize_blocks(values_ptrs, scales_ptrs, amax_ptrs, n_blocks, num_heads, block_token_size, dtype,
+                         e2m1_max, e4m3_max) -> torch.Tensor:
+    out = torch.empty((1, n_blocks * block_token_size, num_heads, 128), dtype=dtype, device=values_ptrs.device)
+    with torch.cuda.device(values_ptrs.device):
+        code = load().ll_kv_dequantize_blocks(values_ptrs.data_ptr(), scales_ptrs.data_ptr(), amax_ptrs.data_ptr(),
+                                              n_blocks, num_heads, block_token_size, DTYPE_CODES[dtype],
+                                              float(e2m1_max), float(e4m3_max), out.data_ptr(), _stream())
+    _check(code, "ll_kv_dequantize_blocks")
+    return out
+
+
+def kv_attention(q, tables, n_cached, block_token_size, e2m1_max, e4m3_max, k_new, v_new, softmax_scale):
+    """q [Lq, H, 128] bf16; tables = six int64 device tensors of slot pointers (or None when n_cached == 0)."""
+    _require_cuda(q, k_new, v_new)
+    if q.dtype != torch.bfloat16 or q.ndim != 3 or q.shape[-1] != 128 or not q.is_contiguous():
+        raise ValueError("q must be a contiguous bfloat16 [Lq, H, 128] tensor")
+    Lq, H, _ = q.shape
+    n_new = 0
+    if k_new is not None:
+        if k_new.shape != v_new.shape or k_new.shape[1:] != (H, 128) or k_new.dtype != torch.bfloat16:
+            raise ValueError("k_new / v_new must be bfloat16 [n_new, H, 128]")
+        k_new = k_new.contiguous()
+        v_new = v_new.contiguous()
+        n_new = k_new.shape[0]
+    out = torch.empty_like(q)
+    t = [None] * 6 if tables is None else [x.data_ptr() for x in tables]
+    with torch.cuda.device(q.device):
+        code = load().ll_kv_attention(q.data_ptr(), Lq, H, *t, n_cached, block_token_size, float(e2m1_max),
+                                      float(e4m3_max), _ptr(k_new), _ptr(v_new), n_new, float(softmax_scale),
+                                      out.data_ptr(), _stream())
+    _check(code, "ll_kv_attention")
+    return out
+
+
+def attention_bf16(q, k, v, softmax_scale):
+    return kv_attention(q, None, 0, 0, 6.0, 256.0, k, v, softmax_scale)
+
+
+# --------------------------------------------------------------------------- elementwise
+def rope_apply(x, cos, sin, seq_len=None):
+    _require_cuda(x, cos, sin)
+    if x.ndim != 3 or x.dtype != torch.bfloat16 or x.stride(2) != 1:
+        raise ValueError("x must be bfloat16 [S, N, D] with a contiguous last dimension")
+    S, N, D = x.shape
+    seq_len = S if seq_len is None else seq_len
+    if cos.shape != (seq_len, D // 2) or sin.shape != cos.shape or cos.dtype != torch.float32:
+        raise ValueError(f"cos/sin must be float32 [{seq_len}, {D // 2}]")
+    cos = cos.contiguous()
+    sin = sin.contiguous()
+    out = torch.empty((S, N, D), dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        code = load().ll_rope_apply(x.data_ptr(), S, N, D, x.stride(0), x.stride(1), cos.data_ptr(), sin.data_ptr(),
+                                    seq_len, out.data_ptr(), _stream())
+    _check(code, "ll_rope_apply")
+    return out
+
+
+def adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps=1e-6, add_one_to_scale=True):
+    _require_cuda(x, e_scale, e_shift)
+    if x.ndim != 3 or x.dtype != torch.bfloat16 or not x.is_contiguous():
+        raise ValueError("x must be a contiguous bfloat16 [B, L, C] tensor")
+    B, L, C = x.shape
+    F = L // frame_seqlen
+    for name, e in (("e_scale", e_scale), ("e_shift", e_shift)):
+        if e.shape != (B, F, 1, C) or e.dtype != torch.bfloat16 or e.stride(3) != 1:
+            raise ValueError(f"{name} must be bfloat16 [B, F, 1, C] = {(B, F, 1, C)}, got {tuple(e.shape)}")
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        code = load().ll_adaln_modulate(x.data_ptr(), B, L, C, e_scale.data_ptr(), e_shift.data_ptr(),
+                                        e_scale.stride(0), e_scale.stride(1), e_shift.stride(0), e_shift.stride(1),
+                                        frame_seqlen, float(eps), int(add_one_to_scale), out.data_ptr(), _stream())
+    _check(code, "ll_adaln_modulate")
+    return out
+
+
+def rms_norm(x, weight, eps=1e-6):
+    _require_cuda(x, weight)
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16:
+        raise ValueError("rms_norm takes bfloat16 input and weight")
+    C = x.shape[-1]
+    x2 = x.reshape(-1, C)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    out = torch.empty_like(x2)
+    with torch.cuda.device(x.device):
+        code = load().ll_rms_norm(x2.data_ptr(), x2.shape[0], C, weight.contiguous().data_ptr(), float(eps),
+                                  out.data_ptr(), _stream())
+    _check(code, "ll_rms_norm")
+    return out.view(x.shape)
+
+
+def debug_convert(x: torch.Tensor, mode: int) -> torch.Tensor:
+    x = x.contiguous().float()
+    out = torch.empty(x.numel(), dtype=torch.uint8, device=x.device)
+    code = load().ll_debug_convert(x.data_ptr(), x.numel(), mode, out.data_ptr(), _stream())
+    _check(code, "ll_debug_convert")
+    return out

@@ -1,0 +1,228 @@
+// Memory-bound fused kernels of the DiT block for gfx950: 3-D RoPE apply, adaLN modulate, RMSNorm.
+// All of them read bf16 with 128-bit loads, compute in fp32 and round where the reference rounds.
+#include "ll_common.h"
+
+#pragma clang fp contract(off)
+
+namespace ll {
+
+__device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __uint_as_float(w[i] << 16);
+    f[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+  }
+}
+__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
+  uint32_t w[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) w[i] = f32_to_bf16_bits(f[2 * i]) | (f32_to_bf16_bits(f[2 * i + 1]) << 16);
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
+
+// ----------------------------------------------------------------------------- RoPE
+// utils/rope_triton.py:36-81.  One thread = 8 consecutive elements (4 rotation pairs) of one (token, head).
+__global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ x, int64_t S, int N, int D,
+                                                   int64_t xs, int64_t xn, const float* __restrict__ cosp,
+                                                   const float* __restrict__ sinp, int64_t seq_len,
+                                                   uint16_t* __restrict__ out) {
+  const int gpr = D >> 3;  // groups per (token, head)
+  const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int64_t total = S * N * gpr;
+  if (g >= total) return;
+  const int64_t s = g / ((int64_t)N * gpr);
+  const int rem = (int)(g - s * (int64_t)N * gpr);
+  const int n = rem / gpr, c = (rem - n * gpr) * 8;
+  const uint4 v = *reinterpret_cast<const uint4*>(x + s * xs + (int64_t)n * xn + c);
+  uint4 o = v;
+  if (s < seq_len) {
+    float f[8], r[8];
+    unpack8(v, f);
+    const float4 cs = *reinterpret_cast<const float4*>(cosp + s * (D >> 1) + (c >> 1));
+    const float4 sn = *reinterpret_cast<const float4*>(sinp + s * (D >> 1) + (c >> 1));
+    const float cc[4] = {cs.x, cs.y, cs.z, cs.w}, ss[4] = {sn.x, sn.y, sn.z, sn.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float a = f[2 * i], b = f[2 * i + 1];
+      r[2 * i] = a * cc[i] - b * ss[i];
+      r[2 * i + 1] = a * ss[i] + b * cc[i];
+    }
+    o = pack8(r);
+  }
+  *reinterpret_cast<uint4*>(out + (s * N + n) * (int64_t)D + c) = o;
+}
+
+// ----------------------------------------------------------------------------- block reductions
+template <int NT>
+__device__ __forceinline__ float block_sum(float v, float* sm) {
+  v = wave_sum(v);
+  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NT / 64; ++i) r += sm[i];
+  __syncthreads();
+  return r;
+}
+
+constexpr int kRowThreads = 128;
+constexpr int kMaxChunks = 8;  // 8 elements each: C <= 128 * 8 * 8 = 8192
+
+// ----------------------------------------------------------------------------- adaLN
+// utils/adaln_triton.py:36-86.  One workgroup = one token row.
+__global__ __launch_bounds__(kRowThreads) void adaln_kernel(const uint16_t* __restrict__ x, int64_t L, int C,
+                                                            const uint16_t* __restrict__ scale,
+                                                            const uint16_t* __restrict__ shift, int64_t sc_sb,
+                                                            int64_t sc_sf, int64_t sh_sb, int64_t sh_sf,
+                                                            int64_t frame_seqlen, float eps, int add_one,
+                                                            uint16_t* __restrict__ out) {
+  __shared__ float sm[kRowThreads / 64];
+  const int64_t row = blockIdx.x;
+  const int64_t b = row / L, l = row - b * L, f = l / frame_seqlen;
+  const uint16_t* xr = x + row * (int64_t)C;
+  const int nchunks = C >> 3;
+  float v[kMaxChunks][8];
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kMaxChunks; ++i) {
+    const int c = threadIdx.x + i * kRowThreads;
+    if (c < nchunks) {
+      unpack8(*reinterpret_cast<const uint4*>(xr + c * 8), v[i]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sum += v[i][j];
+    }
+  }
+  const float inv_c = 1.0f / (float)C;
+  const float mean = block_sum<kRowThreads>(sum, sm) * inv_c;
+  float sq = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kMaxChunks; ++i) {
+    const int c = threadIdx.x + i * kRowThreads;
+    if (c < nchunks) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[i][j] -= mean;
+        sq += v[i][j] * v[i][j];
+      }
+    }
+  }
+  const float var = block_sum<kRowThreads>(sq, sm) * inv_c;
+  const float rstd = 1.0f / sqrtf(var + eps);
+  const uint16_t* scr = scale + b * sc_sb + f * sc_sf;
+  const uint16_t* shr = shift + b * sh_sb + f * sh_sf;
+  uint16_t* orow = out + row * (int64_t)C;
+#pragma unroll
+  for (int i = 0; i < kMaxChunks; ++i) {
+    const int c = threadIdx.x + i * kRowThreads;
+    if (c < nchunks) {
+      float s8[8], h8[8], y[8];
+      unpack8(*reinterpret_cast<const uint4*>(scr + c * 8), s8);
+      unpack8(*reinterpret_cast<const uint4*>(shr + c * 8), h8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float xn = round_to_bf16(v[i][j] * rstd);
+        const float s = add_one ? round_to_bf16(s8[j] + 1.0f) : s8[j];
+        const float prod = round_to_bf16(xn * s);
+        y[j] = prod + h8[j];
+      }
+      *reinterpret_cast<uint4*>(orow + c * 8) = pack8(y);
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------- RMSNorm
+// wan_5b/modules/model.py:82-98.
+__global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(const uint16_t* __restrict__ x, int C,
+                                                              const uint16_t* __restrict__ w, float eps,
+                                                              uint16_t* __restrict__ out) {
+  __shared__ float sm[kRowThreads / 64];
+  const int64_t row = blockIdx.x;
+  const uint16_t* xr = x + row * (int64_t)C;
+  const int nchunks = C >> 3;
+  float v[kMaxChunks][8];
+  float sq = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kMaxChunks; ++i) {
+    const int c = threadIdx.x + i * kRowThreads;
+    if (c < nchunks) {
+      unpack8(*reinterpret_cast<const uint4*>(xr + c * 8), v[i]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sq += v[i][j] * v[i][j];
+    }
+  }
+  const float ms = block_sum<kRowThreads>(sq, sm) / (float)C;
+  const float r = 1.0f / sqrtf(ms + eps);
+  uint16_t* orow = out + row * (int64_t)C;
+#pragma unroll
+  for (int i = 0; i < kMaxChunks; ++i) {
+    const int c = threadIdx.x + i * kRowThreads;
+    if (c < nchunks) {
+      float w8[8], y[8];
+      unpack8(*reinterpret_cast<const uint4*>(w + c * 8), w8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = round_to_bf16(v[i][j] * r) * w8[j];
+      *reinterpret_cast<uint4*>(orow + c * 8) = pack8(y);
+    }
+  }
+}
+
+}  // namespace ll
+
+extern "C" int ll_rope_apply(const void* x, int64_t S, int N, int D, int64_t x_stride_s, int64_t x_stride_n,
+                             const float* cos, const float* sin, int64_t seq_len, void* out, void* stream) {
+  using namespace ll;
+  LL_REQUIRE(x && cos && sin && out, "ll_rope_apply: null pointer");
+  LL_REQUIRE(S > 0 && N > 0 && D > 0 && D % 16 == 0 && seq_len >= 0 && seq_len <= S,
+             "ll_rope_apply: bad shape S=%lld N=%d D=%d seq_len=%lld (D must be a multiple of 16)", (long long)S, N, D,
+             (long long)seq_len);
+  LL_REQUIRE(x_stride_s % 8 == 0 && x_stride_n % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+                 (reinterpret_cast<uintptr_t>(out) & 15) == 0 && (reinterpret_cast<uintptr_t>(cos) & 15) == 0 &&
+                 (reinterpret_cast<uintptr_t>(sin) & 15) == 0,
+             "ll_rope_apply: pointers must be 16-byte aligned and strides multiples of 8 elements");
+  const int64_t groups = S * N * (D / 8);
+  hipLaunchKernelGGL(rope_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x), S, N, D, x_stride_s,
+                     x_stride_n, cos, sin, seq_len, static_cast<uint16_t*>(out));
+  LL_CHECK_LAUNCH("rope_kernel");
+  return LL_OK;
+}
+
+extern "C" int ll_adaln_modulate(const void* x, int64_t B, int64_t L, int C, const void* scale, const void* shift,
+                                 int64_t scale_stride_b, int64_t scale_stride_f, int64_t shift_stride_b,
+                                 int64_t shift_stride_f, int64_t frame_seqlen, float eps, int add_one_to_scale,
+                                 void* out, void* stream) {
+  using namespace ll;
+  LL_REQUIRE(x && scale && shift && out, "ll_adaln_modulate: null pointer");
+  LL_REQUIRE(B > 0 && L > 0 && C > 0 && C % 8 == 0 && C <= kRowThreads * kMaxChunks * 8 && frame_seqlen > 0 &&
+                 L % frame_seqlen == 0,
+             "ll_adaln_modulate: bad shape B=%lld L=%lld C=%d frame_seqlen=%lld (C %% 8 == 0, C <= %d)", (long long)B,
+             (long long)L, C, (long long)frame_seqlen, kRowThreads * kMaxChunks * 8);
+  LL_REQUIRE(scale_stride_b % 8 == 0 && scale_stride_f % 8 == 0 && shift_stride_b % 8 == 0 && shift_stride_f % 8 == 0 &&
+                 ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(scale) |
+                   reinterpret_cast<uintptr_t>(shift) | reinterpret_cast<uintptr_t>(out)) & 15) == 0,
+             "ll_adaln_modulate: pointers must be 16-byte aligned and strides multiples of 8 elements");
+  LL_REQUIRE(B * L <= 0x7FFFFFFF, "ll_adaln_modulate: too many rows");
+  hipLaunchKernelGGL(adaln_kernel, dim3((unsigned)(B * L)), dim3(kRowThreads), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(x), L, C, static_cast<const uint16_t*>(scale),
+                     static_cast<const uint16_t*>(shift), scale_stride_b, scale_stride_f, shift_stride_b,
+                     shift_stride_f, frame_seqlen, eps, add_one_to_scale, static_cast<uint16_t*>(out));
+  LL_CHECK_LAUNCH("adaln_kernel");
+  return LL_OK;
+}
+
+extern "C" int ll_rms_norm(const void* x, int64_t rows, int C, const void* weight, float eps, void* out,
+                           void* stream) {
+  using namespace ll;
+  LL_REQUIRE(x && weight && out, "ll_rms_norm: null pointer");
+  LL_REQUIRE(rows > 0 && rows <= 0x7FFFFFFF && C > 0 && C % 8 == 0 && C <= kRowThreads * kMaxChunks * 8,
+             "ll_rms_norm: bad shape rows=%lld C=%d", (long long)rows, C);
+  LL_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) |
+               reinterpret_cast<uintptr_t>(out)) & 15) == 0,
+             "ll_rms_norm: pointers must be 16-byte aligned");
+  hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const uint16_t*>(x), C, static_cast<const uint16_t*>(weight), eps,
+                     static_cast<uint16_t*>(out));
+  LL_CHECK_LAUNCH("rmsnorm_kernel");
+  return LL_OK;
+}

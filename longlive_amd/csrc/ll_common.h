@@ -1,0 +1,99 @@
+// Shared device/host helpers for the gfx950 NVFP4 kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/ll_nvfp4.h"
+
+namespace ll {
+
+// ----------------------------------------------------------------------------- errors
+void set_error(const char* fmt, ...);
+
+#define LL_REQUIRE(cond, ...)      \
+  do {                             \
+    if (!(cond)) {                 \
+      ll::set_error(__VA_ARGS__);  \
+      return LL_EINVAL;            \
+    }                              \
+  } while (0)
+
+#define LL_CHECK_LAUNCH(name)                                              \
+  do {                                                                     \
+    hipError_t e__ = hipGetLastError();                                    \
+    if (e__ != hipSuccess) {                                               \
+      ll::set_error("%s: launch failed: %s", name, hipGetErrorString(e__)); \
+      return LL_ELAUNCH;                                                   \
+    }                                                                      \
+  } while (0)
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+// ----------------------------------------------------------------------------- formats
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// fp32 -> bf16 bits, round to nearest even (NaN stays NaN).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
+  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+}
+__device__ __forceinline__ float round_to_bf16(float f) { return __uint_as_float(f32_to_bf16_bits(f) << 16); }
+
+// e4m3fn byte -> fp32 (exact). 0x7F / 0xFF decode to NaN.
+__device__ __forceinline__ float e4m3_to_f32(uint32_t b) {
+  uint32_t e = (b >> 3) & 0xFu, m = b & 7u;
+  float v;
+  if (e == 0) {
+    v = (float)m * 0.001953125f;  // m * 2^-9
+  } else if (e == 15 && m == 7) {
+    v = __uint_as_float(0x7FC00000u);
+  } else {
+    v = __uint_as_float(((e + 120u) << 23) | (m << 20));
+  }
+  return (b & 0x80u) ? -v : v;
+}
+
+// fp32 -> e4m3fn byte, round to nearest even, |x| > 464 -> NaN (0x7F): the value torch's
+// float8_e4m3fn cast produces.
+__device__ __forceinline__ uint32_t f32_to_e4m3(float x) {
+  uint32_t u = __float_as_uint(x);
+  uint32_t sign = (u >> 24) & 0x80u;
+  u &= 0x7FFFFFFFu;
+  float a = __uint_as_float(u);
+  if (!(a <= 464.0f)) return sign | 0x7Fu;  // NaN, inf, overflow
+  if (a >= 0.015625f) {                     // normal range: keep 3 mantissa bits
+    uint32_t r = (u + 0x7FFFFu + ((u >> 20) & 1u)) >> 20;
+    return sign | (r - (120u << 3));
+  }
+  return sign | (uint32_t)__builtin_rintf(a * 512.0f);  // sub-normal grid 2^-9, 8 -> 2^-6
+}
+
+__device__ __constant__ const float kE2M1[16] = {0.0f,  0.5f,  1.0f,  1.5f,  2.0f,  3.0f,  4.0f,  6.0f,
+                                                 -0.0f, -0.5f, -1.0f, -1.5f, -2.0f, -3.0f, -4.0f, -6.0f};
+
+// Offset of scale (r, c) of a [rows, cols] e4m3 matrix stored in 128x4 blocked order.
+__host__ __device__ __forceinline__ int64_t blocked_scale_offset(int64_t r, int64_t c, int64_t cols) {
+  int64_t rb = r >> 7, ri = r & 127, cb = c >> 2, ci = c & 3;
+  return ((rb * (cols >> 2) + cb) * 32 + (ri & 31)) * 16 + (ri >> 5) * 4 + ci;
+}
+
+__host__ __device__ __forceinline__ void rule_limits(int rule, float& e2, float& e4) {
+  e2 = (rule == LL_RULE_STATIC_4) ? 4.0f : 6.0f;
+  e4 = (rule == LL_RULE_STATIC_6 || rule == LL_RULE_STATIC_4) ? 448.0f : 256.0f;
+}
+
+// ----------------------------------------------------------------------------- wave helpers
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+
+}  // namespace ll

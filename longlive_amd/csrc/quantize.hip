@@ -1,0 +1,292 @@
+// NVFP4 quantization for gfx950: tensor amax, block-16 e4m3 scales, e2m1 codes, and the
+// four-over-six per-block choice.  Arithmetic follows the reference's PyTorch backend
+// (fouroversix/src/fouroversix/quantize/pytorch/reference.py:121-368) operation by operation, so
+// the packed bytes are identical to what that backend produces on a CPU.
+//
+// This file must be compiled without floating-point contraction: every product and sum below is
+// rounded separately, as the eager PyTorch graph rounds it.
+#include "ll_common.h"
+
+#pragma clang fp contract(off)
+
+namespace ll {
+
+constexpr int kAmaxParts = 1024;  // partial maxima written by the amax kernel
+constexpr int kThreads = 256;
+
+// ----------------------------------------------------------------------------- amax
+// Each workgroup folds a grid-strided share of x into one partial maximum; the quantize kernel
+// reduces the kAmaxParts partials again, so no atomics and no zero-initialised state are needed.
+__global__ __launch_bounds__(kThreads) void amax_partial_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
+                                                                 int64_t ldx, float* __restrict__ parts) {
+  float m = 0.0f;
+  const int64_t tid = (int64_t)blockIdx.x * kThreads + threadIdx.x;
+  const int64_t nthreads = (int64_t)gridDim.x * kThreads;
+  const bool vec = ((K & 7) == 0) && ((ldx & 7) == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+  if (vec) {
+    const int64_t kc = K >> 3;
+    const int64_t nchunks = M * kc;
+    for (int64_t c = tid; c < nchunks; c += nthreads) {
+      const int64_t r = c / kc, cc = c - r * kc;
+      const uint4 v = *reinterpret_cast<const uint4*>(x + r * ldx + cc * 8);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        m = fmaxf(m, fabsf(__uint_as_float(w[i] << 16)));
+        m = fmaxf(m, fabsf(__uint_as_float(w[i] & 0xFFFF0000u)));
+      }
+    }
+  } else {
+    const int64_t n = M * K;
+    for (int64_t i = tid; i < n; i += nthreads) {
+      const int64_t r = i / K, c = i - r * K;
+      m = fmaxf(m, fabsf(bf16_bits_to_f32(x[r * ldx + c])));
+    }
+  }
+  m = wave_max(m);
+  __shared__ float sm[kThreads / 64];
+  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float r = sm[0];
+    for (int i = 1; i < kThreads / 64; ++i) r = fmaxf(r, sm[i]);
+    parts[blockIdx.x] = r;
+  }
+}
+
+// ----------------------------------------------------------------------------- exact block math
+// reference.py:18-34, nearest rounding: the e2m1 grid with half-to-even ties, no clamp at 6.
+__device__ __forceinline__ float fake_quantize_e2m1(float y) {
+  const float a = fabsf(y);
+  float q;
+  if (a < 2.0f) {
+    q = __builtin_rintf(2.0f * a) / 2.0f;
+  } else if (a < 4.0f) {
+    q = __builtin_rintf(a);
+  } else {
+    q = 2.0f * __builtin_rintf(a / 2.0f);
+  }
+  return y > 0.0f ? q : (y < 0.0f ? -q : 0.0f);  // sign(y) * q with sign(+-0) = 0
+}
+
+// reference.py:37-63: the 4-bit code is read from the bf16 bit pattern of q with 16-bit integer
+// arithmetic and truncated to 8 bits; values of |q| >= 8 overflow the nibble exactly as there.
+__device__ __forceinline__ uint32_t code_from_q(float q) {
+  const int32_t bx = (int32_t)(int16_t)f32_to_bf16_bits(q);
+  int32_t s = (bx >> 15) & 1;
+  int32_t e = (bx >> 7) & 0xFF;
+  int32_t m = bx & 0x7F;
+  const bool is_zero = (e == 0) && (m == 0);
+  m = (m >> 6) & 1;
+  if (e == 126 && m == 0) m = 1;
+  e -= 126;
+  if (is_zero) {
+    e = 0;
+    m = 0;
+  }
+  return (uint32_t)((s << 3) | (e << 1) | m) & 0xFFu;
+}
+
+struct Candidate {
+  float q[16];
+  uint32_t scale_byte;
+  float scale;
+};
+
+// reference.py:121-173 for one block.  hp is the high-precision scale (already expanded by 1.5 for the
+// "4" candidate); dec = 1 / (E2*E4 / amax).
+__device__ __forceinline__ void make_candidate(const float (&X)[16], float hp, float dec, Candidate& c) {
+  c.scale_byte = f32_to_e4m3(hp);
+  c.scale = e4m3_to_f32(c.scale_byte);
+  const float r = 1.0f / (dec * c.scale);
+  const bool nz = c.scale != 0.0f;  // torch.where(scales != 0, x * r, 0); a NaN scale compares != 0
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const float y = nz ? X[i] * r : 0.0f;
+    c.q[i] = fake_quantize_e2m1(y);
+  }
+}
+
+// reference.py:196-225: error of one candidate against the block, summed in the order torch's CPU
+// reduction uses for 16 contiguous floats (p[i] = t[i] + t[i+8], then p[0] + p[1] + ... + p[7]).
+template <int RULE>
+__device__ __forceinline__ float candidate_error(const float (&X)[16], const Candidate& c, float amax) {
+  float t[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const float d = ((c.q[i] * c.scale) * amax) / 1536.0f;
+    const float e = d - X[i];
+    t[i] = (RULE == LL_RULE_MSE) ? e * e : fabsf(e);
+  }
+  if (RULE == LL_RULE_ABS_MAX) {
+    float m = t[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) m = fmaxf(m, t[i]);
+    return m;
+  }
+  float acc = t[0] + t[8];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) acc = acc + (t[i] + t[i + 8]);
+  return acc;
+}
+
+// Quantize one block of 16 values; returns the 8 packed bytes (lo, hi) and the scale byte.
+template <int RULE>
+__device__ __forceinline__ void quantize_block(const float (&X)[16], float amax, uint32_t& lo, uint32_t& hi,
+                                               uint32_t& scale_byte) {
+  constexpr bool kStatic = (RULE == LL_RULE_STATIC_6 || RULE == LL_RULE_STATIC_4);
+  constexpr float E2 = (RULE == LL_RULE_STATIC_4) ? 4.0f : 6.0f;
+  constexpr float E4 = kStatic ? 448.0f : 256.0f;
+  float bmax = fabsf(X[0]);
+#pragma unroll
+  for (int i = 1; i < 16; ++i) bmax = fmaxf(bmax, fabsf(X[i]));
+  const float enc = (E2 * E4) / amax;
+  const float hp = (amax == 0.0f) ? 0.0f : (bmax / E2) * enc;
+  const float dec = 1.0f / enc;
+
+  Candidate c6;
+  make_candidate(X, hp, dec, c6);
+  const Candidate* pick = &c6;
+  Candidate c4;
+  if (!kStatic) {
+    make_candidate(X, hp * 1.5f, dec, c4);
+    const float e4 = candidate_error<RULE>(X, c4, amax);
+    const float e6 = candidate_error<RULE>(X, c6, amax);
+    if (e4 < e6) pick = &c4;
+  }
+  uint32_t b[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const uint32_t cl = code_from_q(pick->q[2 * j]);
+    const uint32_t ch = code_from_q(pick->q[2 * j + 1]);
+    b[j] = ((ch << 4) | cl) & 0xFFu;  // uint8 arithmetic of reference.py:85-87
+  }
+  lo = b[0] | (b[1] << 8) | (b[2] << 16) | (b[3] << 24);
+  hi = b[4] | (b[5] << 8) | (b[6] << 16) | (b[7] << 24);
+  scale_byte = pick->scale_byte;
+}
+
+// ----------------------------------------------------------------------------- quantize kernel
+// One workgroup = a 128-row x 64-column tile = 512 blocks of 16 = one 512-byte tile of the blocked
+// scale layout, which is staged in LDS and written with coalesced 4-byte stores.
+template <int RULE>
+__global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
+                                                            int64_t ldx, int64_t Kp, uint8_t* __restrict__ values,
+                                                            uint8_t* __restrict__ scales, float* __restrict__ amax_io,
+                                                            const float* __restrict__ parts, int amax_given) {
+  __shared__ float s_red[kThreads / 64];
+  __shared__ float s_amax;
+  __shared__ uint32_t s_scales[128];  // 512 bytes in blocked order
+
+  if (amax_given) {
+    if (threadIdx.x == 0) s_amax = amax_io[0];
+  } else {
+    const float4 p = reinterpret_cast<const float4*>(parts)[threadIdx.x];  // kAmaxParts == 4 * kThreads
+    float m = wave_max(fmaxf(fmaxf(p.x, p.y), fmaxf(p.z, p.w)));
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      float r = s_red[0];
+      for (int i = 1; i < kThreads / 64; ++i) r = fmaxf(r, s_red[i]);
+      s_amax = r;
+      if (blockIdx.x == 0 && blockIdx.y == 0) amax_io[0] = r;
+    }
+  }
+  __syncthreads();
+  const float amax = s_amax;
+
+  const int64_t row0 = (int64_t)blockIdx.y * 128;
+  const int64_t col0 = (int64_t)blockIdx.x * 64;
+  const bool vec = ((ldx & 7) == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
+  uint8_t* s_bytes = reinterpret_cast<uint8_t*>(s_scales);
+
+#pragma unroll 1
+  for (int it = 0; it < 2; ++it) {
+    const int b = threadIdx.x + it * kThreads;  // block within the tile
+    const int r = b >> 2, cb = b & 3;
+    const int64_t row = row0 + r, col = col0 + cb * 16;
+    float X[16];
+    if (row < M && col + 16 <= K && vec) {
+      const uint4* p = reinterpret_cast<const uint4*>(x + row * ldx + col);
+      const uint4 v0 = p[0], v1 = p[1];
+      const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        X[2 * i] = __uint_as_float(w[i] << 16);
+        X[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        X[i] = (row < M && col + i < K) ? bf16_bits_to_f32(x[row * ldx + col + i]) : 0.0f;
+    }
+    uint32_t lo, hi, sb;
+    quantize_block<RULE>(X, amax, lo, hi, sb);
+    *reinterpret_cast<uint2*>(values + row * (Kp >> 1) + (col >> 1)) = make_uint2(lo, hi);
+    s_bytes[(r & 31) * 16 + (r >> 5) * 4 + cb] = (uint8_t)sb;
+  }
+  __syncthreads();
+  if (threadIdx.x < 128) {
+    const int64_t tile = (int64_t)blockIdx.y * (Kp >> 6) + blockIdx.x;
+    reinterpret_cast<uint32_t*>(scales)[tile * 128 + threadIdx.x] = s_scales[threadIdx.x];
+  }
+}
+
+// ----------------------------------------------------------------------------- hardware codec probe
+__global__ void debug_convert_kernel(const float* __restrict__ in, int64_t n, int mode, uint8_t* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float v = in[i];
+  if (mode == 0) {
+    out[i] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(v, 0.0f, 0, false) & 0xFF);
+  } else {
+    out[i] = (uint8_t)(__builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v, 0.0f, 1.0f, 0) & 0xF);
+  }
+}
+
+}  // namespace ll
+
+extern "C" size_t ll_nvfp4_quantize_workspace_floats(void) { return ll::kAmaxParts; }
+
+extern "C" int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ldx, int rule, uint8_t* values,
+                                 uint8_t* scales, float* amax, int amax_given, float* workspace, void* stream) {
+  using namespace ll;
+  LL_REQUIRE(x && values && scales && amax, "ll_nvfp4_quantize: null pointer");
+  LL_REQUIRE(M > 0 && K > 0 && ldx >= K, "ll_nvfp4_quantize: bad shape M=%lld K=%lld ldx=%lld", (long long)M,
+             (long long)K, (long long)ldx);
+  LL_REQUIRE(rule >= 0 && rule <= 4, "ll_nvfp4_quantize: unknown scale rule %d", rule);
+  LL_REQUIRE(amax_given || workspace, "ll_nvfp4_quantize: workspace required to compute amax");
+  LL_REQUIRE((reinterpret_cast<uintptr_t>(values) & 7) == 0 && (reinterpret_cast<uintptr_t>(scales) & 3) == 0,
+             "ll_nvfp4_quantize: outputs must be 8-byte (values) / 4-byte (scales) aligned");
+  const int64_t Mp = round_up(M, 128), Kp = round_up(K, 64);
+  LL_REQUIRE(Kp / 64 <= 0x7FFFFFFF && Mp / 128 <= 65535, "ll_nvfp4_quantize: tensor too large for one launch");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const uint16_t* xp = static_cast<const uint16_t*>(x);
+  if (!amax_given) {
+    hipLaunchKernelGGL(amax_partial_kernel, dim3(kAmaxParts), dim3(kThreads), 0, s, xp, M, K, ldx, workspace);
+    LL_CHECK_LAUNCH("amax_partial_kernel");
+  }
+  const dim3 grid((unsigned)(Kp / 64), (unsigned)(Mp / 128));
+#define LL_LAUNCH_Q(R)                                                                                          \
+  hipLaunchKernelGGL(quantize_kernel<R>, grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales, amax, \
+                     workspace, amax_given)
+  switch (rule) {
+    case LL_RULE_STATIC_6: LL_LAUNCH_Q(LL_RULE_STATIC_6); break;
+    case LL_RULE_STATIC_4: LL_LAUNCH_Q(LL_RULE_STATIC_4); break;
+    case LL_RULE_MAE: LL_LAUNCH_Q(LL_RULE_MAE); break;
+    case LL_RULE_MSE: LL_LAUNCH_Q(LL_RULE_MSE); break;
+    default: LL_LAUNCH_Q(LL_RULE_ABS_MAX); break;
+  }
+#undef LL_LAUNCH_Q
+  LL_CHECK_LAUNCH("quantize_kernel");
+  return LL_OK;
+}
+
+extern "C" int ll_debug_convert(const float* in, int64_t n, int mode, uint8_t* out, void* stream) {
+  using namespace ll;
+  LL_REQUIRE(in && out && n > 0 && (mode == 0 || mode == 1), "ll_debug_convert: bad arguments");
+  hipLaunchKernelGGL(debug_convert_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), in, n, mode, out);
+  LL_CHECK_LAUNCH("debug_convert_kernel");
+  return LL_OK;
+}

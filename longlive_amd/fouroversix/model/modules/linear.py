@@ -1,0 +1,106 @@
+"""FourOverSixLinear: W4A4 replacement for nn.Linear, inference forward
+(mirror of fouroversix/src/fouroversix/model/modules/linear.py:153-355; the autograd backward of
+the reference is a training feature and is not provided)."""
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+import torch.nn as nn
+
+from ...matmul import fp4_matmul
+from ...quantize import QuantizationConfig, QuantizedTensor, quantize_to_fp4
+from ..config import ModuleQuantizationConfig
+from ..quantize import QuantizedModule
+
+
+@QuantizedModule.register(nn.Linear)
+class FourOverSixLinear(nn.Linear):
+    """Activations are quantized to NVFP4 on the fly, the weight is held pre-quantized in the
+    buffers ``quantized_weight_{values,scale_factors,amax,metadata}`` (same names, dtypes and
+    shapes as the reference, so packed NVFP4 checkpoints load with ``load_state_dict``)."""
+
+    _INT32_MAX = 2_147_483_647
+
+    def __init__(self, module: nn.Linear, config: ModuleQuantizationConfig) -> None:
+        super().__init__(module.in_features, module.out_features, module.bias is not None,
+                         module.weight.device, module.weight.dtype)
+        self.weight = module.weight
+        self.bias = module.bias
+        self.config = config
+        if not self.config.keep_master_weights:
+            dev = module.weight.device
+            self.register_buffer("quantized_weight_values",
+                                 torch.zeros(self.out_features, self.in_features // 2, dtype=torch.uint8, device=dev))
+            self.register_buffer("quantized_weight_scale_factors",
+                                 torch.zeros(self.out_features * self.in_features // config.dtype.block_size(),
+                                             dtype=config.dtype.scale_dtype(), device=dev))
+            self.register_buffer("quantized_weight_amax", torch.zeros(1, dtype=torch.float32, device=dev))
+            self.register_buffer("quantized_weight_metadata", torch.zeros(4, dtype=torch.int32, device=dev))
+
+    # ------------------------------------------------------------------ weight materialisation
+    @property
+    def parameters_to_quantize(self) -> tuple[str, ...]:
+        return ("weight",)
+
+    def get_element_size(self, parameter_name: str) -> float:
+        return {"quantized_weight_values": 0.5, "weight": 9 / 16}.get(
+            parameter_name, getattr(self, parameter_name).element_size())
+
+    def get_quantized_parameters(self, parameter_name: str, parameter: torch.Tensor,
+                                 include_transposed: bool = False) -> dict[str, Any]:
+        if parameter_name != "weight":
+            raise ValueError(f"Unsupported high-precision parameter: {parameter_name}")
+        if include_transposed:
+            raise ValueError("transposed weight caches are a training feature and are not supported")
+        cfg = QuantizationConfig(backend=self.config.quantize_backend, block_scale_2d=self.config.weight_scale_2d,
+                                 dtype=self.config.dtype, scale_rule=self.config.weight_scale_rule)
+        return self._serialize_quantized_weight("quantized_weight", quantize_to_fp4(parameter, cfg))
+
+    @staticmethod
+    def _serialize_quantized_weight(prefix: str, q: QuantizedTensor) -> dict[str, torch.Tensor]:
+        return {
+            f"{prefix}_values": q.values,
+            f"{prefix}_scale_factors": q.scale_factors,
+            f"{prefix}_amax": q.amax,
+            f"{prefix}_metadata": torch.tensor([*q.original_shape, *q.padded_shape], dtype=torch.int32),
+        }
+
+    def _build_quantized_weight(self, prefix: str) -> QuantizedTensor | None:
+        parts = [getattr(self, f"{prefix}_{n}", None) for n in ("values", "scale_factors", "amax", "metadata")]
+        if any(p is None for p in parts):
+            return None
+        values, scale_factors, amax, metadata = parts
+        meta = metadata.tolist()
+        return QuantizedTensor(values.data, scale_factors.data, amax.data, self.config.dtype, tuple(meta[:2]),
+                               self.config.weight_scale_rule, tuple(meta[2:]))
+
+    def quantized_weight(self) -> QuantizedTensor | torch.Tensor:
+        if not hasattr(self, "_quantized_weight"):
+            if self.config.keep_master_weights:
+                return self.weight
+            self._quantized_weight = self._build_quantized_weight("quantized_weight")
+        return self._quantized_weight
+
+    def quantized_weight_transposed(self) -> None:
+        return None
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        if input.requires_grad and torch.is_grad_enabled():
+            raise NotImplementedError("FourOverSixLinear on gfx950 is inference-only; run under torch.no_grad()")
+        x2d = input.reshape(-1, input.shape[-1])
+        if x2d.shape[0] * x2d.shape[1] > self._INT32_MAX:  # same guard as the reference: two halves
+            mid = x2d.shape[0] // 2
+            out = torch.cat([self._forward_2d(x2d[:mid]), self._forward_2d(x2d[mid:])], dim=0)
+        else:
+            out = self._forward_2d(x2d)
+        return out.reshape(*input.shape[:-1], out.shape[-1])
+
+    def _forward_2d(self, x2d: torch.Tensor) -> torch.Tensor:
+        weight = self.quantized_weight()
+        if not isinstance(weight, QuantizedTensor):
+            weight = quantize_to_fp4(weight.data, self.config.get_weight_config())
+        xq = quantize_to_fp4(x2d, self.config.get_activation_config())
+        return fp4_matmul(xq, weight, backend=self.config.matmul_backend, out_dtype=self.config.output_dtype,
+                          bias=self.bias)

@@ -1,0 +1,156 @@
+"""NVFP4 KV cache: allocation, attention over [sink | window | current chunk], roll + insert.
+
+Same cache dictionary as the reference pipeline allocates
+(pipeline/causal_diffusion_inference.py:767-813) and the same cache policy as
+``CausalWanSelfAttention.forward`` / ``CausalWanModel._apply_cache_updates``
+(wan_5b/modules/causal_model.py:491-724, 1371-1483), for whole-block sinks and windows.  Where the
+reference dequantizes all slots to bf16, copies the chunk in and calls flash attention, this
+module hands the slot list and the chunk's bf16 K/V to one kernel that decodes FP4 tiles on load.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import _native
+from ..fouroversix import QuantizationConfig, QuantizedTensor, quantize_to_fp4
+from .quant import SlotPointerTable, clone_quantized_tensor, copy_quantized_into, k_smooth
+
+
+def initialize_kv_cache(num_layers: int, block_token_size: int, max_blocks: int, num_heads: int, head_dim: int,
+                        kv_quant_config: QuantizationConfig, device, dtype=torch.bfloat16) -> list[dict]:
+    """One dict per layer; ``k`` / ``v`` are lists of ``max_blocks`` all-zero NVFP4 slots of logical
+    shape [block_token_size*num_heads, head_dim]."""
+    if head_dim != 128:
+        raise ValueError("the KV-cache kernels are built for head_dim 128")
+    zero = quantize_to_fp4(torch.zeros(block_token_size * num_heads, head_dim, dtype=dtype, device=device),
+                           kv_quant_config)
+    cache = []
+    for _ in range(num_layers):
+        cache.append({
+            "k": [clone_quantized_tensor(zero) for _ in range(max_blocks)],
+            "v": [clone_quantized_tensor(zero) for _ in range(max_blocks)],
+            "quantized": True,
+            "block_token_size": block_token_size,
+            "max_blocks": max_blocks,
+            "num_heads": num_heads,
+            "num_filled_blocks": 0,
+            "global_end_index": torch.tensor([0], dtype=torch.long, device=device),
+            "local_end_index": torch.tensor([0], dtype=torch.long, device=device),
+            "pinned_start": torch.tensor([-1], dtype=torch.long, device=device),
+            "pinned_len": torch.tensor([0], dtype=torch.long, device=device),
+            # host copies of the two indices: the reference publishes them once per forward to avoid
+            # device syncs (utils/wan_5b_wrapper.py:355-366); here they are kept in step on the host
+            "_global_end": 0,
+            "_local_end": 0,
+            "_tables": {},
+        })
+    return cache
+
+
+def _tables_for(cache: dict, slot_ids: tuple[int, ...]):
+    entry = cache["_tables"].get(slot_ids)
+    if entry is None:
+        kt = SlotPointerTable([cache["k"][i] for i in slot_ids])
+        vt = SlotPointerTable([cache["v"][i] for i in slot_ids])
+        entry = (kt, vt)
+        cache["_tables"][slot_ids] = entry
+    return entry
+
+
+def plan_cache_step(cache: dict, current_start: int, num_new_tokens: int, sink_tokens: int,
+                    max_attention_size: int | None = None):
+    """Host-side cache policy for one forward of one layer: which slots are attended (in order) and
+    what ``_apply_cache_updates`` must do afterwards.  Returns (slot_ids, update_info, local_end)."""
+    blk = cache["block_token_size"]
+    size = cache["max_blocks"] * blk
+    g_end, l_end = cache["_global_end"], cache["_local_end"]
+    current_end = current_start + num_new_tokens
+    if num_new_tokens % blk or sink_tokens % blk:
+        raise NotImplementedError("the FP4 KV cache works on whole blocks: chunk and sink sizes must be "
+                                  f"multiples of block_token_size={blk}")
+    if current_end > g_end and num_new_tokens + l_end > size:
+        evicted = num_new_tokens + l_end - size
+        rolled = l_end - evicted - sink_tokens
+        local_end = l_end + current_end - g_end - evicted
+        local_start = local_end - num_new_tokens
+        if evicted % blk or rolled % blk or rolled < 0:
+            raise NotImplementedError("cache roll must move whole blocks")
+        sink_b, ev_b, roll_b = sink_tokens // blk, evicted // blk, rolled // blk
+        slot_ids = tuple(range(sink_b)) + tuple(range(sink_b + ev_b, sink_b + ev_b + roll_b))
+        info = {"action": "roll_and_insert", "sink_tokens": sink_tokens, "num_rolled_tokens": rolled,
+                "num_evicted_tokens": evicted, "local_start_index": local_start, "local_end_index": local_end,
+                "current_end": current_end, "pinned_shift": 0}
+    else:
+        local_end = l_end + current_end - g_end
+        local_start = local_end - num_new_tokens
+        if local_start % blk or local_start < 0:
+            raise NotImplementedError("chunks must start on a block boundary of the cache")
+        slot_ids = tuple(range(local_start // blk))
+        info = {"action": "direct_insert", "local_start_index": local_start, "local_end_index": local_end,
+                "current_end": current_end, "pinned_shift": 0}
+    if max_attention_size is not None and local_end - max_attention_size > 0:
+        # sliding window shorter than the cache: keep the sink blocks, then the most recent blocks
+        window_start = local_end - max_attention_size
+        if window_start % blk or max_attention_size % blk:
+            raise NotImplementedError("attention window must cover whole blocks")
+        n_cached_blocks = (max_attention_size - num_new_tokens) // blk
+        sink_b = sink_tokens // blk
+        keep_tail = max(n_cached_blocks - sink_b, 0)
+        head = slot_ids[:min(sink_b, n_cached_blocks)]
+        tail = slot_ids[len(slot_ids) - keep_tail:] if keep_tail else ()
+        slot_ids = tuple(dict.fromkeys(head + tuple(t for t in tail if t not in head)))
+    return slot_ids, info, local_end
+
+
+def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Tensor, cache: dict,
+                       current_start: int, sink_tokens: int, softmax_scale: float | None = None,
+                       max_attention_size: int | None = None):
+    """Self-attention of one chunk against the FP4 cache.
+
+    q, key_to_cache (RoPE'd, un-smoothed), v: bf16 [1, S, H, 128].  Attends
+    [selected FP4 slots | k_smooth(key_to_cache), v] without a mask and returns
+    ``(out [1, S, H, 128], (current_end, local_end_index, cache_update_info))`` exactly like the
+    reference's attention module, with ``new_k`` / ``new_v`` = the un-smoothed chunk to be written.
+    """
+    if q.shape[0] != 1:
+        raise ValueError("the quantized KV cache holds one sequence (batch size 1)")
+    S, H, D = q.shape[1:]
+    slot_ids, info, local_end = plan_cache_step(cache, current_start, S, sink_tokens, max_attention_size)
+    info["new_k"], info["new_v"] = key_to_cache, v
+    k_new = k_smooth(key_to_cache)[0]
+    scale = D ** -0.5 if softmax_scale is None else softmax_scale
+    rule = cache["k"][0].scale_rule
+    if slot_ids:
+        kt, vt = _tables_for(cache, slot_ids)
+        tables = (kt.values, kt.scales, kt.amax, vt.values, vt.scales, vt.amax)
+    else:
+        tables = None
+    out = _native.kv_attention(q[0].contiguous(), tables, len(slot_ids) * cache["block_token_size"],
+                               cache["block_token_size"], rule.max_allowed_e2m1_value(),
+                               rule.max_allowed_e4m3_value(), k_new, v[0], scale)
+    return out.unsqueeze(0), (current_start + S, local_end, info)
+
+
+def apply_cache_update(cache: dict, current_end: int, local_end_index: int, info: dict | None,
+                       kv_quant_config: QuantizationConfig) -> None:
+    """Roll whole slots and quantize the chunk's K / V into their slots, in place."""
+    if info is not None:
+        blk = cache["block_token_size"]
+        if info["action"] == "roll_and_insert":
+            sink_b = info["sink_tokens"] // blk
+            ev_b = info["num_evicted_tokens"] // blk
+            for i in range(info["num_rolled_tokens"] // blk):
+                copy_quantized_into(cache["k"][sink_b + i], cache["k"][sink_b + ev_b + i])
+                copy_quantized_into(cache["v"][sink_b + i], cache["v"][sink_b + ev_b + i])
+        start_blk = info["local_start_index"] // blk
+        n_insert = (info["local_end_index"] - info["local_start_index"]) // blk
+        rule = kv_quant_config.scale_rule.value
+        for bi in range(n_insert):
+            for name, new in (("k", info["new_k"]), ("v", info["new_v"])):
+                slot: QuantizedTensor = cache[name][start_blk + bi]
+                block = new[0, bi * blk:(bi + 1) * blk].reshape(-1, new.shape[-1])
+                _native.quantize(block, rule, out=(slot.values, slot.scale_factors, slot.amax))
+    cache["global_end_index"].fill_(current_end)
+    cache["local_end_index"].fill_(local_end_index)
+    cache["_global_end"] = current_end
+    cache["_local_end"] = local_end_index

@@ -1,0 +1,186 @@
+"""GPU parity: FP4 KV-cache dequantize, quantize-on-write, fused-dequant attention, RoPE, adaLN, RMSNorm.
+Bars: dequant bit-exact; attention <= 2e-2 max-abs on bf16 outputs; RoPE one bf16 ulp; adaLN 3.1e-2."""
+import numpy as np
+import pytest
+import torch
+
+import nvfp4_oracle as o
+from helpers import bits_of, u8
+from longlive_amd import _native
+from longlive_amd.fouroversix import QuantizationConfig, quantize_to_fp4
+from longlive_amd.utils import kv_cache as kvc
+from longlive_amd.utils.adaln import adaln_modulate
+from longlive_amd.utils.quant import dequantize_kv_cache
+from longlive_amd.utils.rope import build_rope_angles, rope_apply, rope_cos_sin
+
+pytestmark = pytest.mark.gpu
+CFG = QuantizationConfig(scale_rule="mse")
+
+
+def _randn(shape, seed, scale=1.0):
+    return (torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale).bfloat16()
+
+
+def _oracle_slot(t):
+    """[T, H, 128] bf16 tensor -> oracle dequantized bf16 values after quantize-on-write."""
+    T, H, D = t.shape
+    v, s, a, _ = o.quantize_to_fp4(bits_of(t.reshape(-1, D)), "mse")
+    return o.kv_dequantize(v, s, a).reshape(T, H, D), (v, s, a)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_kv_dequantize_blocks_bit_exact(gpu, dtype):
+    H, T = 4, 96  # 384 rows per slot
+    slots, refs = [], []
+    for i in range(3):
+        t = _randn((T, H, 128), i, scale=1 + i)
+        slots.append(quantize_to_fp4(t.reshape(-1, 128).to(gpu), CFG))
+        refs.append(_oracle_slot(t)[0])
+    got = dequantize_kv_cache(slots, 3, H, T, dtype, gpu)
+    assert got.shape == (1, 3 * T, H, 128) and got.dtype == dtype
+    ref = np.concatenate(refs)
+    if dtype == torch.bfloat16:
+        assert np.array_equal(got[0].float().cpu().numpy(), ref)
+    else:
+        assert np.abs(got[0].cpu().numpy() - ref).max() <= 2 ** -8 * np.abs(ref).max()
+        assert np.array_equal(o.round_bf16(got[0].cpu().numpy()), ref)
+
+
+def test_quantize_on_write_into_slot_is_bit_exact_and_in_place(gpu):
+    H, T = 2, 64
+    cache = kvc.initialize_kv_cache(1, T, 2, H, 128, CFG, gpu)[0]
+    assert not cache["k"][0].values.any() and float(cache["k"][0].amax) == 0.0
+    ptrs = [cache["k"][0].values.data_ptr(), cache["k"][0].scale_factors.data_ptr(), cache["k"][0].amax.data_ptr()]
+    q, k, v = (_randn((1, T, H, 128), s).to(gpu) for s in (1, 2, 3))
+    out, (ce, le, info) = kvc.kv_cache_attention(q, k, v, cache, 0, sink_tokens=T)
+    kvc.apply_cache_update(cache, ce, le, info, CFG)
+    _, (vals, sc, am) = _oracle_slot(k[0].cpu())
+    slot = cache["k"][0]
+    assert np.array_equal(u8(slot.values), vals) and np.array_equal(u8(slot.scale_factors), sc)
+    assert float(slot.amax.cpu()) == float(am)
+    assert ptrs == [slot.values.data_ptr(), slot.scale_factors.data_ptr(), slot.amax.data_ptr()]
+    assert int(cache["global_end_index"]) == T and int(cache["local_end_index"]) == T
+
+
+@pytest.mark.parametrize("Lq,Lk,H", [(64, 64, 1), (128, 200, 2), (100, 333, 3), (257, 130, 2)])
+def test_plain_bf16_attention(gpu, Lq, Lk, H):
+    q, k, v = _randn((Lq, H, 128), 1), _randn((Lk, H, 128), 2), _randn((Lk, H, 128), 3)
+    got = _native.attention_bf16(q.to(gpu), k.to(gpu), v.to(gpu), 128 ** -0.5)
+    ref = o.attention(q.float().numpy(), k.float().numpy(), v.float().numpy())
+    assert np.abs(got.float().cpu().numpy() - ref).max() <= 2e-2
+
+
+def test_attention_properties(gpu):
+    """Rows of softmax sum to one: with V = ones the output is all ones; a single key returns its value."""
+    q = _randn((130, 2, 128), 4).to(gpu)
+    k = _randn((77, 2, 128), 5).to(gpu)
+    ones = torch.ones(77, 2, 128, dtype=torch.bfloat16, device=gpu)
+    out = _native.attention_bf16(q, k, ones, 128 ** -0.5)
+    assert (out.float() - 1).abs().max() <= 2 ** -7
+    v1 = _randn((1, 2, 128), 6).to(gpu)
+    out = _native.attention_bf16(q, k[:1], v1, 128 ** -0.5)
+    assert torch.equal(out, v1.expand(130, 2, 128))
+
+
+@pytest.mark.parametrize("H,T,n_chunks,sink_blocks,max_blocks", [(2, 64, 6, 1, 4), (3, 128, 4, 1, 3), (2, 192, 3, 0, 2)])
+def test_cache_streaming_against_oracle(gpu, H, T, n_chunks, sink_blocks, max_blocks):
+    """Streams chunks through fill and roll phases; each chunk runs two forwards (the second one
+    re-inserts into the same slot, like the clean-context pass).  The oracle keeps a list of
+    dequantized slots and applies the reference's policy by hand."""
+    cache = kvc.initialize_kv_cache(1, T, max_blocks, H, 128, CFG, gpu)[0]
+    ref_slots_k, ref_slots_v = [None] * max_blocks, [None] * max_blocks
+    filled = 0
+    for c in range(n_chunks):
+        for fwd in range(2):
+            q, k, v = (_randn((1, T, H, 128), 100 * c + 10 * fwd + s) for s in (1, 2, 3))
+            out, (ce, le, info) = kvc.kv_cache_attention(q.to(gpu), k.to(gpu), v.to(gpu), cache, c * T,
+                                                         sink_tokens=sink_blocks * T)
+            # oracle policy
+            if fwd == 0 and filled == max_blocks:  # roll: evict the oldest non-sink slot
+                order = list(range(sink_blocks)) + list(range(sink_blocks + 1, max_blocks))
+                assert info["action"] == "roll_and_insert"
+            elif fwd == 0:
+                order = list(range(filled))
+            else:
+                order = list(range(min(filled, max_blocks) - 1))
+            ks = [ref_slots_k[i] for i in order] + [o.k_smooth(k[0].float().numpy())]
+            vs = [ref_slots_v[i] for i in order] + [v[0].float().numpy()]
+            ref = o.attention(q[0].float().numpy(), np.concatenate(ks), np.concatenate(vs))
+            err = np.abs(out[0].float().cpu().numpy() - ref).max()
+            assert err <= 2e-2, (c, fwd, err)
+            kvc.apply_cache_update(cache, ce, le, info, CFG)
+            # oracle cache update
+            if fwd == 0 and filled == max_blocks:
+                for i in range(sink_blocks, max_blocks - 1):
+                    ref_slots_k[i], ref_slots_v[i] = ref_slots_k[i + 1], ref_slots_v[i + 1]
+                dst = max_blocks - 1
+            elif fwd == 0:
+                dst = filled
+                filled += 1
+            else:
+                dst = min(filled, max_blocks) - 1
+            ref_slots_k[dst] = _oracle_slot(k[0])[0]
+            ref_slots_v[dst] = _oracle_slot(v[0])[0]
+        got_k = dequantize_kv_cache(cache["k"], max_blocks, H, T, torch.bfloat16, gpu)[0].float().cpu().numpy()
+        for i in range(min(filled, max_blocks)):
+            assert np.array_equal(got_k[i * T:(i + 1) * T], ref_slots_k[i]), (c, i)
+
+
+def test_rope_matches_oracle_bit_exact_and_complex_reference(gpu):
+    f, h, w, N = 3, 4, 6, 5
+    angles = build_rope_angles()
+    cos, sin = rope_cos_sin(angles, f, h, w, start_frame=7, device=gpu)
+    oc, os_ = o.rope_cos_sin(f, h, w, start_frame=7)
+    assert np.array_equal(cos.cpu().numpy(), oc) and np.array_equal(sin.cpu().numpy(), os_)
+    x = _randn((f * h * w + 8, N, 128), 11)
+    got = rope_apply(x.to(gpu), cos, sin, seq_len=f * h * w)
+    ref = o.rope_apply(x.float().numpy(), oc, os_, seq_len=f * h * w)
+    assert np.array_equal(got.float().cpu().numpy(), ref)
+    assert torch.equal(got[f * h * w:].cpu(), x[f * h * w:])  # tail rows pass through
+    strided = torch.zeros(f * h * w + 8, N, 256, dtype=torch.bfloat16, device=gpu)
+    strided[:, :, :128] = x.to(gpu)
+    assert torch.equal(rope_apply(strided[:, :, :128], cos, sin, seq_len=f * h * w), got)
+
+
+def test_rope_benchmark_shape_norm_preservation(gpu):
+    f, h, w = 3, 22, 40
+    cos, sin = rope_cos_sin(build_rope_angles(), f, h, w, start_frame=12, device=gpu)
+    x = _randn((f * h * w, 24, 128), 12).to(gpu)
+    y = rope_apply(x, cos, sin)
+    n_in = x.float().reshape(-1, 24, 64, 2).norm(dim=-1)
+    n_out = y.float().reshape(-1, 24, 64, 2).norm(dim=-1)
+    assert ((n_in - n_out).abs() <= 2 ** -7 * n_in + 1e-3).all()
+
+
+@pytest.mark.parametrize("L,C,fs", [(12, 256, 4), (48, 3072, 16), (6, 1000 - 1000 % 8, 3)])
+def test_adaln_against_oracle_and_torch(gpu, L, C, fs):
+    F = L // fs
+    x = _randn((1, L, C), 13)
+    sc, sh = _randn((1, F, 1, C), 14), _randn((1, F, 1, C), 15)
+    got = adaln_modulate(x.to(gpu), sc.to(gpu), sh.to(gpu), fs).float().cpu().numpy()[0]
+    ref = o.adaln_modulate(x[0].float().numpy(), sc[0, :, 0].float().numpy(), sh[0, :, 0].float().numpy(), fs)
+    diff = np.abs(got - ref)
+    assert diff.max() <= 3.1e-2 and (diff != 0).mean() < 5e-3
+    ln = torch.nn.functional.layer_norm(x.float(), (C,), eps=1e-6).bfloat16()
+    eager = (ln.unflatten(1, (F, fs)) * (1 + sc) + sh).flatten(1, 2).float().numpy()[0]
+    assert np.abs(got - eager).max() <= 3.1e-2
+
+
+def test_adaln_strided_modulation_views(gpu):
+    """scale / shift are chunk(6) views of one [B, F, 6, C] tensor in the block forward."""
+    L, C, fs = 8, 512, 4
+    x = _randn((1, L, C), 16).to(gpu)
+    e = _randn((1, 2, 6, C), 17).to(gpu)
+    parts = e.chunk(6, dim=2)
+    got = adaln_modulate(x, parts[1], parts[0], fs)
+    ref = adaln_modulate(x, parts[1].contiguous(), parts[0].contiguous(), fs)
+    assert torch.equal(got, ref)
+
+
+def test_rms_norm_against_oracle(gpu):
+    x = _randn((50, 3072), 18, scale=3.0)
+    w = (1 + 0.1 * torch.randn(3072, generator=torch.Generator().manual_seed(19))).bfloat16()
+    got = _native.rms_norm(x.to(gpu), w.to(gpu), 1e-6).float().cpu().numpy()
+    ref = o.rms_norm(x.float().numpy(), w.float().numpy())
+    diff = np.abs(got - ref)
+    assert diff.max() <= 2 ** -5 and (diff != 0).mean() < 5e-3

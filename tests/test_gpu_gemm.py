@@ -1,0 +1,141 @@
+"""GPU parity: W4A4 GEMM and the quantized Linear against the oracle's dequantize-then-fp32-matmul.
+Bar (floating point): relative Frobenius error <= 1e-3."""
+import numpy as np
+import pytest
+import torch
+import torch.nn as nn
+
+import nvfp4_oracle as o
+from helpers import activations, bits_of, u8, weights
+from longlive_amd import _native
+from longlive_amd.fouroversix import (FourOverSixLinear, ModelQuantizationConfig, QuantizationConfig,
+                                      QuantizedTensor, fp4_matmul, quantize_to_fp4)
+from longlive_amd.utils.quant import quantize_model_with_filter
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-3
+
+
+def _as_oracle(q):
+    return dict(values=u8(q.values), scales=u8(q.scale_factors), amax=np.float32(q.amax.item()),
+                rule=q.scale_rule.value, padded=q.padded_shape, orig=q.original_shape)
+
+
+def _rel(a, b):
+    return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / max(np.linalg.norm(b.astype(np.float64)), 1e-30))
+
+
+def test_integer_special_case_is_exact(gpu):
+    """Unit scales and amax = 1536: the product is an exact integer-valued matrix (bf16-representable
+    here because entries stay below 256 in magnitude for K = 64 of small codes)."""
+    rng = np.random.default_rng(0)
+    ca = rng.integers(0, 4, (128, 64)).astype(np.uint8) | (rng.integers(0, 2, (128, 64)).astype(np.uint8) << 3)
+    cb = rng.integers(0, 4, (128, 64)).astype(np.uint8) | (rng.integers(0, 2, (128, 64)).astype(np.uint8) << 3)
+    va = (ca[:, 0::2] | (ca[:, 1::2] << 4)).astype(np.uint8)
+    vb = (cb[:, 0::2] | (cb[:, 1::2] << 4)).astype(np.uint8)
+    sc = torch.full((128 * 4,), 0x38, dtype=torch.uint8, device=gpu)
+    amax = torch.tensor([1536.0], device=gpu)
+    y = _native.gemm(torch.from_numpy(va).to(gpu), sc, torch.from_numpy(vb).to(gpu), sc, 128, 128, amax_a=amax, amax_b=amax)
+    expect = o.E2M1_VALUES[ca].astype(np.float64) @ o.E2M1_VALUES[cb].astype(np.float64).T
+    assert np.array_equal(y.float().cpu().numpy().astype(np.float64), expect)
+
+
+def test_golden_matmul(golden, gpu):
+    def qt(name, shape):
+        v, s, a = (golden[f"{name}/mse/{k}"] for k in ("values", "scales", "amax"))
+        return QuantizedTensor(torch.from_numpy(v).to(gpu), torch.from_numpy(s).to(gpu).view(torch.float8_e4m3fn),
+                               torch.from_numpy(a).to(gpu), "nvfp4", shape, "mse", shape)
+
+    y = fp4_matmul(qt("randn_128x512_s1", (128, 512)), qt("weights_256x512_s2", (256, 512)))
+    ref = o.bf16_to_f32(golden["matmul/randn_128x512_s1__weights_256x512_s2/mse/out_bf16"])
+    assert _rel(y.float().cpu().numpy(), ref) <= TOL
+    diff = np.abs(bits_of(y).astype(np.int32) - golden["matmul/randn_128x512_s1__weights_256x512_s2/mse/out_bf16"].astype(np.int32))
+    assert diff.max() <= 1  # at most one bf16 ulp anywhere
+
+
+@pytest.mark.parametrize("M,N,K,seed", [(128, 128, 64, 0), (200, 192, 256, 1), (130, 70, 200, 2), (1, 3072, 128, 3),
+                                        (640, 384, 1152, 4), (300, 1000, 3072, 5)])
+def test_against_oracle(gpu, M, N, K, seed):
+    x, w = activations((M, K), seed), weights((N, K), seed + 100)
+    xq, wq = quantize_to_fp4(x.to(gpu)), quantize_to_fp4(w.to(gpu))
+    y = fp4_matmul(xq, wq)
+    assert y.shape == (M, N) and y.dtype == torch.bfloat16
+    ref = o.fp4_matmul(_as_oracle(xq), _as_oracle(wq))
+    assert _rel(y.float().cpu().numpy(), ref) <= TOL
+
+
+def test_mixed_scale_rules_and_explicit_alpha(gpu):
+    x, w = activations((128, 256), 6), weights((256, 256), 7)
+    xq = quantize_to_fp4(x.to(gpu), QuantizationConfig(scale_rule="static_6"))
+    wq = quantize_to_fp4(w.to(gpu), QuantizationConfig(scale_rule="mse"))
+    ref = o.fp4_matmul(_as_oracle(xq), _as_oracle(wq))
+    assert _rel(fp4_matmul(xq, wq).float().cpu().numpy(), ref) <= TOL
+    alpha = (xq.amax * wq.amax / (2688.0 * 1536.0)).float()
+    y = _native.gemm(xq.values, xq.scale_factors, wq.values, wq.scale_factors, 128, 256, alpha=alpha)
+    assert _rel(y.float().cpu().numpy(), ref) <= TOL
+
+
+def test_high_precision_operands_are_quantized_on_the_fly(gpu):
+    x, w = activations((128, 128), 8).to(gpu), weights((128, 128), 9).to(gpu)
+    y1 = fp4_matmul(x, w)
+    y2 = fp4_matmul(quantize_to_fp4(x), quantize_to_fp4(w))
+    assert torch.equal(y1, y2)
+
+
+def test_config1_single_linear_full_size(gpu):
+    """BASELINE config 1: X [2640, 3072] seed 0 with outliers, W [3072, 3072] ~ N(0, 0.02), rule mse."""
+    x, w = activations((2640, 3072), 0), weights((3072, 3072), 0)
+    xq, wq = quantize_to_fp4(x.to(gpu)), quantize_to_fp4(w.to(gpu))
+    y = fp4_matmul(xq, wq)
+    ref = o.fp4_matmul(_as_oracle(xq), _as_oracle(wq))
+    r = _rel(y.float().cpu().numpy(), ref)
+    assert r <= TOL, r
+
+
+def test_ffn_shapes_linearity_property(gpu):
+    """BASELINE config 2 FFN shapes (too large for a CPU matmul in a unit test): the GEMM is linear in
+    the tensor scale of A, so doubling amax_a doubles every output exactly (power of two), and rows of
+    A that are zero give zero rows."""
+    for M, N, K in ((2640, 14336, 3072), (2640, 3072, 14336)):
+        x, w = activations((M, K), 1).to(gpu), weights((N, K), 1).to(gpu)
+        x[5] = 0
+        xq, wq = quantize_to_fp4(x), quantize_to_fp4(w)
+        y = fp4_matmul(xq, wq)
+        assert y.shape == (M, N) and torch.isfinite(y.float()).all()
+        assert not y[5].any()
+        y2 = _native.gemm(xq.values, xq.scale_factors, wq.values, wq.scale_factors, M, N, amax_a=xq.amax * 2,
+                          amax_b=wq.amax)
+        assert torch.equal(y2.float(), y.float() * 2)
+        # spot-check 64 rows against the oracle
+        rows = torch.arange(0, M, M // 64)[:64]
+        a = _as_oracle(xq)
+        b = _as_oracle(wq)
+        A = o.dequantize(a["values"], a["scales"], a["amax"], "mse", a["padded"], a["orig"])[rows.numpy()]
+        B = o.dequantize(b["values"], b["scales"], b["amax"], "mse", b["padded"], b["orig"])
+        ref = o.round_bf16(A @ B.T)
+        assert _rel(y[rows.to(gpu)].float().cpu().numpy(), ref) <= TOL
+
+
+def test_linear_module_with_bias_matches_reference_semantics(gpu):
+    torch.manual_seed(0)
+    lin = nn.Linear(256, 192, bias=True).to(gpu).bfloat16()
+    model = nn.Sequential(lin)
+    model, _ = quantize_model_with_filter(model, ModelQuantizationConfig(), materialize_for_inference=True, verbose=False)
+    q = model[0]
+    assert isinstance(q, FourOverSixLinear) and q.weight is None
+    x = activations((2, 50, 256), 3).to(gpu)
+    with torch.no_grad():
+        y = q(x)
+    assert y.shape == (2, 50, 192)
+    xq = quantize_to_fp4(x.reshape(-1, 256))
+    ref = o.fp4_matmul(_as_oracle(xq), _as_oracle(q.quantized_weight()))
+    ref = o.round_bf16(ref + q.bias.float().cpu().numpy()[None, :])  # bf16 add after the bf16 GEMM result
+    got = y.reshape(-1, 192).float().cpu().numpy()
+    assert _rel(got, ref) <= TOL
+    # state-dict round trip: packed buffers reload into a fresh swapped module
+    fresh = nn.Sequential(nn.Linear(256, 192, bias=True).to(gpu).bfloat16())
+    fresh, _ = quantize_model_with_filter(fresh, ModelQuantizationConfig(), verbose=False)
+    fresh[0].weight = None
+    fresh.load_state_dict(model.state_dict(), strict=True)
+    with torch.no_grad():
+        assert torch.equal(fresh[0](x), y)

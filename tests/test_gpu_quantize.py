@@ -1,0 +1,141 @@
+"""GPU parity: NVFP4 quantize / dequantize through the C ABI against the CPU oracle and the golden
+vectors.  Bar: bit-exact packed nibbles, scale bytes and amax."""
+import numpy as np
+import pytest
+import torch
+
+import nvfp4_oracle as o
+from helpers import activations, bits_of, from_bits, u8, weights
+from longlive_amd import _native
+from longlive_amd.fouroversix import QuantizationConfig, QuantizedTensor, quantize_to_fp4
+
+pytestmark = pytest.mark.gpu
+RULES = list(o.SCALE_RULES)
+
+
+def _check(x_bits, rule, dev):
+    q = quantize_to_fp4(from_bits(x_bits, dev), QuantizationConfig(scale_rule=rule))
+    v, s, a, pad = o.quantize_to_fp4(x_bits, rule)
+    assert q.padded_shape == pad
+    assert float(q.amax.cpu()) == float(a)
+    sg = u8(q.scale_factors)
+    assert np.array_equal(sg, s), f"{rule}: {(sg != s).sum()} scale bytes differ"
+    vg = u8(q.values)
+    assert np.array_equal(vg, v), f"{rule}: {(vg != v).sum()} value bytes differ"
+    return q
+
+
+def test_hardware_e4m3_conversion_matches_software_codec(gpu):
+    x = np.concatenate([np.linspace(0, 448, 200001, dtype=np.float32),
+                        o.e4m3_decode(np.arange(127, dtype=np.uint8)),
+                        np.array([2**-10, 2**-10 * 1.001, 3 * 2**-10, 2**-9 * 2.5, 17.0, 19.0, 27.0], dtype=np.float32)])
+    got = _native.debug_convert(torch.from_numpy(x).to(gpu), 0).cpu().numpy()
+    assert np.array_equal(got, o.e4m3_encode(x))
+
+
+def test_hardware_e2m1_conversion_matches_reference_rounding(gpu):
+    x = np.concatenate([np.linspace(-6.9, 6.9, 400001, dtype=np.float32),
+                        np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, -0.25, -2.5, -5.0, -0.1, 0.0], dtype=np.float32)])
+    got = _native.debug_convert(torch.from_numpy(x).to(gpu), 1).cpu().numpy()
+    ref = o._codes_from_fake_quantized(o._fake_quantize_e2m1(x))
+    assert np.array_equal(got, ref)
+
+
+@pytest.mark.parametrize("rule", RULES)
+def test_golden_vectors(golden, gpu, rule):
+    for name in golden["case_names"]:
+        q = quantize_to_fp4(from_bits(golden[f"{name}/x"], gpu), QuantizationConfig(scale_rule=rule))
+        assert float(q.amax.cpu()) == float(golden[f"{name}/{rule}/amax"][0]), name
+        assert np.array_equal(u8(q.scale_factors), golden[f"{name}/{rule}/scales"]), name
+        assert np.array_equal(u8(q.values), golden[f"{name}/{rule}/values"]), name
+
+
+@pytest.mark.parametrize("rule", RULES)
+@pytest.mark.parametrize("shape,seed", [((128, 64), 0), ((256, 192), 1), ((130, 70), 2), ((1, 16), 3), ((257, 1000), 4)])
+def test_random_and_ragged_shapes(gpu, rule, shape, seed):
+    _check(bits_of(activations(shape, seed)), rule, gpu)
+
+
+@pytest.mark.parametrize("rule", ["mse", "static_6"])
+def test_input_classes_of_the_reference_test(gpu, rule):
+    g = torch.Generator().manual_seed(0)
+    for x in (torch.zeros(512, 1024), torch.ones(512, 1024), torch.rand(512, 1024, generator=g),
+              torch.randn(1024, 512, generator=g)):
+        _check(bits_of(x.bfloat16()), rule, gpu)
+
+
+def test_edge_values(gpu):
+    x = torch.randn(128, 128, generator=torch.Generator().manual_seed(5))
+    x[0, :16] = -0.0                      # negative zeros -> code 0
+    x[1, :16] = torch.tensor([-1e-4] * 16)  # negatives that round to zero -> code 8
+    x[2, :] *= 1e-6                       # blocks with sub-normal / zero e4m3 scales
+    x[3, :] *= 3e-5
+    x[4, 0] = 250.0                       # sets amax; other blocks far below
+    for rule in RULES:
+        _check(bits_of(x.bfloat16()), rule, gpu)
+    tiny = (torch.randn(128, 64, generator=torch.Generator().manual_seed(6)) * 1e-30).bfloat16()
+    huge = (torch.randn(128, 64, generator=torch.Generator().manual_seed(7)) * 1e30).bfloat16()
+    for t in (tiny, huge):
+        for rule in ("mse", "static_6"):
+            _check(bits_of(t), rule, gpu)
+
+
+def test_benchmark_activation_full_size(gpu):
+    """Config 1 activation [2640, 3072], seed 0, rule mse: full-size bit-exact comparison."""
+    _check(bits_of(activations((2640, 3072), 0)), "mse", gpu)
+
+
+def test_strided_input_and_given_amax(gpu):
+    big = activations((200, 512), 8).to(gpu)
+    view = big[:, 128:384]  # row stride 512, 256 columns
+    q = quantize_to_fp4(view)
+    v, s, a, _ = o.quantize_to_fp4(bits_of(view), "mse")
+    assert np.array_equal(u8(q.values), v) and np.array_equal(u8(q.scale_factors), s)
+    amax = torch.tensor([float(a) * 2], device=gpu)
+    vals, sc, am = _native.quantize(view, "mse", amax=amax)
+    v2, s2, a2, _ = o.quantize_to_fp4(bits_of(view), "mse", amax=np.float32(float(a) * 2))
+    assert np.array_equal(u8(vals), v2) and np.array_equal(u8(sc), s2) and float(am.cpu()) == float(a2)
+
+
+def test_rejects_non_bf16_and_cpu_input(gpu):
+    with pytest.raises(ValueError, match="bfloat16"):
+        quantize_to_fp4(torch.zeros(128, 64, device=gpu))
+
+
+@pytest.mark.parametrize("rule", ["mse", "static_6", "static_4"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_dequantize_matches_oracle(gpu, rule, dtype):
+    x = activations((130, 200), 9)
+    q = quantize_to_fp4(x.to(gpu), QuantizationConfig(scale_rule=rule))
+    got = q.dequantize(dtype)
+    assert got.shape == (130, 200) and got.dtype == dtype
+    ref = o.dequantize(u8(q.values), u8(q.scale_factors), np.float32(q.amax.item()), rule, q.padded_shape, (130, 200))
+    if dtype == torch.float32:
+        assert np.array_equal(got.cpu().numpy(), ref)
+    else:
+        assert torch.equal(got.cpu(), torch.from_numpy(ref).to(dtype))
+
+
+def test_dequantize_golden(golden, gpu):
+    for name, shape in (("randn_128x512_s1", (128, 512)), ("weights_256x512_s2", (256, 512))):
+        v, s, a = (golden[f"{name}/mse/{k}"] for k in ("values", "scales", "amax"))
+        qt = QuantizedTensor(torch.from_numpy(v).to(gpu), torch.from_numpy(s).to(gpu).view(torch.float8_e4m3fn),
+                             torch.from_numpy(a).to(gpu), "nvfp4", shape, "mse", shape)
+        assert np.array_equal(qt.dequantize(torch.float32).cpu().numpy(), golden[f"{name}/mse/deq_f32"])
+        assert np.array_equal(bits_of(qt.dequantize(torch.bfloat16)), golden[f"{name}/mse/deq_bf16"])
+
+
+def test_round_trip_property_at_full_ffn_size(gpu):
+    """Size-independent property at the largest benchmark activation [2640, 14336]: dequantize(quantize(x))
+    re-quantized with the same amax and a static rule reproduces the same bytes (idempotence), and the
+    relative error of the four-over-six result is not worse than plain NVFP4."""
+    x = activations((2640, 14336), 10).to(gpu)
+    q6 = quantize_to_fp4(x, QuantizationConfig(scale_rule="static_6"))
+    d6 = q6.dequantize(torch.float32)
+    qm = quantize_to_fp4(x, QuantizationConfig(scale_rule="mse"))
+    dm = qm.dequantize(torch.float32)
+    e6 = (d6 - x.float()).pow(2).sum().item()
+    em = (dm - x.float()).pow(2).sum().item()
+    assert em <= e6 * 1.0001
+    assert float(qm.amax.cpu()) == float(x.float().abs().max().cpu())
+    assert q6.values.shape == (2688, 7168) and not q6.values[2640:].any()

@@ -1,0 +1,154 @@
+"""CPU tests of the host side: the C-ABI library loads and exports every declared symbol, the
+configuration / front-end error behaviour mirrors the reference, module swap and cache policy."""
+import pytest
+import torch
+import torch.nn as nn
+
+from longlive_amd import _native
+from longlive_amd.fouroversix import (DataType, FourOverSixLinear, ModelQuantizationConfig, QuantizationConfig,
+                                      QuantizedTensor, ScaleRule, fp4_matmul, quantize_model, quantize_to_fp4)
+from longlive_amd.utils import kv_cache as kvc
+from longlive_amd.utils.quant import LongLiveQuantizationConfig, quantize_model_with_filter
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = _native.load()
+    declared = _native.declared_symbols()
+    assert len(declared) >= 13
+    for name in declared:
+        assert hasattr(lib, name), name
+    assert set(declared) == set(_native._SIGNATURES), "ctypes table and header disagree"
+    assert lib.ll_version() >= 1
+    assert lib.ll_nvfp4_quantize_workspace_floats() == 1024
+
+
+def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
+    lib = _native.load()
+    assert lib.ll_nvfp4_quantize(None, 1, 1, 1, 3, None, None, None, 0, None, None) == -1
+    assert b"null pointer" in lib.ll_last_error()
+    assert lib.ll_nvfp4_gemm_tnt(None, None, None, None, None, None, None, 1.0, 1.0, 1, 1, 128, 128, 64, None, 1,
+                                 None, None) == -1
+    assert lib.ll_rope_apply(None, 1, 1, 16, 16, 16, None, None, 1, None, None) == -1
+
+
+def test_scale_rule_tables():
+    assert [ScaleRule(r).cuda_id() for r in ("static_6", "static_4", "mae", "mse", "abs_max")] == [0, 1, 2, 3, 4]
+    assert ScaleRule.mse.max_allowed_e4m3_value() == 256 and ScaleRule.static_4.max_allowed_e2m1_value() == 4
+    assert DataType.nvfp4.block_size() == 16 and DataType.nvfp4.scale_dtype() == torch.float8_e4m3fn
+    cfg = QuantizationConfig(scale_rule="mae", backend="cuda")
+    assert cfg.scale_rule is ScaleRule.mae and cfg.dtype is DataType.nvfp4
+
+
+@pytest.mark.parametrize("kwargs", [dict(dtype="mxfp4", scale_rule="static_6"), dict(round_style="stochastic"),
+                                    dict(rht=True), dict(block_scale_2d=True), dict(transpose=True)])
+def test_unsupported_quantization_options_raise_value_error(kwargs):
+    with pytest.raises(ValueError, match="does not support"):
+        quantize_to_fp4(torch.zeros(128, 64, dtype=torch.bfloat16), QuantizationConfig(**kwargs))
+
+
+def test_front_ends_fail_loudly_off_gpu():
+    x = torch.zeros(128, 64, dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="GPU only"):
+        quantize_to_fp4(x)
+    with pytest.raises(ValueError, match="2-D"):
+        quantize_to_fp4(torch.zeros(2, 128, 64, dtype=torch.bfloat16))
+    qt = QuantizedTensor(torch.zeros(128, 32, dtype=torch.uint8), torch.zeros(128 * 4, dtype=torch.float8_e4m3fn),
+                         torch.zeros(1), "nvfp4", (128, 64), "mse")
+    assert qt.padded_shape == (128, 64)
+    other = QuantizedTensor(torch.zeros(128, 64, dtype=torch.uint8), torch.zeros(128 * 8, dtype=torch.float8_e4m3fn),
+                            torch.zeros(1), "nvfp4", (128, 128), "mse")
+    with pytest.raises(ValueError, match="same inner dimension"):
+        fp4_matmul(qt, other)
+    with pytest.raises(ValueError, match="out_dtype"):
+        fp4_matmul(qt, qt, out_dtype=DataType.float16)
+
+
+def test_quantized_tensor_pads_and_blocks_2d_scales():
+    values = torch.arange(100 * 24, dtype=torch.int64).remainder(251).to(torch.uint8).reshape(100, 24)
+    scales = torch.arange(100 * 3).remainder(120).to(torch.uint8).reshape(100, 3)
+    qt = QuantizedTensor(values, scales, torch.ones(1), DataType.nvfp4, (100, 48), ScaleRule.mse)
+    assert qt.padded_shape == (128, 64) and qt.values.shape == (128, 32) and qt.scale_factors.shape == (512,)
+    assert torch.equal(qt.values[:100, :24], values) and not qt.values[100:].any() and not qt.values[:, 24:].any()
+    from longlive_amd.fouroversix.quantize.utils import from_blocked
+
+    back = from_blocked(qt.scale_factors.view(torch.uint8), (128, 4))
+    assert torch.equal(back[:100, :3], scales) and not back[100:].any() and not back[:, 3:].any()
+    with pytest.raises(ValueError, match="scale factors"):  # 1-D scales are taken as already blocked
+        QuantizedTensor(torch.zeros(128, 32, dtype=torch.uint8), torch.zeros(300, dtype=torch.float8_e4m3fn),
+                        torch.ones(1), DataType.nvfp4, (100, 48), ScaleRule.mse)
+
+
+class _Tiny(nn.Module):
+    def __init__(self):
+        super().__init__()
+        self.text_embedding = nn.Sequential(nn.Linear(64, 64), nn.GELU(), nn.Linear(64, 64))
+        self.blocks = nn.ModuleList([nn.ModuleDict(dict(q=nn.Linear(64, 64), norm_q=nn.LayerNorm(64),
+                                                        ffn=nn.Sequential(nn.Linear(64, 128), nn.GELU(), nn.Linear(128, 64))))
+                                     for _ in range(2)])
+        self.head = nn.ModuleDict(dict(head=nn.Linear(64, 16)))
+
+
+def test_quantize_model_with_filter_swaps_only_unfiltered_linears():
+    model, matched = quantize_model_with_filter(_Tiny(), {"scale_rule": "mse"}, use_default_filtered_modules=True,
+                                                verbose=False)
+    assert isinstance(model.blocks[0]["q"], FourOverSixLinear) and isinstance(model.blocks[1]["ffn"][2], FourOverSixLinear)
+    assert type(model.text_embedding[0]) is nn.Linear and type(model.head["head"]) is nn.Linear
+    assert "head.head" in matched and "blocks.0.norm_q" in matched
+    lin = model.blocks[0]["q"]
+    assert lin.weight.dtype == torch.bfloat16
+    sd = lin.state_dict()
+    assert sd["quantized_weight_values"].shape == (64, 32) and sd["quantized_weight_values"].dtype == torch.uint8
+    assert sd["quantized_weight_scale_factors"].shape == (64 * 64 // 16,)
+    assert sd["quantized_weight_scale_factors"].dtype == torch.float8_e4m3fn
+    assert sd["quantized_weight_amax"].shape == (1,) and sd["quantized_weight_metadata"].shape == (4,)
+    with pytest.raises(TypeError):
+        quantize_model_with_filter(_Tiny(), quant_config=3, verbose=False)
+    with pytest.raises(ValueError, match="filter_profile"):
+        quantize_model_with_filter(_Tiny(), use_default_filtered_modules=True, filter_profile="nope", verbose=False)
+    cfg = ModelQuantizationConfig(modules_to_not_convert=["blocks.0.q"])
+    m2 = _Tiny()
+    quantize_model(m2, cfg)
+    assert type(m2.blocks[0]["q"]) is nn.Linear and isinstance(m2.blocks[1]["q"], FourOverSixLinear)
+
+
+def test_longlive_quantization_config_type_field():
+    assert LongLiveQuantizationConfig(scale_rule="mse", backend="cuda", type="kv").type == "kv"
+    with pytest.raises(ValueError, match="Unknown quantization type"):
+        LongLiveQuantizationConfig(type="bogus")
+
+
+def test_install_as_fouroversix_alias():
+    import longlive_amd
+
+    longlive_amd.install_as_fouroversix()
+    from fouroversix import QuantizedTensor as Q2  # noqa: PLC0415
+    from fouroversix.quantize.quantized_tensor import from_blocked  # noqa: F401, PLC0415
+
+    assert Q2 is QuantizedTensor
+
+
+def _fake_cache(blk, max_blocks):
+    return {"block_token_size": blk, "max_blocks": max_blocks, "_global_end": 0, "_local_end": 0}
+
+
+def test_cache_policy_fill_then_roll_matches_reference_numbers():
+    """Benchmark geometry: block 2640 tokens, 5 slots, sink = 1 block
+    (wan_5b/modules/causal_model.py:548-555, 623-626 evaluated by hand)."""
+    blk = 2640
+    cache = _fake_cache(blk, 5)
+    for chunk in range(5):  # fill phase: direct insert at local_end, attends slots [0, chunk)
+        for forward in range(2):  # the second forward of a chunk re-inserts into the same slot
+            slots, info, local_end = kvc.plan_cache_step(cache, chunk * blk, blk, blk, 5 * blk)
+            assert info["action"] == "direct_insert" and slots == tuple(range(chunk))
+            assert (info["local_start_index"], local_end) == (chunk * blk, (chunk + 1) * blk)
+            cache["_global_end"], cache["_local_end"] = info["current_end"], local_end
+    slots, info, local_end = kvc.plan_cache_step(cache, 5 * blk, blk, blk, 5 * blk)
+    assert info["action"] == "roll_and_insert"
+    assert (info["num_evicted_tokens"], info["num_rolled_tokens"], info["sink_tokens"]) == (2640, 7920, 2640)
+    assert (info["local_start_index"], local_end) == (10560, 13200)
+    assert slots == (0, 2, 3, 4)  # sink slot, then the three surviving window slots
+    cache["_global_end"], cache["_local_end"] = info["current_end"], local_end
+    slots, info, local_end = kvc.plan_cache_step(cache, 5 * blk, blk, blk, 5 * blk)  # forwards 2..5 of that chunk
+    assert info["action"] == "direct_insert" and slots == (0, 1, 2, 3) and info["local_start_index"] == 10560
+    with pytest.raises(NotImplementedError):
+        kvc.plan_cache_step(_fake_cache(blk, 5), 0, blk // 2, blk)
