@@ -12,8 +12,12 @@
 //
 // Tiling: 256 threads = 4 waves in a 2x2 grid, each wave owns FA x FB MFMA tiles of 32x32
 // (workgroup tile = 64*FA rows of A by 64*FB rows of B), K step 128 (64 packed bytes per row),
-// two LDS stages filled through registers.  K is consumed in a permuted order (lanes 0-31 and
-// 32-63 take alternate 32-element runs), identical for A and B, so the sum is unchanged.
+// two LDS stages filled through registers.  The kernel keeps to 256 registers per wave so that two
+// workgroups share a CU: while one wave decodes, another wave's MFMAs run.  K is consumed in a
+// permuted order (lanes 0-31 and 32-63 take alternate 32-element runs), identical for A and B, so
+// the sum is unchanged.
+#include <stdlib.h>
+
 #include "ll_common.h"
 
 namespace ll {
@@ -51,7 +55,7 @@ struct GemmSmem {
 };
 
 template <int FA, int FB>
-__global__ __launch_bounds__(kGemmThreads) void gemm_w4a4_kernel(
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
     const uint8_t* __restrict__ Av, const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bv,
     const uint8_t* __restrict__ Bs, const float* __restrict__ alpha_ptr, const float* __restrict__ amax_a,
     const float* __restrict__ amax_b, float inv_denom_a, float inv_denom_b, int M, int N, int Mp, int Np, int Kp,
@@ -101,12 +105,13 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_w4a4_kernel(
   }
   // scales: 1024 contiguous bytes per 128-row block per step (two 128x4 tiles) = 64 threads x 16 bytes
   constexpr int kARb = (BM + 127) / 128, kBRb = (BN + 127) / 128;
-  const int sgrp = tid >> 6;  // which 1024-byte run this thread copies
-  const bool s_active = sgrp < kARb + kBRb;
+  // Waves beyond the number of runs repeat run 0 (same bytes to the same place), which keeps the
+  // copy free of branches.
+  const int sgrp = (tid >> 6) < kARb + kBRb ? (tid >> 6) : 0;
   const bool s_is_a = sgrp < kARb;
-  const uint8_t* s_src = nullptr;
-  int s_dst = 0;
-  if (s_active) {
+  const uint8_t* s_src;
+  int s_dst;
+  {
     const int rbi = s_is_a ? sgrp : sgrp - kARb;
     const int rb = s_is_a ? min(row0 / 128 + rbi, Mp / 128 - 1) : min(col0 / 128 + rbi, Np / 128 - 1);
     s_src = (s_is_a ? As : Bs) + (int64_t)rb * (Kp >> 6) * 512 + (tid & 63) * 16;
@@ -115,23 +120,30 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_w4a4_kernel(
 
   uint4 a_reg[kAChunks], b_reg[kBChunks], s_reg;
   const int nk = (Kp + kBK - 1) / kBK;
+  // Kp is a multiple of 64 but maybe not of 128: in the last step the second 64 elements may not
+  // exist.  Those lanes re-read the first half (in bounds) and are masked to zero, so the loads stay
+  // unconditional.
   auto load_step = [&](int t) {
-    const bool second_half_valid = (t * kBK + 64) < Kp;  // Kp is a multiple of 64, maybe not of 128
+    const bool second_half_valid = (t * kBK + 64) < Kp;
 #pragma unroll
     for (int i = 0; i < kAChunks; ++i) {
-      const int ck = (tid + i * kGemmThreads) & 3;
-      a_reg[i] = (ck < 2 || second_half_valid) ? *reinterpret_cast<const uint4*>(a_src[i] + (int64_t)t * kRowBytes)
-                                               : make_uint4(0, 0, 0, 0);
+      const bool bad = ((tid + i * kGemmThreads) & 2) && !second_half_valid;
+      const uint32_t keep = bad ? 0u : 0xFFFFFFFFu;
+      uint4 v = *reinterpret_cast<const uint4*>(a_src[i] + (int64_t)t * kRowBytes - (bad ? 32 : 0));
+      a_reg[i] = make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
     }
 #pragma unroll
     for (int i = 0; i < kBChunks; ++i) {
-      const int ck = (tid + i * kGemmThreads) & 3;
-      b_reg[i] = (ck < 2 || second_half_valid) ? *reinterpret_cast<const uint4*>(b_src[i] + (int64_t)t * kRowBytes)
-                                               : make_uint4(0, 0, 0, 0);
+      const bool bad = ((tid + i * kGemmThreads) & 2) && !second_half_valid;
+      const uint32_t keep = bad ? 0u : 0xFFFFFFFFu;
+      uint4 v = *reinterpret_cast<const uint4*>(b_src[i] + (int64_t)t * kRowBytes - (bad ? 32 : 0));
+      b_reg[i] = make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
     }
-    if (s_active) {
-      const bool valid = ((tid & 63) < 32) || second_half_valid;
-      s_reg = valid ? *reinterpret_cast<const uint4*>(s_src + (int64_t)t * 1024) : make_uint4(0, 0, 0, 0);
+    {
+      const bool bad = ((tid & 63) >= 32) && !second_half_valid;
+      const uint32_t keep = bad ? 0u : 0xFFFFFFFFu;
+      uint4 v = *reinterpret_cast<const uint4*>(s_src + (int64_t)t * 1024 - (bad ? 512 : 0));
+      s_reg = make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
     }
   };
   auto store_step = [&](int stage) {
@@ -140,7 +152,7 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_w4a4_kernel(
     for (int i = 0; i < kAChunks; ++i) *reinterpret_cast<uint4*>(base + a_dst[i]) = a_reg[i];
 #pragma unroll
     for (int i = 0; i < kBChunks; ++i) *reinterpret_cast<uint4*>(base + b_dst[i]) = b_reg[i];
-    if (s_active) *reinterpret_cast<uint4*>(base + s_dst) = s_reg;
+    *reinterpret_cast<uint4*>(base + s_dst) = s_reg;
   };
 
   // ---- per-lane LDS read offsets
@@ -167,99 +179,133 @@ __global__ __launch_bounds__(kGemmThreads) void gemm_w4a4_kernel(
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[g][f][i] = 0.0f;
 
-  load_step(0);
-  store_step(0);
-  __syncthreads();
-
-  for (int t = 0; t < nk; ++t) {
-    if (t + 1 < nk) load_step(t + 1);
-    const uint8_t* base = smem + (t & 1) * S::kStage;
+  // Register staging of one half step (64 K elements): raw packed dwords and the two f16 block scales.
+  struct Half {
+    uint4 a[FA], b[FB];
+    half2v as[FA][2], bs[FB][2];
+  };
+  auto read_half = [&](Half& h, int stage, int cc) {
+    const uint8_t* base = smem + stage * S::kStage;
 #pragma unroll
-    for (int cc = 0; cc < 2; ++cc) {
-      uint4 araw[FA], braw[FB];
-      half2v asc[FA][2], bsc[FB][2];
-#pragma unroll
-      for (int f = 0; f < FA; ++f) {
-        araw[f] = *reinterpret_cast<const uint4*>(base + a_voff[f] + 32 * cc);
-        const uint32_t sb = *reinterpret_cast<const uint16_t*>(base + a_soff[f] + 512 * cc);
-        const half2v s = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(sb, 1.0f, false);
-        asc[f][0] = half2v{s[0], s[0]};
-        asc[f][1] = half2v{s[1], s[1]};
-      }
-#pragma unroll
-      for (int g = 0; g < FB; ++g) {
-        braw[g] = *reinterpret_cast<const uint4*>(base + b_voff[g] + 32 * cc);
-        const uint32_t sb = *reinterpret_cast<const uint16_t*>(base + b_soff[g] + 512 * cc);
-        const half2v s = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(sb, 1.0f, false);
-        bsc[g][0] = half2v{s[0], s[0]};
-        bsc[g][1] = half2v{s[1], s[1]};
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        half8v a16[FA], b16[FB];
-#pragma unroll
-        for (int f = 0; f < FA; ++f) {
-          const uint32_t w = j == 0 ? araw[f].x : j == 1 ? araw[f].y : j == 2 ? araw[f].z : araw[f].w;
-          a16[f] = decode8(w, asc[f][j >> 1]);
-        }
-#pragma unroll
-        for (int g = 0; g < FB; ++g) {
-          const uint32_t w = j == 0 ? braw[g].x : j == 1 ? braw[g].y : j == 2 ? braw[g].z : braw[g].w;
-          b16[g] = decode8(w, bsc[g][j >> 1]);
-        }
-#pragma unroll
-        for (int g = 0; g < FB; ++g)
-#pragma unroll
-          for (int f = 0; f < FA; ++f)
-            acc[g][f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(b16[g], a16[f], acc[g][f], 0, 0, 0);
-      }
+    for (int f = 0; f < FA; ++f) {
+      h.a[f] = *reinterpret_cast<const uint4*>(base + a_voff[f] + 32 * cc);
+      const uint32_t sb = *reinterpret_cast<const uint16_t*>(base + a_soff[f] + 512 * cc);
+      const half2v sc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(sb, 1.0f, false);
+      h.as[f][0] = half2v{sc[0], sc[0]};
+      h.as[f][1] = half2v{sc[1], sc[1]};
     }
-    if (t + 1 < nk) store_step((t + 1) & 1);
+#pragma unroll
+    for (int g = 0; g < FB; ++g) {
+      h.b[g] = *reinterpret_cast<const uint4*>(base + b_voff[g] + 32 * cc);
+      const uint32_t sb = *reinterpret_cast<const uint16_t*>(base + b_soff[g] + 512 * cc);
+      const half2v sc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(sb, 1.0f, false);
+      h.bs[g][0] = half2v{sc[0], sc[0]};
+      h.bs[g][1] = half2v{sc[1], sc[1]};
+    }
+  };
+  struct Operands {
+    half8v a[FA], b[FB];
+  };
+  auto decode = [&](Operands& o, const Half& h, int j) {
+#pragma unroll
+    for (int f = 0; f < FA; ++f) {
+      const uint32_t w = j == 0 ? h.a[f].x : j == 1 ? h.a[f].y : j == 2 ? h.a[f].z : h.a[f].w;
+      o.a[f] = decode8(w, h.as[f][j >> 1]);
+    }
+#pragma unroll
+    for (int g = 0; g < FB; ++g) {
+      const uint32_t w = j == 0 ? h.b[g].x : j == 1 ? h.b[g].y : j == 2 ? h.b[g].z : h.b[g].w;
+      o.b[g] = decode8(w, h.bs[g][j >> 1]);
+    }
+  };
+  auto mma = [&](const Operands& o) {
+#pragma unroll
+    for (int g = 0; g < FB; ++g)
+#pragma unroll
+      for (int f = 0; f < FA; ++f) acc[g][f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(o.b[g], o.a[f], acc[g][f], 0, 0, 0);
+  };
+  // ---- main loop: two LDS stages, global loads for step t+1 in flight while step t is computed.
+  // No software pipelining inside the wave: two workgroups share a CU and the hardware overlaps one
+  // wave's decode (VALU) with another wave's MFMAs.  The last iteration re-loads its own step
+  // (clamped index) so the loop body has no branch.
+  {
+    load_step(0);
+    store_step(0);
     __syncthreads();
+    for (int t = 0; t < nk; ++t) {
+      load_step(min(t + 1, nk - 1));
+#pragma unroll
+      for (int cc = 0; cc < 2; ++cc) {
+        Half h;
+        read_half(h, t & 1, cc);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          Operands o;
+          decode(o, h, j);
+          mma(o);
+        }
+      }
+      store_step((t + 1) & 1);
+      __syncthreads();
+    }
   }
 
   // ---- epilogue.  acc[g][f][r]: output column n = col0 + wn*32*FB + 32 g + 8 (r/4) + 4 lh + r%4,
   //                               output row    m = row0 + wm*32*FA + 32 f + l32.
+  // Each wave transposes one 32-row slab at a time through its own LDS patch (both stages are free
+  // after the last barrier) and writes rows with coalesced 16-byte stores.
   float alpha;
   if (alpha_ptr) {
     alpha = alpha_ptr[0];
   } else {
     alpha = (amax_a[0] * amax_b[0]) * (inv_denom_a * inv_denom_b);
   }
+  constexpr int kEpiPitch = 64 * FB + 16;  // bytes per slab row: 32*FB bf16 + pad
+  uint8_t* ebuf = smem + wave * (32 * kEpiPitch);
+  constexpr int kChunksPerRow = 4 * FB;     // 16-byte chunks (8 columns) per slab row
+  const int ch = lane % kChunksPerRow;      // this lane's chunk column, the same in every pass
+  const int n_lane = col0 + wn * 32 * FB + 8 * ch;
+  const bool vec_ok = ((ldd & 7) == 0) && ((reinterpret_cast<uintptr_t>(D) & 15) == 0);
+  float bias_f[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) bias_f[i] = (bias && n_lane + i < N) ? bf16_bits_to_f32(bias[n_lane + i]) : 0.0f;
 #pragma unroll
   for (int f = 0; f < FA; ++f) {
-    const int m = row0 + wm * 32 * FA + 32 * f + l32;
-    if (m >= M) continue;
-    uint16_t* drow = D + (int64_t)m * ldd;
 #pragma unroll
-    for (int g = 0; g < FB; ++g) {
+    for (int g = 0; g < FB; ++g)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
-        const int n = col0 + wn * 32 * FB + 32 * g + 8 * rg + 4 * lh;
-        if (n >= N) continue;
-        float v[4];
+        uint32_t o[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = acc[g][f][4 * rg + i] * alpha;
-        if (n + 4 <= N && ((ldd & 3) == 0)) {
-          uint32_t o[4];
+        for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16_bits(acc[g][f][4 * rg + i] * alpha);
+        *reinterpret_cast<uint2*>(ebuf + l32 * kEpiPitch + (32 * g + 8 * rg + 4 * lh) * 2) =
+            make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+      }
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
-          for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16_bits(v[i]);
-          if (bias) {
-            const uint2 bb = *reinterpret_cast<const uint2*>(bias + n);
-            const uint32_t bw[4] = {bb.x & 0xFFFFu, bb.x >> 16, bb.y & 0xFFFFu, bb.y >> 16};
+    for (int it = 0; it < (32 * kChunksPerRow) / 64; ++it) {
+      const int row = (it * 64 + lane) / kChunksPerRow;
+      const int m = row0 + wm * 32 * FA + 32 * f + row;
+      uint4 v = *reinterpret_cast<const uint4*>(ebuf + row * kEpiPitch + ch * 16);
+      if (m < M && n_lane < N) {
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        if (bias) {  // bf16 result + bf16 bias, rounded to bf16 (the separate add of the reference)
 #pragma unroll
-            for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16_bits(__uint_as_float(o[i] << 16) + __uint_as_float(bw[i] << 16));
+          for (int i = 0; i < 4; ++i) {
+            const uint32_t lo = f32_to_bf16_bits(__uint_as_float(w[i] << 16) + bias_f[2 * i]);
+            const uint32_t hi = f32_to_bf16_bits(__uint_as_float(w[i] & 0xFFFF0000u) + bias_f[2 * i + 1]);
+            w[i] = lo | (hi << 16);
           }
-          *reinterpret_cast<uint2*>(drow + n) = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+        }
+        uint16_t* dst = D + (int64_t)m * ldd + n_lane;
+        if (vec_ok && n_lane + 8 <= N) {
+          *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
         } else {
-          for (int i = 0; i < 4 && n + i < N; ++i) {
-            uint32_t o = f32_to_bf16_bits(v[i]);
-            if (bias) o = f32_to_bf16_bits(__uint_as_float(o << 16) + bf16_bits_to_f32(bias[n + i]));
-            drow[n + i] = (uint16_t)o;
-          }
+          for (int i = 0; i < 8 && n_lane + i < N; ++i) dst[i] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
         }
       }
     }
+    __builtin_amdgcn_wave_barrier();
   }
 }
 
@@ -305,32 +351,37 @@ extern "C" int ll_nvfp4_gemm_tnt(const uint8_t* A_values, const uint8_t* A_scale
   LL_REQUIRE(((reinterpret_cast<uintptr_t>(A_values) | reinterpret_cast<uintptr_t>(B_values) |
                reinterpret_cast<uintptr_t>(A_scales) | reinterpret_cast<uintptr_t>(B_scales)) & 15) == 0,
              "ll_nvfp4_gemm_tnt: operands must be 16-byte aligned");
-  LL_REQUIRE((reinterpret_cast<uintptr_t>(D) & 7) == 0 && (!bias || (reinterpret_cast<uintptr_t>(bias) & 7) == 0),
-             "ll_nvfp4_gemm_tnt: D and bias must be 8-byte aligned");
+  LL_REQUIRE((reinterpret_cast<uintptr_t>(D) & 1) == 0 && (!bias || (reinterpret_cast<uintptr_t>(bias) & 1) == 0),
+             "ll_nvfp4_gemm_tnt: D and bias must be 2-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  // Tile choice: the largest tile that still gives every CU (256) work in about whole rounds.
+  // Tile choice.  Two workgroups are resident per CU (512 slots on 256 CUs).  The 256x128 / 128x256
+  // tiles need 6 decode instructions per MFMA, the 128x128 tile 8, so the larger tiles win unless
+  // they fill the slots in whole rounds much worse.
   auto rounds_eff = [&](int bm, int bn) {
     const double tiles = (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn);
-    const double rounds = (tiles + 255.0) / 256.0;
-    return tiles / (256.0 * (double)(int64_t)rounds);
+    const double rounds = (double)(int64_t)((tiles + 511.0) / 512.0);
+    return tiles / (512.0 * rounds);
   };
   struct Cfg { int fa, fb; double bonus; };
-  const Cfg cfgs[4] = {{4, 4, 1.00}, {2, 4, 0.93}, {4, 2, 0.93}, {2, 2, 0.80}};
+  const Cfg cfgs[3] = {{4, 2, 1.00}, {2, 4, 1.00}, {2, 2, 0.85}};
   int best = 0;
   double best_score = -1.0;
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < 3; ++i) {
     const double sc = rounds_eff(64 * cfgs[i].fa, 64 * cfgs[i].fb) * cfgs[i].bonus;
     if (sc > best_score) {
       best_score = sc;
       best = i;
     }
   }
+  if (const char* force = getenv("LL_GEMM_TILE")) {  // tuning aid: 0..3 selects a tile configuration
+    const int f = atoi(force);
+    if (f >= 0 && f < 3) best = f;
+  }
 #define LL_GEMM_ARGS A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, (int)M, (int)N, \
                      (int)Mp, (int)Np, (int)Kp, D, ldd, bias, s
   switch (best) {
-    case 0: return launch_gemm<4, 4>(LL_GEMM_ARGS);
+    case 0: return launch_gemm<4, 2>(LL_GEMM_ARGS);
     case 1: return launch_gemm<2, 4>(LL_GEMM_ARGS);
-    case 2: return launch_gemm<4, 2>(LL_GEMM_ARGS);
     default: return launch_gemm<2, 2>(LL_GEMM_ARGS);
   }
 #undef LL_GEMM_ARGS
