@@ -166,6 +166,115 @@ __device__ __forceinline__ void quantize_block(const float (&X)[16], float amax,
   scale_byte = pick->scale_byte;
 }
 
+// ----------------------------------------------------------------------------- fast block math
+// Same results as quantize_block above, with the per-element divisions and software codecs replaced:
+//
+//  * everything that depends only on the scale byte s and the tensor amax is tabulated once per
+//    workgroup for the 127 finite e4m3 values:  r(s) = 1 / (dec * f32(s)),  d1(s) = ((1 * s) * amax) / 1536,
+//    d3(s) = ((1.5 * s) * amax) / 1536, each computed with the reference's operations;
+//  * the dequantized value ((q * s) * amax) / 1536 of an e2m1 value q = m * 2^k (m = 1 or 1.5) equals
+//    2^k * d1(s) or 2^k * d3(s) exactly (scaling by a power of two commutes with both roundings while
+//    nothing under- or overflows, which the caller guarantees by bounding amax);
+//  * fp32 -> e4m3 and fp32 -> e2m1 use the gfx950 conversion instructions, which round to nearest even
+//    like the reference (checked exhaustively by the test-suite); they saturate, where the reference
+//    produces out-of-range codes for |y| >= 7, so such blocks are sent to the exact path;
+//  * y = fma(x, r, +0) equals x * r and turns -0 into +0, which is what sign(y) * |q| does there;
+//  * bmax / 6 = fma(fma(-6, q0, bmax), 1/6, q0) with q0 = bmax * (1/6) is the correctly rounded
+//    quotient for every fp32 bmax (verified exhaustively on the CPU).
+struct ScaleEntry {
+  float r, d1, d3, pad;
+};
+
+typedef float float2v __attribute__((ext_vector_type(2)));
+
+template <int RULE>
+__device__ __forceinline__ float fast_candidate(const float (&X)[16], const ScaleEntry& e, uint32_t& lo,
+                                                uint32_t& hi) {
+  lo = 0;
+  hi = 0;
+#define LL_PACK(dst, base, k)                                                                         \
+  dst = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(dst, __builtin_fmaf(X[base + 2 * k], e.r, 0.0f),    \
+                                                 __builtin_fmaf(X[base + 2 * k + 1], e.r, 0.0f), 1.0f, k)
+  LL_PACK(lo, 0, 0);
+  LL_PACK(lo, 0, 1);
+  LL_PACK(lo, 0, 2);
+  LL_PACK(lo, 0, 3);
+  LL_PACK(hi, 8, 0);
+  LL_PACK(hi, 8, 1);
+  LL_PACK(hi, 8, 2);
+  LL_PACK(hi, 8, 3);
+#undef LL_PACK
+  constexpr bool kStatic = (RULE == LL_RULE_STATIC_6 || RULE == LL_RULE_STATIC_4);
+  if (kStatic) return 0.0f;
+  float t[16];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    float2v q;
+    switch (k & 3) {
+      case 0: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(k < 4 ? lo : hi, 1.0f, 0); break;
+      case 1: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(k < 4 ? lo : hi, 1.0f, 1); break;
+      case 2: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(k < 4 ? lo : hi, 1.0f, 2); break;
+      default: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(k < 4 ? lo : hi, 1.0f, 3); break;
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const float qv = q[h];
+      const float p = __uint_as_float(__float_as_uint(qv) & 0xFF800000u);  // sign and power of two of q
+      const float d = p * ((qv != p) ? e.d3 : e.d1);
+      const float err = d - X[2 * k + h];
+      t[2 * k + h] = (RULE == LL_RULE_MSE) ? err * err : fabsf(err);
+    }
+  }
+  if (RULE == LL_RULE_ABS_MAX) {
+    float m = t[0];
+#pragma unroll
+    for (int i = 1; i < 16; ++i) m = fmaxf(m, t[i]);
+    return m;
+  }
+  float acc = t[0] + t[8];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) acc = acc + (t[i] + t[i + 8]);
+  return acc;
+}
+
+// Returns false when the block has to take the exact path (an element would round past the e2m1 range).
+template <int RULE>
+__device__ __forceinline__ bool quantize_block_fast(const float (&X)[16], float enc, const ScaleEntry* tab,
+                                                    uint32_t& lo, uint32_t& hi, uint32_t& scale_byte) {
+  constexpr bool kStatic = (RULE == LL_RULE_STATIC_6 || RULE == LL_RULE_STATIC_4);
+  float bmax = fabsf(X[0]);
+#pragma unroll
+  for (int i = 1; i < 16; ++i) bmax = fmaxf(bmax, fabsf(X[i]));
+  float quot;
+  if (RULE == LL_RULE_STATIC_4) {
+    quot = bmax * 0.25f;
+  } else {
+    const float c = 1.0f / 6.0f;
+    const float q0 = bmax * c;
+    quot = __builtin_fmaf(__builtin_fmaf(-6.0f, q0, bmax), c, q0);
+  }
+  const float hp = quot * enc;
+  const uint32_t sb2 = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(hp, hp * 1.5f, 0, false);
+  const uint32_t s6 = sb2 & 0xFFu, s4 = (sb2 >> 8) & 0xFFu;
+  const ScaleEntry e6 = tab[s6];
+  if (!(bmax * e6.r < 7.0f)) return false;
+  if (kStatic) {
+    fast_candidate<RULE>(X, e6, lo, hi);
+    scale_byte = s6;
+    return true;
+  }
+  const ScaleEntry e4 = tab[s4];
+  if (!(bmax * e4.r < 7.0f)) return false;
+  uint32_t lo4, hi4;
+  const float err6 = fast_candidate<RULE>(X, e6, lo, hi);
+  const float err4 = fast_candidate<RULE>(X, e4, lo4, hi4);
+  const bool pick4 = err4 < err6;
+  lo = pick4 ? lo4 : lo;
+  hi = pick4 ? hi4 : hi;
+  scale_byte = pick4 ? s4 : s6;
+  return true;
+}
+
 // ----------------------------------------------------------------------------- quantize kernel
 // One workgroup = a 128-row x 64-column tile = 512 blocks of 16 = one 512-byte tile of the blocked
 // scale layout, which is staged in LDS and written with coalesced 4-byte stores.
@@ -177,6 +286,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
   __shared__ float s_red[kThreads / 64];
   __shared__ float s_amax;
   __shared__ uint32_t s_scales[128];  // 512 bytes in blocked order
+  __shared__ ScaleEntry s_tab[128];
 
   if (amax_given) {
     if (threadIdx.x == 0) s_amax = amax_io[0];
@@ -194,6 +304,26 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
   }
   __syncthreads();
   const float amax = s_amax;
+
+  // The fast path needs amax to be the true maximum (so block scales stay within e4m3 range) and far
+  // from the ends of the fp32 range (so powers of two scale exactly); otherwise every block takes the
+  // exact path.  The decision is uniform over the whole launch.
+  constexpr bool kStaticRule = (RULE == LL_RULE_STATIC_6 || RULE == LL_RULE_STATIC_4);
+  constexpr float kE2 = (RULE == LL_RULE_STATIC_4) ? 4.0f : 6.0f;
+  constexpr float kE4 = kStaticRule ? 448.0f : 256.0f;
+  const bool fast = !amax_given && amax >= 0x1p-100f && amax <= 0x1p100f;
+  const float enc = (kE2 * kE4) / amax;
+  if (fast && threadIdx.x < 128) {
+    const float dec = 1.0f / enc;
+    const float sf = e4m3_to_f32(threadIdx.x);
+    ScaleEntry e;
+    e.r = (threadIdx.x == 0 || threadIdx.x == 127) ? 0.0f : 1.0f / (dec * sf);
+    e.d1 = (sf * amax) / 1536.0f;
+    e.d3 = ((1.5f * sf) * amax) / 1536.0f;
+    e.pad = 0.0f;
+    s_tab[threadIdx.x] = e;
+  }
+  __syncthreads();
 
   const int64_t row0 = (int64_t)blockIdx.y * 128;
   const int64_t col0 = (int64_t)blockIdx.x * 64;
@@ -221,7 +351,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
         X[i] = (row < M && col + i < K) ? bf16_bits_to_f32(x[row * ldx + col + i]) : 0.0f;
     }
     uint32_t lo, hi, sb;
-    quantize_block<RULE>(X, amax, lo, hi, sb);
+    if (!fast || !quantize_block_fast<RULE>(X, enc, s_tab, lo, hi, sb)) quantize_block<RULE>(X, amax, lo, hi, sb);
     *reinterpret_cast<uint2*>(values + row * (Kp >> 1) + (col >> 1)) = make_uint2(lo, hi);
     s_bytes[(r & 31) * 16 + (r >> 5) * 4 + cb] = (uint8_t)sb;
   }
