@@ -1,0 +1,70 @@
+"""Streaming chunk-by-chunk generator with an NVFP4 KV cache.
+
+Mirror of the chunk / denoise loop of the reference pipeline
+(pipeline/causal_diffusion_inference.py:532-705): every chunk of ``num_frame_per_block`` latent
+frames is denoised with a few flow-matching steps against the cached context and is then run once
+more at timestep 0 so that the cache holds the clean chunk's K / V (:639-647).  The cache keeps
+``sink_size`` frames plus a sliding window, ``local_attn_size`` frames in total (:775-783).  VAE,
+text encoder and classifier-free guidance are outside this path.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..fouroversix import ModelQuantizationConfig
+from ..utils import kv_cache as kvc
+from ..utils.quant import LongLiveQuantizationConfig, quantize_model_with_filter
+from .model import CausalDiT, DiTConfig
+
+
+class StreamingGenerator:
+    def __init__(self, cfg: DiTConfig, device, timesteps=(1000.0, 750.0, 500.0, 250.0), seed: int = 0,
+                 model_quant: dict | None = None, kv_scale_rule: str = "mse") -> None:
+        self.cfg, self.device = cfg, torch.device(device)
+        self.timesteps = [float(t) for t in timesteps]
+        torch.manual_seed(seed)
+        with torch.device(self.device):
+            model = CausalDiT(cfg)
+        model.rope_angles = model.rope_angles.cpu()
+        # NVFP4 bring-up in the reference's order (inference.py:341-369): swap the block linears,
+        # quantize the weights, drop the bf16 master copies
+        model, _ = quantize_model_with_filter(
+            model, ModelQuantizationConfig(**(model_quant or {"scale_rule": "mse"})),
+            use_default_filtered_modules=True, materialize_for_inference=True, verbose=False)
+        self.model = model.eval()
+        self.kv_quant_config = LongLiveQuantizationConfig(scale_rule=kv_scale_rule, backend="cuda", type="kv")
+        self.model.kv_quant_config = self.kv_quant_config
+        self.kv_cache = None
+
+    def reset_cache(self, frame_seq_length: int) -> None:
+        cfg = self.cfg
+        block_token_size = cfg.num_frame_per_block * frame_seq_length
+        max_blocks = (cfg.local_attn_size * frame_seq_length) // block_token_size
+        self.kv_cache = kvc.initialize_kv_cache(cfg.num_layers, block_token_size, max_blocks, cfg.num_heads,
+                                                cfg.dim // cfg.num_heads, self.kv_quant_config, self.device)
+
+    @torch.no_grad()
+    def generate(self, noise: torch.Tensor, context: torch.Tensor, on_chunk=None) -> torch.Tensor:
+        """noise [1, F, C, H, W] bf16 latents, context [L, text_dim] bf16 -> denoised latents of the
+        same shape.  ``on_chunk(index)`` is called after each chunk (timing hooks)."""
+        cfg = self.cfg
+        _, F, C, H, W = noise.shape
+        fs = (H // cfg.patch_size[1]) * (W // cfg.patch_size[2])
+        if self.kv_cache is None:
+            self.reset_cache(fs)
+        out = torch.empty_like(noise)
+        nb = cfg.num_frame_per_block
+        sigmas = [t / 1000.0 for t in self.timesteps] + [0.0]
+        for ci, start in enumerate(range(0, F, nb)):
+            x = noise[0, start:start + nb].transpose(0, 1).contiguous()  # [C, f, H, W]
+            f = x.shape[1]
+            for si, t in enumerate(self.timesteps):
+                tt = torch.full((1, f), t, device=self.device, dtype=torch.float32)
+                flow = self.model(x, tt, context, self.kv_cache, start * fs)
+                x = (x.float() + (sigmas[si + 1] - sigmas[si]) * flow.float()).to(noise.dtype)
+            out[0, start:start + f] = x.transpose(0, 1)
+            # clean-context pass: rewrites this chunk's K / V in the cache
+            self.model(x, torch.zeros((1, f), device=self.device), context, self.kv_cache, start * fs)
+            if on_chunk is not None:
+                on_chunk(ci)
+        return out

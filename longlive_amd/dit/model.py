@@ -1,0 +1,221 @@
+"""Causal DiT block and model (inference with an NVFP4 KV cache).
+
+Module and parameter names follow the reference model so that its checkpoints, its module filter
+(utils/quant.py:44-58) and its NVFP4 state dicts apply unchanged:
+``CausalWanAttentionBlock`` (wan_5b/modules/causal_model.py:794-930), ``CausalWanSelfAttention``
+(:298-791), ``MultiShotT2VCrossAttention`` (:197-262), ``CausalHead`` (:933-959), ``CausalWanModel``
+(:1040-1110, forward :1485-1654).  The ten Linear layers of every block become ``FourOverSixLinear``
+through ``quantize_model_with_filter``; norms, RoPE, adaLN and attention call the gfx950 kernels;
+the bf16 ends of the model (patch / time / text embeddings, head) are plain torch modules.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+
+import torch
+import torch.nn as nn
+
+from .. import _native
+from ..utils import kv_cache as kvc
+from ..utils.adaln import adaln_modulate
+from ..utils.rope import build_rope_angles, rope_apply, rope_cos_sin
+
+
+@dataclass
+class DiTConfig:
+    """Wan2.2-TI2V-5B shape by default (wan_5b/configs/wan_ti2v_5B.py:20-29)."""
+
+    dim: int = 3072
+    ffn_dim: int = 14336
+    num_heads: int = 24
+    num_layers: int = 30
+    in_dim: int = 48
+    out_dim: int = 48
+    text_dim: int = 4096
+    text_len: int = 512
+    freq_dim: int = 256
+    patch_size: tuple = (1, 2, 2)
+    eps: float = 1e-6
+    num_frame_per_block: int = 3
+    local_attn_size: int = 15   # frames kept in the KV cache (sink + window)
+    sink_size: int = 3          # frames
+
+
+class WanRMSNorm(nn.Module):
+    """RMS norm over the full model dimension (wan_5b/modules/model.py:82-98)."""
+
+    def __init__(self, dim: int, eps: float = 1e-5) -> None:
+        super().__init__()
+        self.dim, self.eps = dim, eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return _native.rms_norm(x, self.weight.data, self.eps)
+
+
+class WanLayerNorm(nn.LayerNorm):
+    def __init__(self, dim: int, eps: float = 1e-6, elementwise_affine: bool = False) -> None:
+        super().__init__(dim, elementwise_affine=elementwise_affine, eps=eps)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return super().forward(x).type_as(x)
+
+
+class CausalSelfAttention(nn.Module):
+    def __init__(self, dim: int, num_heads: int, eps: float = 1e-6) -> None:
+        super().__init__()
+        self.dim, self.num_heads, self.head_dim = dim, num_heads, dim // num_heads
+        self.q, self.k, self.v, self.o = (nn.Linear(dim, dim) for _ in range(4))
+        self.norm_q, self.norm_k = WanRMSNorm(dim, eps), WanRMSNorm(dim, eps)
+
+    def forward(self, x, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size):
+        b, s = x.shape[:2]
+        n, d = self.num_heads, self.head_dim
+        q = self.norm_q(self.q(x)).view(b, s, n, d)
+        k = self.norm_k(self.k(x)).view(b, s, n, d)
+        v = self.v(x).view(b, s, n, d)
+        roped_q = rope_apply(q[0], cos, sin).unsqueeze(0)
+        roped_k = rope_apply(k[0], cos, sin).unsqueeze(0)
+        out, update = kvc.kv_cache_attention(roped_q, roped_k, v, kv_cache, current_start, sink_tokens,
+                                             max_attention_size=max_attention_size)
+        return self.o(out.flatten(2)), update
+
+
+class CrossAttention(nn.Module):
+    def __init__(self, dim: int, num_heads: int, eps: float = 1e-6) -> None:
+        super().__init__()
+        self.dim, self.num_heads, self.head_dim = dim, num_heads, dim // num_heads
+        self.q, self.k, self.v, self.o = (nn.Linear(dim, dim) for _ in range(4))
+        self.norm_q, self.norm_k = WanRMSNorm(dim, eps), WanRMSNorm(dim, eps)
+
+    def forward(self, x, context):
+        b, n, d = x.shape[0], self.num_heads, self.head_dim
+        q = self.norm_q(self.q(x)).view(b, -1, n, d)
+        # K / V of the text context are recomputed on every call, as the reference does (:229-235)
+        k = self.norm_k(self.k(context)).view(b, -1, n, d)
+        v = self.v(context).view(b, -1, n, d)
+        out = _native.attention_bf16(q[0].contiguous(), k[0].contiguous(), v[0].contiguous(), d ** -0.5)
+        return self.o(out.unsqueeze(0).flatten(2))
+
+
+class DiTBlock(nn.Module):
+    def __init__(self, dim: int, ffn_dim: int, num_heads: int, eps: float = 1e-6) -> None:
+        super().__init__()
+        self.dim, self.eps = dim, eps
+        self.norm1 = WanLayerNorm(dim, eps)
+        self.self_attn = CausalSelfAttention(dim, num_heads, eps)
+        self.norm3 = WanLayerNorm(dim, eps, elementwise_affine=True)
+        self.cross_attn = CrossAttention(dim, num_heads, eps)
+        self.norm2 = WanLayerNorm(dim, eps)
+        self.ffn = nn.Sequential(nn.Linear(dim, ffn_dim), nn.GELU(approximate="tanh"), nn.Linear(ffn_dim, dim))
+        self.modulation = nn.Parameter(torch.randn(1, 6, dim) / dim ** 0.5)
+
+    def forward(self, x, e, cos, sin, context, kv_cache, current_start, sink_tokens, max_attention_size=None):
+        """x [1, L, C]; e [1, F, 6, C]; returns (x, (current_end, local_end_index, cache_update_info))."""
+        num_frames, frame_seqlen = e.shape[1], x.shape[1] // e.shape[1]
+        e = (self.modulation.unsqueeze(1) + e).chunk(6, dim=2)
+        y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.eps)
+        y, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size)
+        x = x + (y.unflatten(1, (num_frames, frame_seqlen)) * e[2]).flatten(1, 2)
+        x = x + self.cross_attn(self.norm3(x), context)
+        y = self.ffn(adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps))
+        x = x + (y.unflatten(1, (num_frames, frame_seqlen)) * e[5]).flatten(1, 2)
+        return x, update
+
+
+class CausalHead(nn.Module):
+    def __init__(self, dim: int, out_dim: int, patch_size, eps: float = 1e-6) -> None:
+        super().__init__()
+        self.norm = WanLayerNorm(dim, eps)
+        self.head = nn.Linear(dim, math.prod(patch_size) * out_dim)
+        self.modulation = nn.Parameter(torch.randn(1, 2, dim) / dim ** 0.5)
+
+    def forward(self, x, e):
+        num_frames, frame_seqlen = e.shape[1], x.shape[1] // e.shape[1]
+        e = (self.modulation.unsqueeze(1) + e).chunk(2, dim=2)
+        return self.head(self.norm(x).unflatten(1, (num_frames, frame_seqlen)) * (1 + e[1]) + e[0])
+
+
+def sinusoidal_embedding_1d(dim: int, position: torch.Tensor) -> torch.Tensor:
+    half = dim // 2
+    position = position.to(torch.float64)
+    sinusoid = torch.outer(position, torch.pow(10000, -torch.arange(half, device=position.device).to(position).div(half)))
+    return torch.cat([torch.cos(sinusoid), torch.sin(sinusoid)], dim=1)
+
+
+class CausalDiT(nn.Module):
+    def __init__(self, cfg: DiTConfig) -> None:
+        super().__init__()
+        self.cfg = cfg
+        self.patch_embedding = nn.Conv3d(cfg.in_dim, cfg.dim, kernel_size=cfg.patch_size, stride=cfg.patch_size)
+        self.text_embedding = nn.Sequential(nn.Linear(cfg.text_dim, cfg.dim), nn.GELU(approximate="tanh"),
+                                            nn.Linear(cfg.dim, cfg.dim))
+        self.time_embedding = nn.Sequential(nn.Linear(cfg.freq_dim, cfg.dim), nn.SiLU(), nn.Linear(cfg.dim, cfg.dim))
+        self.time_projection = nn.Sequential(nn.SiLU(), nn.Linear(cfg.dim, cfg.dim * 6))
+        self.blocks = nn.ModuleList([DiTBlock(cfg.dim, cfg.ffn_dim, cfg.num_heads, cfg.eps) for _ in range(cfg.num_layers)])
+        self.head = CausalHead(cfg.dim, cfg.out_dim, cfg.patch_size, cfg.eps)
+        self.rope_angles = build_rope_angles(cfg.dim // cfg.num_heads)
+        self.kv_quant_config = None
+        self._rope_cache: dict = {}
+        self.init_weights()
+
+    def init_weights(self) -> None:
+        """Xavier for linears, N(0, 0.02) for the text / time MLPs, zero output head
+        (wan_5b/modules/causal_model.py:1860-1882), with a small non-zero head so that random-init
+        runs produce non-trivial outputs."""
+        for m in self.modules():
+            if isinstance(m, nn.Linear):
+                nn.init.xavier_uniform_(m.weight)
+                if m.bias is not None:
+                    nn.init.zeros_(m.bias)
+        nn.init.xavier_uniform_(self.patch_embedding.weight.flatten(1))
+        for seq in (self.text_embedding, self.time_embedding):
+            for m in seq:
+                if isinstance(m, nn.Linear):
+                    nn.init.normal_(m.weight, std=0.02)
+        nn.init.normal_(self.head.head.weight, std=0.02)
+
+    def _rope(self, f: int, h: int, w: int, start_frame: int, device) -> tuple[torch.Tensor, torch.Tensor]:
+        key = (f, h, w, start_frame, str(device))
+        if key not in self._rope_cache:
+            if len(self._rope_cache) > 64:
+                self._rope_cache.clear()
+            self._rope_cache[key] = rope_cos_sin(self.rope_angles, f, h, w, start_frame, device)
+        return self._rope_cache[key]
+
+    def unpatchify(self, x: torch.Tensor, grid) -> torch.Tensor:
+        c = self.cfg.out_dim
+        f, h, w = grid
+        u = x[: f * h * w].view(f, h, w, *self.cfg.patch_size, c)
+        u = torch.einsum("fhwpqrc->cfphqwr", u)
+        return u.reshape(c, *[i * j for i, j in zip(grid, self.cfg.patch_size)])
+
+    @torch.no_grad()
+    def forward(self, x: torch.Tensor, t: torch.Tensor, context: torch.Tensor, kv_cache: list[dict],
+                current_start: int, apply_cache_updates: bool = True) -> torch.Tensor:
+        """x [C_in, F, H, W] latents of one chunk, t [1, F] timesteps, context [L, text_dim];
+        returns the flow prediction [C_out, F, H, W] and updates the KV cache like the reference
+        (all layers' updates applied after the last block)."""
+        cfg = self.cfg
+        x = self.patch_embedding(x.unsqueeze(0))
+        f, h, w = x.shape[2:]
+        frame_seqlen = h * w
+        x = x.flatten(2).transpose(1, 2).contiguous()
+        tt = t.flatten()
+        e = self.time_embedding(sinusoidal_embedding_1d(cfg.freq_dim, tt).unflatten(0, t.shape).type_as(x))
+        e0 = self.time_projection(e).unflatten(2, (6, cfg.dim))
+        ctx = torch.cat([context, context.new_zeros(cfg.text_len - context.size(0), context.size(1))]).unsqueeze(0)
+        ctx = self.text_embedding(ctx)
+        cos, sin = self._rope(f, h, w, current_start // frame_seqlen, x.device)
+        sink_tokens = cfg.sink_size * frame_seqlen
+        max_attn = cfg.local_attn_size * frame_seqlen
+        updates = []
+        for i, block in enumerate(self.blocks):
+            x, upd = block(x, e0, cos, sin, ctx, kv_cache[i], current_start, sink_tokens, max_attn)
+            updates.append(upd)
+        if apply_cache_updates:
+            for i, (cur_end, loc_end, info) in enumerate(updates):
+                kvc.apply_cache_update(kv_cache[i], cur_end, loc_end, info, self.kv_quant_config)
+        x = self.head(x, e.unsqueeze(2))
+        return self.unpatchify(x[0].flatten(0, 1) if x.dim() == 4 else x[0], (f, h, w))

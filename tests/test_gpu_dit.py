@@ -1,0 +1,171 @@
+"""GPU tests of the DiT block and the streaming generator on top of the NVFP4 kernels."""
+import numpy as np
+import pytest
+import torch
+
+import dit_oracle
+import nvfp4_oracle as o
+from helpers import bits_of, u8
+from longlive_amd.dit import CausalDiT, DiTBlock, DiTConfig, StreamingGenerator
+from longlive_amd.fouroversix import ModelQuantizationConfig, QuantizationConfig
+from longlive_amd.utils import kv_cache as kvc
+from longlive_amd.utils.quant import quantize_model_with_filter
+from longlive_amd.utils.rope import build_rope_angles, rope_cos_sin
+
+pytestmark = pytest.mark.gpu
+KV = QuantizationConfig(scale_rule="mse")
+
+
+def _f(t):
+    return t.detach().float().cpu().numpy()
+
+
+def _oracle_params(block):
+    p = {"modulation": _f(block.modulation)[0]}
+    for name in ("self_attn.q", "self_attn.k", "self_attn.v", "self_attn.o", "cross_attn.q", "cross_attn.k",
+                 "cross_attn.v", "cross_attn.o", "ffn.0", "ffn.2"):
+        lin = block.get_submodule(name)
+        qw = lin.quantized_weight()
+        p[name + ".w"] = dict(values=u8(qw.values), scales=u8(qw.scale_factors), amax=np.float32(qw.amax.item()),
+                              rule="mse", padded=qw.padded_shape, orig=qw.original_shape)
+        p[name + ".b"] = _f(lin.bias)
+    for name in ("self_attn.norm_q", "self_attn.norm_k", "cross_attn.norm_q", "cross_attn.norm_k"):
+        p[name] = _f(block.get_submodule(name).weight)
+    p["norm3.w"], p["norm3.b"] = _f(block.norm3.weight), _f(block.norm3.bias)
+    return p
+
+
+def _rel(a, b):
+    return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / np.linalg.norm(b.astype(np.float64)))
+
+
+def test_block_against_oracle_with_cache(gpu):
+    """Reduced Wan-shaped block (dim 256, 2 heads x 128, FFN 512; chunk = 2 frames x 64 tokens), two
+    chunks so that the second one attends an FP4 slot.  Tolerance: relative Frobenius 3e-2 on the bf16
+    block output (FP4 re-quantization of activations amplifies one-ulp differences upstream)."""
+    torch.manual_seed(0)
+    dim, heads, ffn, F, h, w, T = 256, 2, 512, 2, 8, 8, 16
+    fs, L = h * w, 2 * 8 * 8
+    block = DiTBlock(dim, ffn, heads).to(gpu)
+    for m in block.modules():
+        if isinstance(m, torch.nn.Linear):
+            torch.nn.init.normal_(m.bias, std=0.1)
+    block, _ = quantize_model_with_filter(block, ModelQuantizationConfig(), use_default_filtered_modules=True,
+                                          materialize_for_inference=True, verbose=False)
+    params = _oracle_params(block)
+    cache = kvc.initialize_kv_cache(1, L, 3, heads, 128, KV, gpu)[0]
+    angles = build_rope_angles(128)
+    g = torch.Generator().manual_seed(1)
+    ctx = torch.randn(1, T, dim, generator=g).bfloat16()
+    cached_k = cached_v = None
+    for chunk in range(2):
+        x = torch.randn(1, L, dim, generator=g).bfloat16()
+        e0 = torch.randn(1, F, 6, dim, generator=g).bfloat16()
+        cos, sin = rope_cos_sin(angles, F, h, w, start_frame=chunk * F, device=gpu)
+        with torch.no_grad():
+            y, (ce, le, info) = block(x.to(gpu), e0.to(gpu), cos, sin, ctx.to(gpu), cache, chunk * L, sink_tokens=L)
+        ocs, osn = o.rope_cos_sin(F, h, w, start_frame=chunk * F)
+        ref, rk, v = dit_oracle.block_forward(_f(x)[0], _f(e0)[0], _f(ctx)[0], params, ocs, osn, cached_k, cached_v,
+                                              heads, fs)
+        r = _rel(_f(y)[0], ref)
+        assert r <= 3e-2, (chunk, r)
+        kvc.apply_cache_update(cache, ce, le, info, KV)
+        # oracle cache: quantize-on-write of this chunk's un-smoothed K and V
+        vals, sc, am, _ = o.quantize_to_fp4(o.f32_to_bf16(rk.reshape(-1, 128)), "mse")
+        cached_k = o.kv_dequantize(vals, sc, am).reshape(L, heads, 128)
+        vals, sc, am, _ = o.quantize_to_fp4(o.f32_to_bf16(v.reshape(-1, 128)), "mse")
+        cached_v = o.kv_dequantize(vals, sc, am).reshape(L, heads, 128)
+
+
+def test_config4_full_size_block_runs_and_matches_a_dequantized_torch_graph(gpu):
+    """BASELINE config 4 shape: dim 3072, 24 heads, FFN 14336, 2640 tokens, 512 text tokens, KV cache of
+    4 full slots.  The CPU oracle is too slow at this size, so the check is against the same graph
+    evaluated with torch on the GPU from the dequantized NVFP4 weights and fake-quantized activations
+    (each of those conversions is verified bit-exactly elsewhere); tolerance 3e-2 relative Frobenius."""
+    torch.manual_seed(3)
+    dim, heads, ffn, F, h, w, T = 3072, 24, 14336, 3, 22, 40, 512
+    fs, L = h * w, 3 * 22 * 40
+    block = DiTBlock(dim, ffn, heads).to(gpu)
+    block, _ = quantize_model_with_filter(block, ModelQuantizationConfig(), use_default_filtered_modules=True,
+                                          materialize_for_inference=True, verbose=False)
+    cache = kvc.initialize_kv_cache(1, L, 5, heads, 128, KV, gpu)[0]
+    g = torch.Generator().manual_seed(3)
+    angles = build_rope_angles(128)
+    ctx = torch.randn(1, T, dim, generator=g).bfloat16().to(gpu)
+    for chunk in range(5):  # fill 4 slots, then measure the 5th chunk (sink + 3 window slots + itself)
+        x = torch.randn(1, L, dim, generator=g).bfloat16().to(gpu)
+        e0 = torch.randn(1, F, 6, dim, generator=g).bfloat16().to(gpu)
+        cos, sin = rope_cos_sin(angles, F, h, w, start_frame=chunk * F, device=gpu)
+        with torch.no_grad():
+            y, (ce, le, info) = block(x, e0, cos, sin, ctx, cache, chunk * L, sink_tokens=L)
+        if chunk < 4:
+            kvc.apply_cache_update(cache, ce, le, info, KV)
+    assert torch.isfinite(y.float()).all() and y.shape == (1, L, dim)
+
+    from longlive_amd.fouroversix import quantize_to_fp4
+    from longlive_amd.utils.quant import dequantize_kv_cache, k_smooth
+
+    def lin(name, t):
+        m = block.get_submodule(name)
+        wd = m.quantized_weight().dequantize(torch.float32)
+        td = quantize_to_fp4(t.reshape(-1, t.shape[-1])).dequantize(torch.float32)
+        return ((td @ wd.T).bfloat16() + m.bias).reshape(*t.shape[:-1], -1)
+
+    def rms(name, t):
+        m = block.get_submodule(name)
+        tf = t.float()
+        return (tf * torch.rsqrt(tf.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16() * m.weight
+
+    def rope(t):
+        tc = torch.view_as_complex(t[0].double().reshape(L, heads, 64, 2))
+        fr = torch.polar(torch.ones_like(cos.double()), torch.atan2(sin.double(), cos.double())).unsqueeze(1)
+        return torch.view_as_real(tc * fr).flatten(2).bfloat16().unsqueeze(0)
+
+    def attn(q_, k_, v_):
+        return torch.nn.functional.scaled_dot_product_attention(
+            q_.transpose(1, 2).float(), k_.transpose(1, 2).float(), v_.transpose(1, 2).float()).transpose(1, 2).bfloat16()
+
+    with torch.no_grad():
+        e = (block.modulation.unsqueeze(1) + e0).chunk(6, dim=2)
+        ln = lambda t: torch.nn.functional.layer_norm(t.float(), (dim,), eps=1e-6).bfloat16()
+        mod = lambda t, sc, sh: (ln(t).unflatten(1, (F, fs)) * (1 + sc) + sh).flatten(1, 2)
+        y1 = mod(x, e[1], e[0])
+        q_ = rope(rms("self_attn.norm_q", lin("self_attn.q", y1)).view(1, L, heads, 128))
+        k_ = rope(rms("self_attn.norm_k", lin("self_attn.k", y1)).view(1, L, heads, 128))
+        v_ = lin("self_attn.v", y1).view(1, L, heads, 128)
+        ck = dequantize_kv_cache(cache["k"], 5, heads, L, torch.bfloat16, gpu)[:, :4 * L]
+        cv = dequantize_kv_cache(cache["v"], 5, heads, L, torch.bfloat16, gpu)[:, :4 * L]
+        a = attn(q_, torch.cat([ck, k_smooth(k_)], 1), torch.cat([cv, v_], 1))
+        xr = x + (lin("self_attn.o", a.flatten(2)).unflatten(1, (F, fs)) * e[2]).flatten(1, 2)
+        n3 = torch.nn.functional.layer_norm(xr.float(), (dim,), block.norm3.weight.float(), block.norm3.bias.float(), 1e-6).bfloat16()
+        cq = rms("cross_attn.norm_q", lin("cross_attn.q", n3)).view(1, L, heads, 128)
+        ckk = rms("cross_attn.norm_k", lin("cross_attn.k", ctx)).view(1, T, heads, 128)
+        cvv = lin("cross_attn.v", ctx).view(1, T, heads, 128)
+        xr = xr + lin("cross_attn.o", attn(cq, ckk, cvv).flatten(2))
+        hdn = torch.nn.functional.gelu(lin("ffn.0", mod(xr, e[4], e[3])), approximate="tanh")
+        xr = xr + (lin("ffn.2", hdn).unflatten(1, (F, fs)) * e[5]).flatten(1, 2)
+    r = _rel(_f(y)[0], _f(xr)[0])
+    assert r <= 3e-2, r
+
+
+def test_streaming_generator_small_end_to_end(gpu):
+    """Config-5-shaped run at reduced size: 2 layers, dim 256, 6 chunks of 2 frames (8x8 tokens), cache of
+    3 blocks with a 1-block sink -> exercises fill, roll and the clean-context pass."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    gen = StreamingGenerator(cfg, gpu, seed=4)
+    g = torch.Generator().manual_seed(4)
+    noise = torch.randn(1, 12, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    out = gen.generate(noise, ctx)
+    assert out.shape == noise.shape and torch.isfinite(out.float()).all()
+    assert (out.float() - noise.float()).abs().max() > 1e-3
+    c0 = gen.kv_cache[0]
+    assert c0["_global_end"] == 12 * 64 and c0["_local_end"] == 3 * 128
+    assert all(float(s.amax) > 0 for s in c0["k"])
+    # determinism and cache reset
+    gen2 = StreamingGenerator(cfg, gpu, seed=4)
+    assert torch.equal(gen2.generate(noise, ctx), out)
+    # the first chunk only depends on itself: generating just that chunk gives the same latents
+    gen3 = StreamingGenerator(cfg, gpu, seed=4)
+    assert torch.equal(gen3.generate(noise[:, :2], ctx), out[:, :2])
