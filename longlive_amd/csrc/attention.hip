@@ -62,58 +62,169 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return __builtin_bit_cast(uint32_t, p);
 }
 
-// Raw data of 16 consecutive head-dim elements of one key, as fetched from HBM.
-struct KeyChunk {
-  uint4 a, b;  // fp4: a.x,a.y = 8 packed bytes, a.z = scale byte, b.x = global scale bits; bf16: 32 bytes
-  int kind;    // 0 = fp4, 1 = bf16, 2 = beyond the end (zeros)
-};
-
-__device__ __forceinline__ KeyChunk fetch_chunk(const AttnParams& p, const SlotTable& tab, bool is_v, int64_t key,
-                                                int head, int blk) {
-  KeyChunk c;
-  c.a = make_uint4(0, 0, 0, 0);
-  c.b = make_uint4(0, 0, 0, 0);
-  if (key < p.n_cached) {
-    const int slot = (int)(key / p.bts);
-    const int64_t row = (key - (int64_t)slot * p.bts) * p.H + head;
-    const uint8_t* vals = is_v ? tab.vv[slot] : tab.kv[slot];
-    const uint8_t* scs = is_v ? tab.vs[slot] : tab.ks[slot];
-    const uint2 v = *reinterpret_cast<const uint2*>(vals + row * 64 + blk * 8);
-    c.a.x = v.x;
-    c.a.y = v.y;
-    c.a.z = scs[blocked_scale_offset(row, blk, 8)];
-    c.b.x = __float_as_uint(is_v ? tab.vg[slot] : tab.kg[slot]);
-    c.kind = 0;
-  } else if (key < p.n_cached + p.n_new) {
-    const uint16_t* src = (is_v ? p.v_new : p.k_new) + ((key - p.n_cached) * p.H + head) * kHeadDim + blk * 16;
-    c.a = reinterpret_cast<const uint4*>(src)[0];
-    c.b = reinterpret_cast<const uint4*>(src)[1];
-    c.kind = 1;
-  } else {
-    c.kind = 2;
-  }
-  return c;
+__device__ __forceinline__ float fp8_byte_to_f32(uint32_t word, int byte) {
+  typedef float float2v_ __attribute__((ext_vector_type(2)));
+  const float2v_ lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)word, false);
+  const float2v_ hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)word, true);
+  return byte == 0 ? lo[0] : byte == 1 ? lo[1] : byte == 2 ? hi[0] : hi[1];
 }
 
-// 16 bf16 values (as 8 packed dwords) of a chunk.
-__device__ __forceinline__ void chunk_to_bf16(const KeyChunk& c, uint32_t (&o)[8]) {
-  if (c.kind == 0) {
-    const float sf = e4m3_to_f32(c.a.z) * __uint_as_float(c.b.x);
-    const uint32_t w[2] = {c.a.x, c.a.y};
+// 8 e2m1 codes (one dword) times sf -> 8 floats
+__device__ __forceinline__ void fp4x8_to_f32(uint32_t w, float sf, float (&o)[8]) {
+  const float2v q0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0);
+  const float2v q1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1);
+  const float2v q2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2);
+  const float2v q3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3);
+  o[0] = q0[0] * sf; o[1] = q0[1] * sf; o[2] = q1[0] * sf; o[3] = q1[1] * sf;
+  o[4] = q2[0] * sf; o[5] = q2[1] * sf; o[6] = q3[0] * sf; o[7] = q3[1] * sf;
+}
+
+// Swizzled position of the 8-byte chunk (4 keys) `chunk` (0..15) in row `row` of a V^T tile: rows that
+// are 16 apart (written by neighbouring lanes) land in different LDS banks.
+__device__ __forceinline__ int vt_chunk(int row, int chunk) {
+  const int b = (row >> 4) & 7;
+  return chunk ^ b ^ ((b & 1) << 3);
+}
+
+// Prefetched (one iteration ahead) raw data.  Only FP4 slot data is held in registers across the MFMA
+// phase; keys of the current bf16 chunk are read when they are stored (they are a fifth of the keys, and
+// keeping 128 bytes per thread live would spill).
+struct KFetch {       // K of one key, one half of the head dimension (64 elements)
+  uint4 v0, v1;       // 32 packed bytes
+  uint32_t scales;    // 4 e4m3 block scales
+  float gs;           // amax / (e2m1_max * e4m3_max) of the slot
+  const uint4* src;   // bf16 source row (kind 1)
+  int kind;           // 0 = fp4 slot, 1 = bf16 chunk, 2 = beyond the end (zeros)
+};
+struct VFetch {       // V of one key, one 16-element block
+  uint2 v;            // 8 packed bytes
+  uint32_t scale;     // e4m3 block scale byte
+  float gs;
+  const uint4* src;
+  int kind;
+};
+
+// (slot, off) = key / block_token_size and key % block_token_size, tracked incrementally by the caller.
+__device__ __forceinline__ void fetch_k(const AttnParams& p, const SlotTable& tab, int key, int slot, int off,
+                                        int head, int half, KFetch& f) {
+  f.src = nullptr;
+  if (key < (int)p.n_cached) {
+    const int64_t row = (int64_t)off * p.H + head;
+    const uint4* src = reinterpret_cast<const uint4*>(tab.kv[slot] + row * 64 + half * 32);
+    f.v0 = src[0];
+    f.v1 = src[1];
+    f.scales = *reinterpret_cast<const uint32_t*>(tab.ks[slot] + blocked_scale_offset(row, half * 4, 8));
+    f.gs = tab.kg[slot];
+    f.kind = 0;
+  } else if (key < (int)(p.n_cached + p.n_new)) {
+    f.src = reinterpret_cast<const uint4*>(p.k_new + ((int64_t)(key - (int)p.n_cached) * p.H + head) * kHeadDim + half * 64);
+    f.kind = 1;
+  } else {
+    f.kind = 2;
+  }
+}
+
+__device__ __forceinline__ void fetch_v(const AttnParams& p, const SlotTable& tab, int key, int slot, int off,
+                                        int head, int blk, VFetch& f) {
+  f.src = nullptr;
+  if (key < (int)p.n_cached) {
+    const int64_t row = (int64_t)off * p.H + head;
+    f.v = *reinterpret_cast<const uint2*>(tab.vv[slot] + row * 64 + blk * 8);
+    f.scale = tab.vs[slot][blocked_scale_offset(row, blk, 8)];
+    f.gs = tab.vg[slot];
+    f.kind = 0;
+  } else if (key < (int)(p.n_cached + p.n_new)) {
+    f.src = reinterpret_cast<const uint4*>(p.v_new + ((int64_t)(key - (int)p.n_cached) * p.H + head) * kHeadDim + blk * 16);
+    f.kind = 1;
+  } else {
+    f.kind = 2;
+  }
+}
+
+// Decode K (64 elements of one key) to bf16 and store the 128 bytes into the key's LDS row.
+__device__ __forceinline__ void store_k(const KFetch& f, uint8_t* dst) {
+  uint4* d4 = reinterpret_cast<uint4*>(dst);
+  if (f.kind == 0) {
+    const uint32_t w[8] = {f.v0.x, f.v0.y, f.v0.z, f.v0.w, f.v1.x, f.v1.y, f.v1.z, f.v1.w};
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const float2v q0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[i], 1.0f, 0);
-      const float2v q1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[i], 1.0f, 1);
-      const float2v q2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[i], 1.0f, 2);
-      const float2v q3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w[i], 1.0f, 3);
-      o[4 * i + 0] = pack_bf16(q0[0] * sf, q0[1] * sf);
-      o[4 * i + 1] = pack_bf16(q1[0] * sf, q1[1] * sf);
-      o[4 * i + 2] = pack_bf16(q2[0] * sf, q2[1] * sf);
-      o[4 * i + 3] = pack_bf16(q3[0] * sf, q3[1] * sf);
+    for (int j = 0; j < 4; ++j) {  // block j: dwords 2j, 2j+1
+      const float sf = fp8_byte_to_f32(f.scales, j) * f.gs;
+      float lo8[8], hi8[8];
+      fp4x8_to_f32(w[2 * j], sf, lo8);
+      fp4x8_to_f32(w[2 * j + 1], sf, hi8);
+      d4[2 * j] = make_uint4(pack_bf16(lo8[0], lo8[1]), pack_bf16(lo8[2], lo8[3]), pack_bf16(lo8[4], lo8[5]),
+                             pack_bf16(lo8[6], lo8[7]));
+      d4[2 * j + 1] = make_uint4(pack_bf16(hi8[0], hi8[1]), pack_bf16(hi8[2], hi8[3]), pack_bf16(hi8[4], hi8[5]),
+                                 pack_bf16(hi8[6], hi8[7]));
+    }
+  } else if (f.kind == 1) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) d4[i] = f.src[i];
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) d4[i] = make_uint4(0, 0, 0, 0);
+  }
+}
+
+// 16 head-dim elements of 4 consecutive keys -> for every element one 8-byte run of 4 bf16 along the key
+// axis, written into the transposed (and swizzled) V tile.  vt_tile points at the tile, row0 = first d row.
+__device__ __forceinline__ void store_v4(const VFetch (&f)[4], uint8_t* vt_tile, int row0, int chunk) {
+  const bool all_fp4 = (f[0].kind | f[1].kind | f[2].kind | f[3].kind) == 0;
+  if (all_fp4) {
+    float v[4][16];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const float sf = fp8_byte_to_f32(f[kk].scale, 0) * f[kk].gs;
+      float lo8[8], hi8[8];
+      fp4x8_to_f32(f[kk].v.x, sf, lo8);
+      fp4x8_to_f32(f[kk].v.y, sf, hi8);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        v[kk][i] = lo8[i];
+        v[kk][8 + i] = hi8[i];
+      }
+    }
+#pragma unroll
+    for (int dd = 0; dd < 16; ++dd) {
+      const int row = row0 + dd;
+      *reinterpret_cast<uint2*>(vt_tile + row * kVPitch + vt_chunk(row, chunk) * 8) =
+          make_uint2(pack_bf16(v[0][dd], v[1][dd]), pack_bf16(v[2][dd], v[3][dd]));
     }
   } else {
-    o[0] = c.a.x; o[1] = c.a.y; o[2] = c.a.z; o[3] = c.a.w;
-    o[4] = c.b.x; o[5] = c.b.y; o[6] = c.b.z; o[7] = c.b.w;
+    // generic: bring every key to 8 dwords of bf16, then interleave halves across keys
+    uint32_t w[4][8];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      if (f[kk].kind == 0) {
+        const float sf = fp8_byte_to_f32(f[kk].scale, 0) * f[kk].gs;
+        float lo8[8], hi8[8];
+        fp4x8_to_f32(f[kk].v.x, sf, lo8);
+        fp4x8_to_f32(f[kk].v.y, sf, hi8);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          w[kk][i] = pack_bf16(lo8[2 * i], lo8[2 * i + 1]);
+          w[kk][4 + i] = pack_bf16(hi8[2 * i], hi8[2 * i + 1]);
+        }
+      } else if (f[kk].kind == 1) {
+        const uint4 a = f[kk].src[0], b = f[kk].src[1];
+        w[kk][0] = a.x; w[kk][1] = a.y; w[kk][2] = a.z; w[kk][3] = a.w;
+        w[kk][4] = b.x; w[kk][5] = b.y; w[kk][6] = b.z; w[kk][7] = b.w;
+      } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) w[kk][i] = 0;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      // v_perm_b32: bytes 0-3 come from the second operand, 4-7 from the first
+      const uint32_t e01 = __builtin_amdgcn_perm(w[1][i], w[0][i], 0x05040100u);
+      const uint32_t e23 = __builtin_amdgcn_perm(w[3][i], w[2][i], 0x05040100u);
+      const uint32_t o01 = __builtin_amdgcn_perm(w[1][i], w[0][i], 0x07060302u);
+      const uint32_t o23 = __builtin_amdgcn_perm(w[3][i], w[2][i], 0x07060302u);
+      const int r0 = row0 + 2 * i, r1 = r0 + 1;
+      *reinterpret_cast<uint2*>(vt_tile + r0 * kVPitch + vt_chunk(r0, chunk) * 8) = make_uint2(e01, e23);
+      *reinterpret_cast<uint2*>(vt_tile + r1 * kVPitch + vt_chunk(r1, chunk) * 8) = make_uint2(o01, o23);
+    }
   }
 }
 
@@ -166,54 +277,49 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   const int n_iter = (int)((Lk + kIterKeys - 1) / kIterKeys);
   __syncthreads();  // slot table visible
 
-  // ---- decode plan.  K: task = (key_local, 16-element block), 4 tasks per thread.
-  //                    V: one task per thread = 4 consecutive keys x one 16-element block (transposed store).
-  KeyChunk kc[4], vc[4];
-  auto fetch_iter = [&](int it) {
-    const int64_t base = (int64_t)it * kIterKeys;
+  // ---- decode plan.  K: thread = (key_local = tid / 2, half of the head dim = tid % 2).
+  //                    V: thread = (block of 16 head-dim elements = tid % 8, 4 consecutive keys = tid / 8).
+  KFetch kf;
+  VFetch vf[4];
+  // slot / offset of this thread's K key and of its first V key; both advance by kIterKeys per fetch
+  int k_key = tid >> 1, v_key = 4 * (tid >> 3);
+  int k_slot = k_key / p.bts, k_off = k_key - k_slot * p.bts;
+  int v_slot = v_key / p.bts, v_off = v_key - v_slot * p.bts;
+  auto fetch_iter = [&]() {
+    fetch_k(p, tab, k_key, k_slot, k_off, head, tid & 1, kf);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int task = tid + i * kAttnThreads;
-      kc[i] = fetch_chunk(p, tab, false, base + (task >> 3), head, task & 7);
+    for (int kk = 0; kk < 4; ++kk) {
+      const bool wrap = v_off + kk >= p.bts;
+      fetch_v(p, tab, v_key + kk, v_slot + (wrap ? 1 : 0), v_off + kk - (wrap ? p.bts : 0), head, tid & 7, vf[kk]);
     }
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) vc[kk] = fetch_chunk(p, tab, true, base + 4 * (tid >> 3) + kk, head, tid & 7);
+    k_key += kIterKeys;
+    v_key += kIterKeys;
+    k_off += kIterKeys;
+    v_off += kIterKeys;
+    while (k_off >= p.bts) {
+      k_off -= p.bts;
+      ++k_slot;
+    }
+    while (v_off >= p.bts) {
+      v_off -= p.bts;
+      ++v_slot;
+    }
   };
   auto decode_iter = [&](int stage) {
     uint8_t* kbase = smem + stage * kStageBytes;
     uint8_t* vbase = kbase + 2 * kKTileBytes;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int task = tid + i * kAttnThreads;
-      const int key_local = task >> 3, blk = task & 7;
-      uint32_t w[8];
-      chunk_to_bf16(kc[i], w);
-      uint4* dst = reinterpret_cast<uint4*>(kbase + (key_local >> 6) * kKTileBytes + (key_local & 63) * kKPitch + blk * 32);
-      dst[0] = make_uint4(w[0], w[1], w[2], w[3]);
-      dst[1] = make_uint4(w[4], w[5], w[6], w[7]);
-    }
-    uint32_t w[4][8];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) chunk_to_bf16(vc[kk], w[kk]);
-    const int key_local = 4 * (tid >> 3), blk = tid & 7;
-    uint8_t* vt = vbase + (key_local >> 6) * kVTileBytes + (key_local & 63) * 2;
-#pragma unroll
-    for (int dd = 0; dd < 16; ++dd) {
-      // element dd of each of the 4 keys -> 4 consecutive bf16 along the key axis
-      const int wi = dd >> 1;
-      uint32_t e[4];
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) e[kk] = (dd & 1) ? (w[kk][wi] >> 16) : (w[kk][wi] & 0xFFFFu);
-      *reinterpret_cast<uint2*>(vt + (blk * 16 + dd) * kVPitch) = make_uint2(e[0] | (e[1] << 16), e[2] | (e[3] << 16));
-    }
+    const int key_local = tid >> 1;
+    store_k(kf, kbase + (key_local >> 6) * kKTileBytes + (key_local & 63) * kKPitch + (tid & 1) * 128);
+    const int vkey = 4 * (tid >> 3);
+    store_v4(vf, vbase + (vkey >> 6) * kVTileBytes, (tid & 7) * 16, (vkey & 63) >> 2);
   };
 
-  fetch_iter(0);
+  fetch_iter();
   decode_iter(0);
   __syncthreads();
 
   for (int it = 0; it < n_iter; ++it) {
-    if (it + 1 < n_iter) fetch_iter(it + 1);
+    if (it + 1 < n_iter) fetch_iter();
     const int64_t tile_base = (int64_t)it * kIterKeys + kp * kTileKeys;
     if (tile_base < Lk) {
       const uint8_t* kt_base = smem + (it & 1) * kStageBytes + kp * kKTileBytes;
@@ -288,12 +394,13 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
-          const int key0 = kt * 32 + hf * 16 + 4 * lh;
+          const int chunk0 = kt * 8 + hf * 4 + lh;  // 8-byte chunk holding keys 4*chunk0 .. +3 of the tile
 #pragma unroll
           for (int dt = 0; dt < 4; ++dt) {
-            const uint8_t* src = vt_base + (dt * 32 + l32) * kVPitch + key0 * 2;
-            const uint2 v0 = *reinterpret_cast<const uint2*>(src);
-            const uint2 v1 = *reinterpret_cast<const uint2*>(src + 16);
+            const int row = dt * 32 + l32;
+            const uint8_t* src = vt_base + row * kVPitch;
+            const uint2 v0 = *reinterpret_cast<const uint2*>(src + vt_chunk(row, chunk0) * 8);
+            const uint2 v1 = *reinterpret_cast<const uint2*>(src + vt_chunk(row, chunk0 + 2) * 8);
             const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(v0.x, v0.y, v1.x, v1.y));
 #pragma unroll
             for (int qt = 0; qt < 2; ++qt) {
@@ -390,6 +497,7 @@ extern "C" int ll_kv_attention(const void* q, int64_t Lq, int num_heads, const u
              "ll_kv_attention: bad sizes Lq=%lld H=%d n_cached=%lld n_new=%lld", (long long)Lq, num_heads,
              (long long)n_cached, (long long)n_new);
   LL_REQUIRE(n_new == 0 || (k_new && v_new), "ll_kv_attention: n_new > 0 needs k_new and v_new");
+  LL_REQUIRE(n_cached + n_new < (1ll << 30) && Lq < (1ll << 30), "ll_kv_attention: sequence too long");
   int n_slots = 0;
   if (n_cached > 0) {
     LL_REQUIRE(k_values_ptrs && k_scales_ptrs && k_amax_ptrs && v_values_ptrs && v_scales_ptrs && v_amax_ptrs,
