@@ -9,7 +9,8 @@ Inputs are synthetic (seed 1) and resident in HBM before the timed region.
 
 Prints one JSON line: whole-step TFLOP/s, plus `roofline` for the dominant kernel (the FFN-up W4A4
 GEMM, timed with HIP events on the launch stream) and `cpu_baseline` (the numpy oracle of the same
-path timed on the host cores on a bounded sample).
+step timed once on the host cores).  `--workload attention|block|e2e` run BASELINE.json configs[2..4]
+alone (one kernel or model under a profiler); the default run reports them under `extras`.
 """
 from __future__ import annotations
 
@@ -24,7 +25,7 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
-M_TOKENS, M_TEXT, DIM, FFN = 2640, 512, 3072, 14336
+M_TOKENS, M_TEXT, DIM, FFN, HEADS = 2640, 512, 3072, 14336, 24
 # (name, M, K, N, count)
 LINEAR_SET = [
     ("attn_qkvo+cross_qo", M_TOKENS, DIM, DIM, 6),
@@ -33,32 +34,134 @@ LINEAR_SET = [
     ("ffn_down", M_TOKENS, FFN, DIM, 1),
 ]
 PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak (the GEMM runs v_mfma_f32_32x32x16_f16)
+# HBM-side bytes of one FFN-up GEMM launch from the rocprofv3 counter runs kept under profiles/:
+# FETCH_SIZE 82078 KiB x 2.0 (the factor a 256 MiB copy calibrates) + WRITE_SIZE 73920 KiB x 1.0
+FFN_UP_TRAFFIC_BYTES = (82078.3 * 2.0 + 73920.0) * 1024
 
 
 def step_flops() -> float:
     return sum(2.0 * m * k * n * c for _, m, k, n, c in LINEAR_SET)
 
 
-def cpu_baseline() -> dict:
-    """Oracle (numpy restatement of the reference's PyTorch path) on config 0's single linear:
-    quantize X [2640,3072] and W [3072,3072] (mse), dequantize both, fp32 matmul, round to bf16."""
+def cpu_baseline(work) -> dict:
+    """Oracle (numpy restatement of the reference's PyTorch path) over one whole step: each of the ten
+    activations quantized (mse), both operands dequantized, fp32 matmul, result rounded to bf16.  The
+    weights are the same pre-quantized operands the GPU step uses, copied to the host beforehand."""
     sys.path.insert(0, os.path.join(ROOT, "oracle"))
     import numpy as np
     import nvfp4_oracle as o
-    from helpers import activations, bits_of, weights
+    import torch
+    from helpers import bits_of
 
-    x, w = bits_of(activations((M_TOKENS, DIM), 0)), bits_of(weights((DIM, DIM), 0))
+    host = []
+    for _, x, wq in work:
+        wd = dict(values=wq.values.cpu().numpy(), scales=wq.scale_factors.cpu().view(torch.uint8).numpy(),
+                  amax=np.float32(wq.amax.item()), rule="mse", padded=tuple(wq.padded_shape), orig=tuple(wq.original_shape))
+        host.append((bits_of(x.cpu()), wd))
     t0 = time.perf_counter()
-    ops = []
-    for t in (x, w):
-        v, s, a, pad = o.quantize_to_fp4(t, "mse")
-        ops.append(dict(values=v, scales=s, amax=a, rule="mse", padded=pad, orig=t.shape))
-    y = o.fp4_matmul(ops[0], ops[1])
+    n_steps = 0
+    while n_steps < 1 or (time.perf_counter() - t0 < 10.0 and n_steps < 8):  # about 10-30 s of CPU work
+        for xb, wd in host:
+            v, sc, a, pad = o.quantize_to_fp4(xb, "mse")
+            y = o.fp4_matmul(dict(values=v, scales=sc, amax=a, rule="mse", padded=pad, orig=xb.shape), wd)
+        n_steps += 1
     dt = time.perf_counter() - t0
     assert np.isfinite(y).all()
-    flops = 2.0 * M_TOKENS * DIM * DIM
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)),
-            "kind": "port", "sample": f"config0 single W4A4 linear M=2640 K=N=3072 incl. quantize of X and W, {dt:.2f} s"}
+    return {"value": n_steps * step_flops() / dt / 1e12, "unit": "TFLOP/s",
+            "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)), "kind": "port",
+            "sample": f"{n_steps} whole step(s) of the same workload (10 linears, 783.4 GFLOP each, weights pre-quantized), {dt:.1f} s"}
+
+
+def _time_events(torch, fn, n, warm=3):
+    for _ in range(warm):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(n):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / n
+
+
+def _filled_cache(torch, dev, g):
+    """BASELINE.json configs[2]: a 5-slot FP4 cache of 2640-token blocks with slots 0..3 written
+    (sink + three window blocks) by four streaming steps, so the next chunk attends 13200 keys."""
+    from longlive_amd.fouroversix import QuantizationConfig
+    from longlive_amd.utils import kv_cache as kvc
+
+    kv_cfg = QuantizationConfig(scale_rule="mse")
+    cache = kvc.initialize_kv_cache(1, M_TOKENS, 5, HEADS, 128, kv_cfg, dev)[0]
+    for chunk in range(4):
+        q, k, v = (torch.randn(1, M_TOKENS, HEADS, 128, generator=g).bfloat16().to(dev) for _ in range(3))
+        _, (g_end, l_end, info) = kvc.kv_cache_attention(q, k, v, cache, chunk * M_TOKENS, sink_tokens=M_TOKENS)
+        kvc.apply_cache_update(cache, g_end, l_end, info, kv_cfg)
+    return cache, kv_cfg
+
+
+def run_attention(torch, dev, steps):
+    """configs[2]: 24 heads x 128, 2640 queries over 10560 cached FP4 keys + the 2640-token bf16 chunk."""
+    from longlive_amd.utils import kv_cache as kvc
+
+    g = torch.Generator().manual_seed(2)
+    cache, kv_cfg = _filled_cache(torch, dev, g)
+    q, k, v = (torch.randn(1, M_TOKENS, HEADS, 128, generator=g).bfloat16().to(dev) for _ in range(3))
+    ms = _time_events(torch, lambda: kvc.kv_cache_attention(q, k, v, cache, 4 * M_TOKENS, sink_tokens=M_TOKENS), steps)
+    flops = 4.0 * M_TOKENS * (5 * M_TOKENS) * 128 * HEADS
+    info = dict(action="direct_insert", local_start_index=4 * M_TOKENS, local_end_index=5 * M_TOKENS, new_k=k, new_v=v)
+    wms = _time_events(torch, lambda: kvc.apply_cache_update(cache, 5 * M_TOKENS, 5 * M_TOKENS, info, kv_cfg), steps)
+    return {"attention_ms": ms, "attention_TFLOPs": flops / ms / 1e9, "attention_frac_of_bf16_peak": flops / ms / 1e9 / PEAK_F16_TFLOPS,
+            "kv_write_ms": wms, "kv_write_GBs": 2 * 2.5625 * M_TOKENS * HEADS * 128 / wms / 1e6,
+            "workload": "configs[2]: Lq=2640, Lk=13200 (4 FP4 slots + bf16 chunk), 24 heads x 128, 428.2 GFLOP"}
+
+
+def run_block(torch, dev, steps):
+    """configs[3]: one DiT block (dim 3072, ffn 14336, 24 heads) on the cache of configs[2]."""
+    from longlive_amd.dit import DiTBlock
+    from longlive_amd.fouroversix import ModelQuantizationConfig
+    from longlive_amd.utils.quant import quantize_model_with_filter
+    from longlive_amd.utils.rope import build_rope_angles, rope_cos_sin
+
+    g = torch.Generator().manual_seed(3)
+    cache, _ = _filled_cache(torch, dev, g)
+    torch.manual_seed(3)
+    block = DiTBlock(DIM, FFN, HEADS).to(dev)
+    block, _ = quantize_model_with_filter(block, ModelQuantizationConfig(), use_default_filtered_modules=True,
+                                          materialize_for_inference=True, verbose=False)
+    x = torch.randn(1, M_TOKENS, DIM, generator=g).bfloat16().to(dev)
+    e0 = torch.randn(1, 3, 6, DIM, generator=g).bfloat16().to(dev)
+    ctx = torch.randn(1, M_TEXT, DIM, generator=g).bfloat16().to(dev)
+    cos, sin = rope_cos_sin(build_rope_angles(128), 3, 22, 40, 12, dev)
+    with torch.no_grad():
+        ms = _time_events(torch, lambda: block(x, e0, cos, sin, ctx, cache, 4 * M_TOKENS, sink_tokens=M_TOKENS), steps)
+    return {"block_ms": ms, "block_TFLOPs": 1228.2 / ms,
+            "workload": "configs[3]: one NVFP4 DiT block forward, 1228.2 GFLOP (783.4 linears + 428.2 self-attn + 16.6 cross-attn)"}
+
+
+def run_e2e(torch, dev):
+    """configs[4]: 30 blocks, 10 chunks of 3 latent frames, 4 denoising forwards + 1 cache-rewrite forward each."""
+    from longlive_amd.dit import DiTConfig, StreamingGenerator
+
+    gen = StreamingGenerator(DiTConfig(), dev, seed=4)
+    g = torch.Generator().manual_seed(4)
+    noise = torch.randn(1, 30, 48, 44, 80, generator=g).bfloat16().to(dev)
+    ctx = torch.randn(M_TEXT, 4096, generator=g).bfloat16().to(dev)
+    marks = []
+
+    def on_chunk(_):
+        torch.cuda.synchronize()
+        marks.append(time.perf_counter())
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    out = gen.generate(noise, ctx, on_chunk)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    per = [marks[0] - t0] + [b - a for a, b in zip(marks, marks[1:])]
+    return {"latent_frames_per_s": 30.0 / dt, "seconds_30_frames": dt, "steady_chunk_ms": 1e3 * min(per[5:]),
+            "steady_latent_frames_per_s": 3.0 / min(per[5:]), "finite": bool(torch.isfinite(out.float()).all().item()),
+            "workload": "configs[4]: 30-block NVFP4 generator, 10 chunks x (4 denoising + 1 recache) forwards, FP4 KV cache "
+                        "sink 3 + window 12 frames; first chunk includes one-time warm-up"}
 
 
 def main() -> None:
@@ -67,6 +170,8 @@ def main() -> None:
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip the attention / block / end-to-end figures")
+    ap.add_argument("--workload", choices=["linears", "attention", "block", "e2e", "copy"], default="linears")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives are part of this path); use --gpus 1")
@@ -80,6 +185,18 @@ def main() -> None:
         sys.exit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     cfg = QuantizationConfig(scale_rule="mse")
+    if args.workload == "copy":
+        # plain device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        ms = _time_events(torch, lambda: dst.copy_(src), args.steps)
+        print(json.dumps({"copy_bytes": src.numel(), "ms": ms, "GBs_read_plus_write": 2 * src.numel() / ms / 1e6}))
+        return
+    if args.workload != "linears":
+        res = {"attention": lambda: run_attention(torch, dev, args.steps), "block": lambda: run_block(torch, dev, args.steps),
+               "e2e": lambda: run_e2e(torch, dev)}[args.workload]()
+        print(json.dumps(res))
+        return
 
     # weights pre-quantized offline, activations resident in HBM
     work = []
@@ -149,13 +266,23 @@ def main() -> None:
         "config": {"workload": "configs[1]: 10 W4A4 linears of one Wan2.2-TI2V-5B block, M=2640 (512 for cross k/v), "
                                "dim 3072, ffn 14336, rule mse, seed 1", "flop_per_step": step_flops()},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_F16_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_F16_TFLOPS, "traffic": FFN_UP_TRAFFIC_BYTES,
                      "kernel": "gemm_w4a4_kernel M=2640 N=14336 K=3072", "avg_ms": gemm_ms},
         "quantize": {"shape": [M_TOKENS, FFN], "avg_ms": q_ms, "GB_per_s": q_gbs, "frac_of_hbm_8TBs": q_gbs / 8000.0,
                      "note": "amax + quantize kernels, 2.5625 algorithmic bytes per element"},
     }
+    if not args.no_extras:
+        extras = {}
+        for key, fn in (("attention", lambda: run_attention(torch, dev, 10)), ("block", lambda: run_block(torch, dev, 10)),
+                        ("e2e", lambda: run_e2e(torch, dev))):
+            try:
+                extras[key] = fn()
+            except Exception as exc:  # secondary figures must not lose the main line
+                extras[key] = {"error": f"{type(exc).__name__}: {exc}"}
+            torch.cuda.empty_cache()
+        out["extras"] = extras
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"] = cpu_baseline(work)
     print(json.dumps(out))
 
 
