@@ -99,7 +99,7 @@ int ll_kv_dequantize_blocks(const uint64_t* values_ptrs, const uint64_t* scales_
  *   q bf16 [Lq, H, 128]; k_new, v_new bf16 [n_new, H, 128] (the caller passes the smoothed K of the
  *   current chunk, utils/quant.py:797-798); out bf16 [Lq, H, 128].  No mask (causal_model.py:781).
  *   k_* / v_* pointer arrays: DEVICE arrays of device pointers, one per slot, slot layout as above
- *   (rows = token*H + head, 128 columns).  n_cached must be a multiple of 64; n_new may be 0.
+ *   (rows = token*H + head, 128 columns).  Any n_cached >= 0 and n_new >= 0 with n_cached + n_new >= 1.
  */
 int ll_kv_attention(const void* q, int64_t Lq, int num_heads,
                     const uint64_t* k_values_ptrs, const uint64_t* k_scales_ptrs, const uint64_t* k_amax_ptrs,

@@ -185,8 +185,6 @@ def test_quantization_error_bound_and_selection_invariant():
     dm, _ = res["mse"]
     err_mse = ((dm - xf) ** 2).reshape(256, 16, 16).sum(-1)
     # both candidates of four-over-six use e4m3 max 256: rebuild them with the static formula at 256
-    for rule in ("static_6", "static_4"):
-        pass
     # the chosen error can not exceed the error of plain "6" quantization with the same 256 limit,
     # which the oracle exposes as the block-wise candidate
     X = o.bf16_to_f32(x).reshape(-1, 16)
