@@ -11,6 +11,8 @@
 // S^T = K Q^T and O^T = V^T P^T (v_mfma_f32_32x32x16_bf16), so every lane owns one query column:
 // row max / row sum need no cross-lane traffic beyond one swap between the wave halves, and the
 // online-softmax rescale is a per-lane scalar.
+#include <type_traits>
+
 #include "ll_common.h"
 
 namespace ll {
@@ -79,76 +81,60 @@ __device__ __forceinline__ void fp4x8_to_f32(uint32_t w, float sf, float (&o)[8]
   o[4] = q2[0] * sf; o[5] = q2[1] * sf; o[6] = q3[0] * sf; o[7] = q3[1] * sf;
 }
 
-// Swizzled position of the 8-byte chunk (4 keys) `chunk` (0..15) in row `row` of a V^T tile: rows that
-// are 16 apart (written by neighbouring lanes) land in different LDS banks.
-__device__ __forceinline__ int vt_chunk(int row, int chunk) {
-  const int b = (row >> 4) & 7;
-  return chunk ^ b ^ ((b & 1) << 3);
-}
-
-// Prefetched (one iteration ahead) raw data.  Only FP4 slot data is held in registers across the MFMA
-// phase; keys of the current bf16 chunk are read when they are stored (they are a fifth of the keys, and
-// keeping 128 bytes per thread live would spill).
-struct KFetch {       // K of one key, one half of the head dimension (64 elements)
+// Raw FP4 data prefetched one iteration ahead.  Only packed bytes and scale bytes are held in registers
+// across the MFMA phase; everything else (slot scale, kind of key, bf16 source rows of the current chunk)
+// is re-derived from the key index when the data is decoded.
+struct KRaw {         // K of one key, one half of the head dimension (64 elements)
   uint4 v0, v1;       // 32 packed bytes
   uint32_t scales;    // 4 e4m3 block scales
-  float gs;           // amax / (e2m1_max * e4m3_max) of the slot
-  const uint4* src;   // bf16 source row (kind 1)
-  int kind;           // 0 = fp4 slot, 1 = bf16 chunk, 2 = beyond the end (zeros)
 };
-struct VFetch {       // V of one key, one 16-element block
+struct VRaw {         // V of one key, one 16-element block
   uint2 v;            // 8 packed bytes
   uint32_t scale;     // e4m3 block scale byte
-  float gs;
-  const uint4* src;
-  int kind;
 };
 
-// (slot, off) = key / block_token_size and key % block_token_size, tracked incrementally by the caller.
-__device__ __forceinline__ void fetch_k(const AttnParams& p, const SlotTable& tab, int key, int slot, int off,
-                                        int head, int half, KFetch& f) {
-  f.src = nullptr;
-  if (key < (int)p.n_cached) {
-    const int64_t row = (int64_t)off * p.H + head;
-    const uint4* src = reinterpret_cast<const uint4*>(tab.kv[slot] + row * 64 + half * 32);
-    f.v0 = src[0];
-    f.v1 = src[1];
-    f.scales = *reinterpret_cast<const uint32_t*>(tab.ks[slot] + blocked_scale_offset(row, half * 4, 8));
-    f.gs = tab.kg[slot];
-    f.kind = 0;
-  } else if (key < (int)(p.n_cached + p.n_new)) {
-    f.src = reinterpret_cast<const uint4*>(p.k_new + ((int64_t)(key - (int)p.n_cached) * p.H + head) * kHeadDim + half * 64);
-    f.kind = 1;
-  } else {
-    f.kind = 2;
-  }
+// Load through a pointer that is known to address global memory.  Slot pointers come out of a table, so
+// the compiler would otherwise emit flat loads, whose completion also counts as an LDS event and stalls
+// the first LDS wait that follows.
+template <typename T>
+__device__ __forceinline__ T load_global(const void* ptr) {
+  return *(const __attribute__((address_space(1))) T*)ptr;
+}
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 load_global_b128(const void* ptr) {
+  const u32x4 v = load_global<u32x4>(ptr);
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ uint2 load_global_b64(const void* ptr) {
+  const u32x2 v = load_global<u32x2>(ptr);
+  return make_uint2(v[0], v[1]);
 }
 
-__device__ __forceinline__ void fetch_v(const AttnParams& p, const SlotTable& tab, int key, int slot, int off,
-                                        int head, int blk, VFetch& f) {
-  f.src = nullptr;
-  if (key < (int)p.n_cached) {
-    const int64_t row = (int64_t)off * p.H + head;
-    f.v = *reinterpret_cast<const uint2*>(tab.vv[slot] + row * 64 + blk * 8);
-    f.scale = tab.vs[slot][blocked_scale_offset(row, blk, 8)];
-    f.gs = tab.vg[slot];
-    f.kind = 0;
-  } else if (key < (int)(p.n_cached + p.n_new)) {
-    f.src = reinterpret_cast<const uint4*>(p.v_new + ((int64_t)(key - (int)p.n_cached) * p.H + head) * kHeadDim + blk * 16);
-    f.kind = 1;
-  } else {
-    f.kind = 2;
-  }
+// (slot, off) = key / block_token_size and key % block_token_size, tracked incrementally by the caller.
+__device__ __forceinline__ void fetch_k(const SlotTable& tab, int H, int slot, int off, int head, int half, KRaw& f) {
+  const int64_t row = (int64_t)off * H + head;
+  const uint8_t* src = tab.kv[slot] + row * 64 + half * 32;
+  f.v0 = load_global_b128(src);
+  f.v1 = load_global_b128(src + 16);
+  f.scales = load_global<uint32_t>(tab.ks[slot] + blocked_scale_offset(row, half * 4, 8));
+}
+
+__device__ __forceinline__ void fetch_v(const SlotTable& tab, int H, int slot, int off, int head, int blk, VRaw& f) {
+  const int64_t row = (int64_t)off * H + head;
+  f.v = load_global_b64(tab.vv[slot] + row * 64 + blk * 8);
+  f.scale = load_global<uint8_t>(tab.vs[slot] + blocked_scale_offset(row, blk, 8));
 }
 
 // Decode K (64 elements of one key) to bf16 and store the 128 bytes into the key's LDS row.
-__device__ __forceinline__ void store_k(const KFetch& f, uint8_t* dst) {
+// kind: 0 = fp4 slot data in f (gs = slot amax / (e2m1_max * e4m3_max)), 1 = bf16 row at src, 2 = zeros.
+__device__ __forceinline__ void store_k(const KRaw& f, int kind, float gs, const uint4* src, uint8_t* dst) {
   uint4* d4 = reinterpret_cast<uint4*>(dst);
-  if (f.kind == 0) {
+  if (kind == 0) {
     const uint32_t w[8] = {f.v0.x, f.v0.y, f.v0.z, f.v0.w, f.v1.x, f.v1.y, f.v1.z, f.v1.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {  // block j: dwords 2j, 2j+1
-      const float sf = fp8_byte_to_f32(f.scales, j) * f.gs;
+      const float sf = fp8_byte_to_f32(f.scales, j) * gs;
       float lo8[8], hi8[8];
       fp4x8_to_f32(w[2 * j], sf, lo8);
       fp4x8_to_f32(w[2 * j + 1], sf, hi8);
@@ -157,9 +143,9 @@ __device__ __forceinline__ void store_k(const KFetch& f, uint8_t* dst) {
       d4[2 * j + 1] = make_uint4(pack_bf16(hi8[0], hi8[1]), pack_bf16(hi8[2], hi8[3]), pack_bf16(hi8[4], hi8[5]),
                                  pack_bf16(hi8[6], hi8[7]));
     }
-  } else if (f.kind == 1) {
+  } else if (kind == 1) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) d4[i] = f.src[i];
+    for (int i = 0; i < 8; ++i) d4[i] = src[i];
   } else {
 #pragma unroll
     for (int i = 0; i < 8; ++i) d4[i] = make_uint4(0, 0, 0, 0);
@@ -167,14 +153,16 @@ __device__ __forceinline__ void store_k(const KFetch& f, uint8_t* dst) {
 }
 
 // 16 head-dim elements of 4 consecutive keys -> for every element one 8-byte run of 4 bf16 along the key
-// axis, written into the transposed (and swizzled) V tile.  vt_tile points at the tile, row0 = first d row.
-__device__ __forceinline__ void store_v4(const VFetch (&f)[4], uint8_t* vt_tile, int row0, int chunk) {
-  const bool all_fp4 = (f[0].kind | f[1].kind | f[2].kind | f[3].kind) == 0;
+// axis, written into the transposed V tile.  vt_tile points at the tile, row0 = first d row.
+// kind / gs / src per key as in store_k (src = the key's 16 bf16 elements).
+__device__ __forceinline__ void store_v4(const VRaw (&f)[4], const int (&kind)[4], const float (&gs)[4],
+                                         const uint4* const (&src)[4], uint8_t* vt_tile, int row0, int chunk) {
+  const bool all_fp4 = (kind[0] | kind[1] | kind[2] | kind[3]) == 0;
   if (all_fp4) {
     float v[4][16];
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      const float sf = fp8_byte_to_f32(f[kk].scale, 0) * f[kk].gs;
+      const float sf = fp8_byte_to_f32(f[kk].scale, 0) * gs[kk];
       float lo8[8], hi8[8];
       fp4x8_to_f32(f[kk].v.x, sf, lo8);
       fp4x8_to_f32(f[kk].v.y, sf, hi8);
@@ -187,7 +175,7 @@ __device__ __forceinline__ void store_v4(const VFetch (&f)[4], uint8_t* vt_tile,
 #pragma unroll
     for (int dd = 0; dd < 16; ++dd) {
       const int row = row0 + dd;
-      *reinterpret_cast<uint2*>(vt_tile + row * kVPitch + vt_chunk(row, chunk) * 8) =
+      *reinterpret_cast<uint2*>(vt_tile + row * kVPitch + chunk * 8) =
           make_uint2(pack_bf16(v[0][dd], v[1][dd]), pack_bf16(v[2][dd], v[3][dd]));
     }
   } else {
@@ -195,8 +183,8 @@ __device__ __forceinline__ void store_v4(const VFetch (&f)[4], uint8_t* vt_tile,
     uint32_t w[4][8];
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      if (f[kk].kind == 0) {
-        const float sf = fp8_byte_to_f32(f[kk].scale, 0) * f[kk].gs;
+      if (kind[kk] == 0) {
+        const float sf = fp8_byte_to_f32(f[kk].scale, 0) * gs[kk];
         float lo8[8], hi8[8];
         fp4x8_to_f32(f[kk].v.x, sf, lo8);
         fp4x8_to_f32(f[kk].v.y, sf, hi8);
@@ -205,8 +193,8 @@ __device__ __forceinline__ void store_v4(const VFetch (&f)[4], uint8_t* vt_tile,
           w[kk][i] = pack_bf16(lo8[2 * i], lo8[2 * i + 1]);
           w[kk][4 + i] = pack_bf16(hi8[2 * i], hi8[2 * i + 1]);
         }
-      } else if (f[kk].kind == 1) {
-        const uint4 a = f[kk].src[0], b = f[kk].src[1];
+      } else if (kind[kk] == 1) {
+        const uint4 a = src[kk][0], b = src[kk][1];
         w[kk][0] = a.x; w[kk][1] = a.y; w[kk][2] = a.z; w[kk][3] = a.w;
         w[kk][4] = b.x; w[kk][5] = b.y; w[kk][6] = b.z; w[kk][7] = b.w;
       } else {
@@ -222,8 +210,8 @@ __device__ __forceinline__ void store_v4(const VFetch (&f)[4], uint8_t* vt_tile,
       const uint32_t o01 = __builtin_amdgcn_perm(w[1][i], w[0][i], 0x07060302u);
       const uint32_t o23 = __builtin_amdgcn_perm(w[3][i], w[2][i], 0x07060302u);
       const int r0 = row0 + 2 * i, r1 = r0 + 1;
-      *reinterpret_cast<uint2*>(vt_tile + r0 * kVPitch + vt_chunk(r0, chunk) * 8) = make_uint2(e01, e23);
-      *reinterpret_cast<uint2*>(vt_tile + r1 * kVPitch + vt_chunk(r1, chunk) * 8) = make_uint2(o01, o23);
+      *reinterpret_cast<uint2*>(vt_tile + r0 * kVPitch + chunk * 8) = make_uint2(e01, e23);
+      *reinterpret_cast<uint2*>(vt_tile + r1 * kVPitch + chunk * 8) = make_uint2(o01, o23);
     }
   }
 }
@@ -249,8 +237,8 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     tab.ks[tid] = reinterpret_cast<const uint8_t*>(p.ks_ptrs[tid]);
     tab.vv[tid] = reinterpret_cast<const uint8_t*>(p.vv_ptrs[tid]);
     tab.vs[tid] = reinterpret_cast<const uint8_t*>(p.vs_ptrs[tid]);
-    tab.kg[tid] = *reinterpret_cast<const float*>(p.ka_ptrs[tid]) * p.inv_denom;
-    tab.vg[tid] = *reinterpret_cast<const float*>(p.va_ptrs[tid]) * p.inv_denom;
+    tab.kg[tid] = load_global<float>(reinterpret_cast<const void*>(p.ka_ptrs[tid])) * p.inv_denom;
+    tab.vg[tid] = load_global<float>(reinterpret_cast<const void*>(p.va_ptrs[tid])) * p.inv_denom;
   }
 
   // Q fragments: B operand, lane = query column, 8 consecutive head-dim elements per k-step
@@ -273,145 +261,294 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       for (int i = 0; i < 16; ++i) o[dt][qt][i] = 0.0f;
   float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
 
-  const int64_t Lk = p.n_cached + p.n_new;
-  const int n_iter = (int)((Lk + kIterKeys - 1) / kIterKeys);
+  const int n_iter = (int)((p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys);
   __syncthreads();  // slot table visible
 
   // ---- decode plan.  K: thread = (key_local = tid / 2, half of the head dim = tid % 2).
-  //                    V: thread = (block of 16 head-dim elements = tid % 8, 4 consecutive keys = tid / 8).
-  KFetch kf;
-  VFetch vf[4];
-  // slot / offset of this thread's K key and of its first V key; both advance by kIterKeys per fetch
-  int k_key = tid >> 1, v_key = 4 * (tid >> 3);
+  //                    V: wave = (64-key tile = wave / 2, four of the eight 16-element blocks = wave % 2),
+  //                       lane = (4 consecutive keys = lane % 16, block = lane / 16): for one head-dim row
+  //                       a wave writes four full 128-byte rows of V^T, which the 136-byte pitch spreads
+  //                       over all LDS banks.
+  // Schedule of iteration `it`: the MFMAs work on LDS stage it & 1 while the raw FP4 bytes of iteration
+  // it + 1 (already in registers) are decoded into the other stage: K during the S phase, V during the PV
+  // phase, so the conversion arithmetic runs under the MFMAs.  As soon as the K (V) registers are free
+  // the raw bytes of iteration it + 2 are requested, which gives each load most of an iteration to land.
+  KRaw kf;
+  VRaw vf[4];
+  const int n_cached = (int)p.n_cached, Lk_i = (int)(p.n_cached + p.n_new);
+  const int v_blk = (lane >> 4) + 4 * (wave & 1), v_chunk = lane & 15, v_tile = wave >> 1;
+  // key, slot and offset in the slot of this thread's K key and of its first V key for the iteration whose
+  // raw data is in kf / vf
+  int k_key = tid >> 1, v_key = v_tile * kTileKeys + 4 * v_chunk;
   int k_slot = k_key / p.bts, k_off = k_key - k_slot * p.bts;
   int v_slot = v_key / p.bts, v_off = v_key - v_slot * p.bts;
-  auto fetch_iter = [&]() {
-    fetch_k(p, tab, k_key, k_slot, k_off, head, tid & 1, kf);
+  const int k_dst_off = ((tid >> 1) >> 6) * kKTileBytes + ((tid >> 1) & 63) * kKPitch + (tid & 1) * 128;
+  const int v_dst_off = 2 * kKTileBytes + v_tile * kVTileBytes + (v_blk * 16) * kVPitch + v_chunk * 8;
+
+  auto fetch_k_next = [&]() __attribute__((always_inline)) {
+    if (k_key < n_cached) fetch_k(tab, p.H, k_slot, k_off, head, tid & 1, kf);
+  };
+  auto fetch_v_next = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
       const bool wrap = v_off + kk >= p.bts;
-      fetch_v(p, tab, v_key + kk, v_slot + (wrap ? 1 : 0), v_off + kk - (wrap ? p.bts : 0), head, tid & 7, vf[kk]);
+      if (v_key + kk < n_cached)
+        fetch_v(tab, p.H, v_slot + (wrap ? 1 : 0), v_off + kk - (wrap ? p.bts : 0), head, v_blk, vf[kk]);
     }
+  };
+  auto advance_k = [&]() __attribute__((always_inline)) {
     k_key += kIterKeys;
-    v_key += kIterKeys;
     k_off += kIterKeys;
-    v_off += kIterKeys;
     while (k_off >= p.bts) {
       k_off -= p.bts;
       ++k_slot;
     }
+  };
+  auto advance_v = [&]() __attribute__((always_inline)) {
+    v_key += kIterKeys;
+    v_off += kIterKeys;
     while (v_off >= p.bts) {
       v_off -= p.bts;
       ++v_slot;
     }
   };
-  auto decode_iter = [&](int stage) {
-    uint8_t* kbase = smem + stage * kStageBytes;
-    uint8_t* vbase = kbase + 2 * kKTileBytes;
-    const int key_local = tid >> 1;
-    store_k(kf, kbase + (key_local >> 6) * kKTileBytes + (key_local & 63) * kKPitch + (tid & 1) * 128);
-    const int vkey = 4 * (tid >> 3);
-    store_v4(vf, vbase + (vkey >> 6) * kVTileBytes, (tid & 7) * 16, (vkey & 63) >> 2);
+  auto decode_k_any = [&](int stage) __attribute__((always_inline)) {
+    const int kind = k_key < n_cached ? 0 : (k_key < Lk_i ? 1 : 2);
+    const float gs = kind == 0 ? tab.kg[k_slot] : 0.0f;
+    const uint4* src = reinterpret_cast<const uint4*>(
+        p.k_new + ((int64_t)(k_key - n_cached) * p.H + head) * kHeadDim + (tid & 1) * 64);  // read only if kind == 1
+    store_k(kf, kind, gs, src, smem + stage * kStageBytes + k_dst_off);
+  };
+  auto decode_v_any = [&](int stage) __attribute__((always_inline)) {
+    int kind[4];
+    float gs[4];
+    const uint4* src[4];
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const int key = v_key + kk;
+      kind[kk] = key < n_cached ? 0 : (key < Lk_i ? 1 : 2);
+      gs[kk] = kind[kk] == 0 ? tab.vg[v_slot + (v_off + kk >= p.bts ? 1 : 0)] : 0.0f;
+      src[kk] = reinterpret_cast<const uint4*>(p.v_new + ((int64_t)(key - n_cached) * p.H + head) * kHeadDim + v_blk * 16);
+    }
+    store_v4(vf, kind, gs, src, smem + stage * kStageBytes + 2 * kKTileBytes + v_tile * kVTileBytes, v_blk * 16, v_chunk);
   };
 
-  fetch_iter();
-  decode_iter(0);
-  __syncthreads();
-
-  for (int it = 0; it < n_iter; ++it) {
-    if (it + 1 < n_iter) fetch_iter();
-    const int64_t tile_base = (int64_t)it * kIterKeys + kp * kTileKeys;
-    if (tile_base < Lk) {
-      const uint8_t* kt_base = smem + (it & 1) * kStageBytes + kp * kKTileBytes;
-      const uint8_t* vt_base = smem + (it & 1) * kStageBytes + 2 * kKTileBytes + kp * kVTileBytes;
-      // ---- S^T = K Q^T  (64 keys x 64 queries)
-      float16v s[2][2];
+  // One iteration handles the wave's 64-key tile as two 32-key halves: S half -> running max -> P, PV half.
+  // S^T of one half (32 keys x 64 queries).  kDecode = 1: convert the prefetched FP4 K row (8 dwords, one
+  // per MFMA step) between the MFMAs; kDecode = 2: convert the prefetched FP4 V data (4 keys x 16 elements,
+  // one quarter every second step); 0: nothing.
+  float16v s[2];
+  auto s_half = [&](const uint8_t* kt_base, int kt, auto decode_tag, uint8_t* dst) __attribute__((always_inline)) {
+    constexpr int kDecode = decltype(decode_tag)::value;
+    float gs = 0.0f, sfv[4] = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (kDecode == 1) gs = tab.kg[k_slot];
+    if constexpr (kDecode == 2) {
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+      for (int kk = 0; kk < 4; ++kk)
+        sfv[kk] = fp8_byte_to_f32(vf[kk].scale, 0) * tab.vg[v_slot + (v_off + kk >= p.bts ? 1 : 0)];
+    }
+    const uint32_t w[8] = {kf.v0.x, kf.v0.y, kf.v0.z, kf.v0.w, kf.v1.x, kf.v1.y, kf.v1.z, kf.v1.w};
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt)
+    for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) s[kt][qt][i] = 0.0f;
+      for (int i = 0; i < 16; ++i) s[qt][i] = 0.0f;
+    // K fragments are read two steps ahead of their MFMAs, and in program order before the LDS stores of
+    // the interleaved conversion (the compiler cannot prove those stores go to the other stage).
+    const uint8_t* krow = kt_base + (kt * 32 + l32) * kKPitch + lh * 16;
+    uint4 afrag[8];
+    afrag[0] = *reinterpret_cast<const uint4*>(krow);
+    afrag[1] = *reinterpret_cast<const uint4*>(krow + 32);
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
+    for (int ks = 0; ks < 8; ++ks) {
+      if (ks + 2 < 8) afrag[ks + 2] = *reinterpret_cast<const uint4*>(krow + (ks + 2) * 32);
+      __builtin_amdgcn_sched_barrier(0);  // keep the read up here instead of next to its MFMA
+      const bf16x8 a = __builtin_bit_cast(bf16x8, afrag[ks]);
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-          const bf16x8 a = __builtin_bit_cast(
-              bf16x8, *reinterpret_cast<const uint4*>(kt_base + (kt * 32 + l32) * kKPitch + ks * 32 + lh * 16));
+      for (int qt = 0; qt < 2; ++qt) s[qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[qt][ks], s[qt], 0, 0, 0);
+      if constexpr (kDecode == 1) {
+        const float sf = fp8_byte_to_f32(kf.scales, ks >> 1) * gs;
+        float v8[8];
+        fp4x8_to_f32(w[ks], sf, v8);
+        reinterpret_cast<uint4*>(dst)[ks] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
+                                                        pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
+      }
+      if constexpr (kDecode == 2) {
+        if (ks & 1) {
+          // piece: elements 4 * piece .. + 3 of the thread's 16, for its 4 keys
+          const int piece = ks >> 1;
+          float e[4][4];
 #pragma unroll
-          for (int qt = 0; qt < 2; ++qt) s[kt][qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[qt][ks], s[kt][qt], 0, 0, 0);
+          for (int kk = 0; kk < 4; ++kk) {
+            const uint32_t word = (piece & 2) ? vf[kk].v.y : vf[kk].v.x;
+            const float2v lo = (piece & 1) ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2)
+                                           : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0);
+            const float2v hi = (piece & 1) ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3)
+                                           : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1);
+            e[kk][0] = lo[0] * sfv[kk];
+            e[kk][1] = lo[1] * sfv[kk];
+            e[kk][2] = hi[0] * sfv[kk];
+            e[kk][3] = hi[1] * sfv[kk];
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            *reinterpret_cast<uint2*>(dst + (4 * piece + j) * kVPitch) =
+                make_uint2(pack_bf16(e[0][j], e[1][j]), pack_bf16(e[2][j], e[3][j]));
         }
       }
-      // ---- mask keys beyond the end (only the last tile)
-      if (tile_base + kTileKeys > Lk) {
+    }
+  };
+
+  // Reference point of the exponentials.  m_run is not the exact running maximum: it is raised only when
+  // the maximum has grown by more than kRescaleStep (in the exp2 domain) since it was last raised, so P can
+  // reach 2^kRescaleStep instead of 1 (harmless in fp32 / bf16) and the 128 accumulator registers per lane
+  // are rescaled a handful of times per kernel instead of at almost every tile.  The final division by
+  // the row sum, which is accumulated against the same reference, makes the result independent of it.
+  constexpr float kRescaleStep = 8.0f;
+  float neg[2];
+  auto softmax_max = [&]() __attribute__((always_inline)) {
+    float alpha[2];
 #pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
+    for (int qt = 0; qt < 2; ++qt) {
+      float mx = s[qt][0];
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int64_t key = tile_base + kt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-            if (key >= Lk) {
-              s[kt][0][r] = -INFINITY;
-              s[kt][1][r] = -INFINITY;
-            }
-          }
-      }
-      // ---- online softmax (per lane: one query per qt)
-      uint32_t pb[2][2][2][4];  // [qt][kt][half of the 32 keys][4 dwords = 8 bf16]
+      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[qt][r]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const bool raise = (mx - m_run[qt]) * p.scale_log2 > kRescaleStep;  // also true for m_run = -inf
+      const float m_new = raise ? mx : m_run[qt];
+      alpha[qt] = raise ? __builtin_amdgcn_exp2f((m_run[qt] - m_new) * p.scale_log2) : 1.0f;
+      neg[qt] = -m_new * p.scale_log2;
+      m_run[qt] = m_new;
+    }
+    if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f) != 0) {
 #pragma unroll
       for (int qt = 0; qt < 2; ++qt) {
-        float mx = s[0][qt][0];
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[kt][qt][r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run[qt], mx);
-        const float alpha = __builtin_amdgcn_exp2f((m_run[qt] - m_new) * p.scale_log2);
-        const float neg = -m_new * p.scale_log2;
-        float sum = 0.0f;
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-          float pr[16];
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            pr[r] = __builtin_amdgcn_exp2f(fmaf(s[kt][qt][r], p.scale_log2, neg));
-            sum += pr[r];
-          }
-#pragma unroll
-          for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) pb[qt][kt][hf][i] = pack_bf16(pr[8 * hf + 2 * i], pr[8 * hf + 2 * i + 1]);
-        }
-        l_run[qt] = l_run[qt] * alpha + sum;
-        m_run[qt] = m_new;
+        l_run[qt] *= alpha[qt];
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) o[dt][qt][i] *= alpha;
+          for (int i = 0; i < 16; ++i) o[dt][qt][i] *= alpha[qt];
       }
-      // ---- O^T += V^T P^T.  k-slot e of wave half lh <-> key 16 step + 8 (e / 4) + 4 lh + e % 4
+    }
+  };
+
+  // P = exp2(...) sixteen keys at a time, then O^T += V^T P^T for those keys.  k-slot e of wave half lh
+  // <-> key 16 hf + 8 (e / 4) + 4 lh + e % 4 of the 32-key half tile.
+  auto pv_half = [&](const uint8_t* vt_base, int kt) __attribute__((always_inline)) {
+    float sum[2] = {0.0f, 0.0f};
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+    for (int hf = 0; hf < 2; ++hf) {
+      // V^T fragments of this step first, so that their LDS latency runs under the exponentials
+      const int chunk0 = kt * 8 + hf * 4 + lh;  // 8-byte chunk holding keys 4*chunk0 .. +3 of the tile
+      uint2 vfrag[4][2];
 #pragma unroll
-        for (int hf = 0; hf < 2; ++hf) {
-          const int chunk0 = kt * 8 + hf * 4 + lh;  // 8-byte chunk holding keys 4*chunk0 .. +3 of the tile
+      for (int dt = 0; dt < 4; ++dt) {
+        const uint8_t* src = vt_base + (dt * 32 + l32) * kVPitch;
+        vfrag[dt][0] = *reinterpret_cast<const uint2*>(src + chunk0 * 8);
+        vfrag[dt][1] = *reinterpret_cast<const uint2*>(src + (chunk0 + 2) * 8);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // keep the reads up here instead of next to their MFMAs
+      bf16x8 pb[2];
 #pragma unroll
-          for (int dt = 0; dt < 4; ++dt) {
-            const int row = dt * 32 + l32;
-            const uint8_t* src = vt_base + row * kVPitch;
-            const uint2 v0 = *reinterpret_cast<const uint2*>(src + vt_chunk(row, chunk0) * 8);
-            const uint2 v1 = *reinterpret_cast<const uint2*>(src + vt_chunk(row, chunk0 + 2) * 8);
-            const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(v0.x, v0.y, v1.x, v1.y));
+      for (int qt = 0; qt < 2; ++qt) {
+        uint32_t w[4];
 #pragma unroll
-            for (int qt = 0; qt < 2; ++qt) {
-              const bf16x8 b = __builtin_bit_cast(
-                  bf16x8, make_uint4(pb[qt][kt][hf][0], pb[qt][kt][hf][1], pb[qt][kt][hf][2], pb[qt][kt][hf][3]));
-              o[dt][qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, o[dt][qt], 0, 0, 0);
+        for (int i = 0; i < 4; ++i) {
+          const float p0 = __builtin_amdgcn_exp2f(fmaf(s[qt][8 * hf + 2 * i], p.scale_log2, neg[qt]));
+          const float p1 = __builtin_amdgcn_exp2f(fmaf(s[qt][8 * hf + 2 * i + 1], p.scale_log2, neg[qt]));
+          sum[qt] += p0 + p1;
+          w[i] = pack_bf16(p0, p1);
+        }
+        pb[qt] = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+      }
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt) {
+        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(vfrag[dt][0].x, vfrag[dt][0].y, vfrag[dt][1].x, vfrag[dt][1].y));
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) o[dt][qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[qt], o[dt][qt], 0, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int qt = 0; qt < 2; ++qt) l_run[qt] += sum[qt];
+  };
+  using Tag0 = std::integral_constant<int, 0>;
+  using Tag1 = std::integral_constant<int, 1>;
+  using Tag2 = std::integral_constant<int, 2>;
+
+  // prologue: stage 0 <- iteration 0, raw registers <- iteration 1
+  fetch_k_next();
+  fetch_v_next();
+  decode_k_any(0);
+  decode_v_any(0);
+  advance_k();
+  advance_v();
+  if (n_iter > 1) {
+    fetch_k_next();
+    fetch_v_next();
+  }
+  __syncthreads();
+  // Every load issued so far (Q fragments, first tiles) has to have landed before the loop: otherwise the
+  // compiler's wait-count bookkeeping carries them into the loop and makes the MFMA phase wait for the
+  // prefetch loads it has just issued.  0x0F70 = vmcnt(0), other counters untouched.
+  __builtin_amdgcn_s_waitcnt(0x0F70);
+
+  // Iterations whose own 128 keys all exist and whose successor is all FP4 form a prefix of the key range;
+  // they run the interleaved body.  The rest (the bf16 chunk, the tail) runs the plain body in a loop of
+  // its own, so that its large temporaries do not add to the register pressure of the first loop.
+  int n_fast = n_cached / kIterKeys - 1;
+  n_fast = n_fast < 0 ? 0 : (n_fast > n_iter ? n_iter : n_fast);
+  int it = 0;
+  for (; it < n_fast; ++it) {
+    const uint8_t* cur = smem + (it & 1) * kStageBytes;
+    uint8_t* nxt = smem + ((it + 1) & 1) * kStageBytes;
+    const uint8_t* kt_base = cur + kp * kKTileBytes;
+    const uint8_t* vt_base = cur + 2 * kKTileBytes + kp * kVTileBytes;
+    const bool has_next2 = it + 2 < n_iter;
+    s_half(kt_base, 0, Tag1{}, nxt + k_dst_off);
+    advance_k();
+    if (has_next2) fetch_k_next();
+    softmax_max();
+    pv_half(vt_base, 0);
+    s_half(kt_base, 1, Tag2{}, nxt + v_dst_off);
+    advance_v();
+    if (has_next2) fetch_v_next();
+    softmax_max();
+    pv_half(vt_base, 1);
+    __syncthreads();
+  }
+  for (; it < n_iter; ++it) {
+    const uint8_t* cur = smem + (it & 1) * kStageBytes;
+    const uint8_t* kt_base = cur + kp * kKTileBytes;
+    const uint8_t* vt_base = cur + 2 * kKTileBytes + kp * kVTileBytes;
+    const int tile_base = it * kIterKeys + kp * kTileKeys;
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      const int half_base = tile_base + kt * 32;
+      if (half_base < Lk_i) {
+        s_half(kt_base, kt, Tag0{}, nullptr);
+        if (half_base + 32 > Lk_i) {  // mask keys beyond the end (only in the last tile)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int key = half_base + 8 * (r >> 2) + 4 * lh + (r & 3);
+            if (key >= Lk_i) {
+              s[0][r] = -INFINITY;
+              s[1][r] = -INFINITY;
             }
           }
         }
+        softmax_max();
+        pv_half(vt_base, kt);
+      }
     }
-    if (it + 1 < n_iter) decode_iter((it + 1) & 1);
+    if (it + 1 < n_iter) {
+      decode_k_any((it + 1) & 1);
+      decode_v_any((it + 1) & 1);
+      advance_k();
+      advance_v();
+      if (it + 2 < n_iter) {
+        fetch_k_next();
+        fetch_v_next();
+      }
+    }
     __syncthreads();
   }
 
