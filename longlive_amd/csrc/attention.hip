@@ -500,19 +500,172 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   for (; it < n_fast; ++it) {
     const uint8_t* cur = smem + (it & 1) * kStageBytes;
     uint8_t* nxt = smem + ((it + 1) & 1) * kStageBytes;
-    const uint8_t* kt_base = cur + kp * kKTileBytes;
     const uint8_t* vt_base = cur + 2 * kKTileBytes + kp * kVTileBytes;
     const bool has_next2 = it + 2 < n_iter;
-    s_half(kt_base, 0, Tag1{}, nxt + k_dst_off);
+
+    // ---- S phase: S^T (64 keys x 64 queries) = 32 MFMAs, eight steps of four.  Each step also converts
+    //      one dword of the prefetched K row and half a "piece" (2 of the 16 elements x 4 keys) of the
+    //      prefetched V data into the other LDS stage: 32 conversion instructions per four MFMAs.
+    float16v sc[2][2];
+    {
+      const float gsk = tab.kg[k_slot];
+      float sfv[4];
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk)
+        sfv[kk] = fp8_byte_to_f32(vf[kk].scale, 0) * tab.vg[v_slot + (v_off + kk >= p.bts ? 1 : 0)];
+      const uint32_t w[8] = {kf.v0.x, kf.v0.y, kf.v0.z, kf.v0.w, kf.v1.x, kf.v1.y, kf.v1.z, kf.v1.w};
+      uint8_t* kdst = nxt + k_dst_off;
+      uint8_t* vdst = nxt + v_dst_off;
+      const uint8_t* krow0 = cur + kp * kKTileBytes + l32 * kKPitch + lh * 16;
+      const uint8_t* krow1 = krow0 + 32 * kKPitch;
+#pragma unroll
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) sc[kt][qt][i] = 0.0f;
+      uint4 a0 = *reinterpret_cast<const uint4*>(krow0), a1 = *reinterpret_cast<const uint4*>(krow1);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        uint4 n0 = a0, n1 = a1;
+        if (ks < 7) {
+          n0 = *reinterpret_cast<const uint4*>(krow0 + (ks + 1) * 32);
+          n1 = *reinterpret_cast<const uint4*>(krow1 + (ks + 1) * 32);
+        }
+        const bf16x8 fa0 = __builtin_bit_cast(bf16x8, a0), fa1 = __builtin_bit_cast(bf16x8, a1);
+        sc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, qf[0][ks], sc[0][0], 0, 0, 0);
+        sc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, qf[1][ks], sc[0][1], 0, 0, 0);
+        sc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, qf[0][ks], sc[1][0], 0, 0, 0);
+        sc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, qf[1][ks], sc[1][1], 0, 0, 0);
+        {  // K: dword ks of the row
+          const float sf = fp8_byte_to_f32(kf.scales, ks >> 1) * gsk;
+          float v8[8];
+          fp4x8_to_f32(w[ks], sf, v8);
+          reinterpret_cast<uint4*>(kdst)[ks] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
+                                                           pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
+        }
+        {  // V: elements 2 ks, 2 ks + 1 of the thread's 16, for its 4 keys -> two rows of V^T
+          float e[4][2];
+#pragma unroll
+          for (int kk = 0; kk < 4; ++kk) {
+            const uint32_t word = (ks & 4) ? vf[kk].v.y : vf[kk].v.x;
+            float2v q;
+            switch (ks & 3) {
+              case 0: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0); break;
+              case 1: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1); break;
+              case 2: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2); break;
+              default: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3); break;
+            }
+            e[kk][0] = q[0] * sfv[kk];
+            e[kk][1] = q[1] * sfv[kk];
+          }
+#pragma unroll
+          for (int j = 0; j < 2; ++j)
+            *reinterpret_cast<uint2*>(vdst + (2 * ks + j) * kVPitch) =
+                make_uint2(pack_bf16(e[0][j], e[1][j]), pack_bf16(e[2][j], e[3][j]));
+        }
+        a0 = n0;
+        a1 = n1;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);  // eight conversion instructions under it
+        }
+      }
+    }
     advance_k();
-    if (has_next2) fetch_k_next();
-    softmax_max();
-    pv_half(vt_base, 0);
-    s_half(kt_base, 1, Tag2{}, nxt + v_dst_off);
     advance_v();
-    if (has_next2) fetch_v_next();
-    softmax_max();
-    pv_half(vt_base, 1);
+    if (has_next2) {
+      fetch_k_next();
+      fetch_v_next();
+    }
+
+    // ---- reference point of the exponentials over the 64 keys (see softmax_max)
+    float neg2[2];
+    {
+      float alpha[2];
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) {
+        float mx = sc[0][qt][0];
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[kt][qt][r]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const bool raise = (mx - m_run[qt]) * p.scale_log2 > kRescaleStep;
+        const float m_new = raise ? mx : m_run[qt];
+        alpha[qt] = raise ? __builtin_amdgcn_exp2f((m_run[qt] - m_new) * p.scale_log2) : 1.0f;
+        neg2[qt] = -m_new * p.scale_log2;
+        m_run[qt] = m_new;
+      }
+      if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f) != 0) {
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+          l_run[qt] *= alpha[qt];
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[dt][qt][i] *= alpha[qt];
+        }
+      }
+    }
+
+    // ---- PV phase: four steps of 16 keys.  The exponentials of step j + 1 are computed under the eight
+    //      MFMAs of step j.
+    {
+      float sum[2] = {0.0f, 0.0f};
+      auto make_p = [&](int step, bf16x8 (&dst)[2]) __attribute__((always_inline)) {
+        const int kt = step >> 1, hf = step & 1;
+#pragma unroll
+        for (int qt = 0; qt < 2; ++qt) {
+          uint32_t w[4];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[kt][qt][8 * hf + 2 * i], p.scale_log2, neg2[qt]));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[kt][qt][8 * hf + 2 * i + 1], p.scale_log2, neg2[qt]));
+            sum[qt] += p0 + p1;
+            w[i] = pack_bf16(p0, p1);
+          }
+          dst[qt] = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+        }
+      };
+      auto read_v = [&](int step, uint2 (&dst)[4][2]) __attribute__((always_inline)) {
+        const int chunk0 = (step >> 1) * 8 + (step & 1) * 4 + lh;  // 8-byte chunk holding keys 4*chunk0 .. +3
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+          const uint8_t* src = vt_base + (dt * 32 + l32) * kVPitch;
+          dst[dt][0] = *reinterpret_cast<const uint2*>(src + chunk0 * 8);
+          dst[dt][1] = *reinterpret_cast<const uint2*>(src + (chunk0 + 2) * 8);
+        }
+      };
+      bf16x8 pb[2][2];
+      uint2 vfr[2][4][2];
+      read_v(0, vfr[0]);
+      make_p(0, pb[0]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int step = 0; step < 4; ++step) {
+        if (step < 3) read_v(step + 1, vfr[(step + 1) & 1]);
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) {
+          const uint2(&v)[2] = vfr[step & 1][dt];
+          const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(v[0].x, v[0].y, v[1].x, v[1].y));
+#pragma unroll
+          for (int qt = 0; qt < 2; ++qt) o[dt][qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[step & 1][qt], o[dt][qt], 0, 0, 0);
+        }
+        if (step < 3) {
+          make_p(step + 1, pb[(step + 1) & 1]);
+#pragma unroll
+          for (int g = 0; g < 8; ++g) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+            __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);  // two exponentials
+            __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);  // their multiply-adds, sums and packing
+          }
+        }
+      }
+#pragma unroll
+      for (int qt = 0; qt < 2; ++qt) l_run[qt] += sum[qt];
+    }
     __syncthreads();
   }
   for (; it < n_iter; ++it) {
