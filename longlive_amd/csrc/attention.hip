@@ -111,19 +111,18 @@ __device__ __forceinline__ uint2 load_global_b64(const void* ptr) {
   return make_uint2(v[0], v[1]);
 }
 
-// (slot, off) = key / block_token_size and key % block_token_size, tracked incrementally by the caller.
-__device__ __forceinline__ void fetch_k(const SlotTable& tab, int H, int slot, int off, int head, int half, KRaw& f) {
-  const int64_t row = (int64_t)off * H + head;
-  const uint8_t* src = tab.kv[slot] + row * 64 + half * 32;
+// Raw FP4 loads.  vo / so are byte offsets of the thread's data inside the slot's value / scale arrays;
+// the caller keeps them up to date incrementally (both advance by a constant per iteration inside a slot).
+__device__ __forceinline__ void fetch_k(const SlotTable& tab, int slot, uint32_t vo, uint32_t so, KRaw& f) {
+  const uint8_t* src = tab.kv[slot] + vo;
   f.v0 = load_global_b128(src);
   f.v1 = load_global_b128(src + 16);
-  f.scales = load_global<uint32_t>(tab.ks[slot] + blocked_scale_offset(row, half * 4, 8));
+  f.scales = load_global<uint32_t>(tab.ks[slot] + so);
 }
 
-__device__ __forceinline__ void fetch_v(const SlotTable& tab, int H, int slot, int off, int head, int blk, VRaw& f) {
-  const int64_t row = (int64_t)off * H + head;
-  f.v = load_global_b64(tab.vv[slot] + row * 64 + blk * 8);
-  f.scale = load_global<uint8_t>(tab.vs[slot] + blocked_scale_offset(row, blk, 8));
+__device__ __forceinline__ void fetch_v(const SlotTable& tab, int slot, uint32_t vo, uint32_t so, VRaw& f) {
+  f.v = load_global_b64(tab.vv[slot] + vo);
+  f.scale = load_global<uint8_t>(tab.vs[slot] + so);
 }
 
 // Decode K (64 elements of one key) to bf16 and store the 128 bytes into the key's LDS row.
@@ -279,40 +278,73 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   const int v_blk = (lane >> 4) + 4 * (wave & 1), v_chunk = lane & 15, v_tile = wave >> 1;
   // key, slot and offset in the slot of this thread's K key and of its first V key for the iteration whose
   // raw data is in kf / vf
-  int k_key = tid >> 1, v_key = v_tile * kTileKeys + 4 * v_chunk;
-  int k_slot = k_key / p.bts, k_off = k_key - k_slot * p.bts;
-  int v_slot = v_key / p.bts, v_off = v_key - v_slot * p.bts;
-  const int k_dst_off = ((tid >> 1) >> 6) * kKTileBytes + ((tid >> 1) & 63) * kKPitch + (tid & 1) * 128;
+  // Position of the data the raw registers hold (or will hold next): iter_base = first key of that
+  // iteration; per thread the K key iter_base + k_local and the four V keys iter_base + v_local + 0..3,
+  // each as (slot, offset in slot) plus the byte offsets of its packed values and scale(s) in the slot.
+  const int k_local = tid >> 1, v_local = v_tile * kTileKeys + 4 * v_chunk;
+  const uint32_t row_bytes = (uint32_t)p.H * 64u;          // packed bytes between consecutive tokens
+  const uint32_t step_vo = (uint32_t)kIterKeys * row_bytes;  // advance of a value offset per iteration
+  const uint32_t step_so = (uint32_t)p.H * 1024u;            // advance of a scale offset (rows += 128 H)
+  const uint32_t slot_bytes = (uint32_t)p.bts * row_bytes;
+  const int k_dst_off = (k_local >> 6) * kKTileBytes + (k_local & 63) * kKPitch + (tid & 1) * 128;
   const int v_dst_off = 2 * kKTileBytes + v_tile * kVTileBytes + (v_blk * 16) * kVPitch + v_chunk * 8;
-
+  int iter_base = 0;
+  int k_slot = k_local / p.bts, k_off = k_local - k_slot * p.bts;
+  int v_slot = v_local / p.bts, v_off = v_local - v_slot * p.bts;
+  uint32_t k_vo, k_so, v_vo, v_so[4];
+  auto locate_k = [&]() __attribute__((always_inline)) {
+    const int64_t row = (int64_t)k_off * p.H + head;
+    k_vo = (uint32_t)row * 64u + (tid & 1) * 32u;
+    k_so = (uint32_t)blocked_scale_offset(row, (tid & 1) * 4, 8);
+  };
+  auto locate_v = [&]() __attribute__((always_inline)) {
+    v_vo = ((uint32_t)v_off * p.H + head) * 64u + v_blk * 8u;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      int o = v_off + kk;
+      if (o >= p.bts) o -= p.bts;  // the key sits in the next slot
+      v_so[kk] = (uint32_t)blocked_scale_offset((int64_t)o * p.H + head, v_blk, 8);
+    }
+  };
+  locate_k();
+  locate_v();
   auto fetch_k_next = [&]() __attribute__((always_inline)) {
-    if (k_key < n_cached) fetch_k(tab, p.H, k_slot, k_off, head, tid & 1, kf);
+    if (iter_base + k_local < n_cached) fetch_k(tab, k_slot, k_vo, k_so, kf);
   };
   auto fetch_v_next = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
       const bool wrap = v_off + kk >= p.bts;
-      if (v_key + kk < n_cached)
-        fetch_v(tab, p.H, v_slot + (wrap ? 1 : 0), v_off + kk - (wrap ? p.bts : 0), head, v_blk, vf[kk]);
+      if (iter_base + v_local + kk < n_cached)
+        fetch_v(tab, v_slot + (wrap ? 1 : 0), v_vo + kk * row_bytes - (wrap ? slot_bytes : 0u), v_so[kk], vf[kk]);
     }
   };
-  auto advance_k = [&]() __attribute__((always_inline)) {
-    k_key += kIterKeys;
+  auto advance = [&]() __attribute__((always_inline)) {
+    iter_base += kIterKeys;
     k_off += kIterKeys;
-    while (k_off >= p.bts) {
-      k_off -= p.bts;
-      ++k_slot;
+    k_vo += step_vo;
+    k_so += step_so;
+    if (k_off >= p.bts) {
+      do {
+        k_off -= p.bts;
+        ++k_slot;
+      } while (k_off >= p.bts);
+      locate_k();
     }
-  };
-  auto advance_v = [&]() __attribute__((always_inline)) {
-    v_key += kIterKeys;
     v_off += kIterKeys;
-    while (v_off >= p.bts) {
-      v_off -= p.bts;
-      ++v_slot;
+    v_vo += step_vo;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) v_so[kk] += step_so;
+    if (v_off + 3 >= p.bts) {  // a slot boundary at or inside the thread's four keys
+      while (v_off >= p.bts) {
+        v_off -= p.bts;
+        ++v_slot;
+      }
+      locate_v();
     }
   };
   auto decode_k_any = [&](int stage) __attribute__((always_inline)) {
+    const int k_key = iter_base + k_local;
     const int kind = k_key < n_cached ? 0 : (k_key < Lk_i ? 1 : 2);
     const float gs = kind == 0 ? tab.kg[k_slot] : 0.0f;
     const uint4* src = reinterpret_cast<const uint4*>(
@@ -325,7 +357,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     const uint4* src[4];
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      const int key = v_key + kk;
+      const int key = iter_base + v_local + kk;
       kind[kk] = key < n_cached ? 0 : (key < Lk_i ? 1 : 2);
       gs[kk] = kind[kk] == 0 ? tab.vg[v_slot + (v_off + kk >= p.bts ? 1 : 0)] : 0.0f;
       src[kk] = reinterpret_cast<const uint4*>(p.v_new + ((int64_t)(key - n_cached) * p.H + head) * kHeadDim + v_blk * 16);
@@ -479,8 +511,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   fetch_v_next();
   decode_k_any(0);
   decode_v_any(0);
-  advance_k();
-  advance_v();
+  advance();
   if (n_iter > 1) {
     fetch_k_next();
     fetch_v_next();
@@ -573,8 +604,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
         }
       }
     }
-    advance_k();
-    advance_v();
+    advance();
     if (has_next2) {
       fetch_k_next();
       fetch_v_next();
@@ -695,8 +725,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     if (it + 1 < n_iter) {
       decode_k_any((it + 1) & 1);
       decode_v_any((it + 1) & 1);
-      advance_k();
-      advance_v();
+      advance();
       if (it + 2 < n_iter) {
         fetch_k_next();
         fetch_v_next();
@@ -792,7 +821,8 @@ extern "C" int ll_kv_attention(const void* q, int64_t Lq, int num_heads, const u
   if (n_cached > 0) {
     LL_REQUIRE(k_values_ptrs && k_scales_ptrs && k_amax_ptrs && v_values_ptrs && v_scales_ptrs && v_amax_ptrs,
                "ll_kv_attention: n_cached > 0 needs the six slot pointer tables");
-    LL_REQUIRE(block_token_size > 0 && e2m1_max > 0.f && e4m3_max > 0.f, "ll_kv_attention: bad slot geometry");
+    LL_REQUIRE(block_token_size >= 4 && e2m1_max > 0.f && e4m3_max > 0.f, "ll_kv_attention: bad slot geometry");
+    LL_REQUIRE((int64_t)block_token_size * num_heads * 64 < (1ll << 31), "ll_kv_attention: slot too large");
     LL_REQUIRE(((int64_t)block_token_size * num_heads) % 128 == 0,
                "ll_kv_attention: slot rows (block_token_size*num_heads = %lld) must be a multiple of 128",
                (long long)block_token_size * num_heads);

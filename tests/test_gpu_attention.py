@@ -82,7 +82,7 @@ def test_attention_properties(gpu):
     assert torch.equal(out, v1.expand(130, 2, 128))
 
 
-@pytest.mark.parametrize("H,T,n_chunks,sink_blocks,max_blocks", [(2, 64, 6, 1, 4), (3, 128, 4, 1, 3), (2, 192, 3, 0, 2)])
+@pytest.mark.parametrize("H,T,n_chunks,sink_blocks,max_blocks", [(2, 64, 6, 1, 4), (3, 128, 4, 1, 3), (2, 192, 3, 0, 2), (4, 352, 7, 1, 5)])
 def test_cache_streaming_against_oracle(gpu, H, T, n_chunks, sink_blocks, max_blocks):
     """Streams chunks through fill and roll phases; each chunk runs two forwards (the second one
     re-inserts into the same slot, like the clean-context pass).  The oracle keeps a list of
