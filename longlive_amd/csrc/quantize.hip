@@ -282,7 +282,8 @@ template <int RULE>
 __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
                                                             int64_t ldx, int64_t Kp, uint8_t* __restrict__ values,
                                                             uint8_t* __restrict__ scales, float* __restrict__ amax_io,
-                                                            const float* __restrict__ parts, int amax_given) {
+                                                            const float* __restrict__ parts, int amax_given,
+                                                            int64_t total_tiles) {
   __shared__ float s_red[kThreads / 64];
   __shared__ float s_amax;
   __shared__ uint32_t s_scales[128];  // 512 bytes in blocked order
@@ -299,7 +300,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
       float r = s_red[0];
       for (int i = 1; i < kThreads / 64; ++i) r = fmaxf(r, s_red[i]);
       s_amax = r;
-      if (blockIdx.x == 0 && blockIdx.y == 0) amax_io[0] = r;
+      if (blockIdx.x == 0) amax_io[0] = r;
     }
   }
   __syncthreads();
@@ -325,11 +326,16 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
   }
   __syncthreads();
 
-  const int64_t row0 = (int64_t)blockIdx.y * 128;
-  const int64_t col0 = (int64_t)blockIdx.x * 64;
   const bool vec = ((ldx & 7) == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
   uint8_t* s_bytes = reinterpret_cast<uint8_t*>(s_scales);
+  const int64_t tiles_x = Kp >> 6;
 
+  // Tiles are dealt to the resident workgroups round-robin, so the prologue above (amax reduction,
+  // scale table) is paid once per workgroup and not once per tile.
+#pragma unroll 1
+  for (int64_t tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
+  const int64_t row0 = (tile / tiles_x) * 128;
+  const int64_t col0 = (tile % tiles_x) * 64;
 #pragma unroll 1
   for (int it = 0; it < 2; ++it) {
     const int b = threadIdx.x + it * kThreads;  // block within the tile
@@ -356,9 +362,8 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
     s_bytes[(r & 31) * 16 + (r >> 5) * 4 + cb] = (uint8_t)sb;
   }
   __syncthreads();
-  if (threadIdx.x < 128) {
-    const int64_t tile = (int64_t)blockIdx.y * (Kp >> 6) + blockIdx.x;
-    reinterpret_cast<uint32_t*>(scales)[tile * 128 + threadIdx.x] = s_scales[threadIdx.x];
+  if (threadIdx.x < 128) reinterpret_cast<uint32_t*>(scales)[tile * 128 + threadIdx.x] = s_scales[threadIdx.x];
+  __syncthreads();  // the staged scale tile is rewritten by the next tile
   }
 }
 
@@ -389,17 +394,20 @@ extern "C" int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ld
   LL_REQUIRE((reinterpret_cast<uintptr_t>(values) & 7) == 0 && (reinterpret_cast<uintptr_t>(scales) & 3) == 0,
              "ll_nvfp4_quantize: outputs must be 8-byte (values) / 4-byte (scales) aligned");
   const int64_t Mp = round_up(M, 128), Kp = round_up(K, 64);
-  LL_REQUIRE(Kp / 64 <= 0x7FFFFFFF && Mp / 128 <= 65535, "ll_nvfp4_quantize: tensor too large for one launch");
+  const int64_t total_tiles = (Kp / 64) * (Mp / 128);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const uint16_t* xp = static_cast<const uint16_t*>(x);
   if (!amax_given) {
     hipLaunchKernelGGL(amax_partial_kernel, dim3(kAmaxParts), dim3(kThreads), 0, s, xp, M, K, ldx, workspace);
     LL_CHECK_LAUNCH("amax_partial_kernel");
   }
-  const dim3 grid((unsigned)(Kp / 64), (unsigned)(Mp / 128));
+  // one workgroup per tile up to what the chip holds at once (256 CUs x 8 for the static rules,
+  // x 4 for the rules that evaluate two candidates and need twice the registers)
+  const int64_t resident = (rule == LL_RULE_STATIC_6 || rule == LL_RULE_STATIC_4) ? 2048 : 1024;
+  const dim3 grid((unsigned)(total_tiles < resident ? total_tiles : resident));
 #define LL_LAUNCH_Q(R)                                                                                          \
   hipLaunchKernelGGL(quantize_kernel<R>, grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales, amax, \
-                     workspace, amax_given)
+                     workspace, amax_given, total_tiles)
   switch (rule) {
     case LL_RULE_STATIC_6: LL_LAUNCH_Q(LL_RULE_STATIC_6); break;
     case LL_RULE_STATIC_4: LL_LAUNCH_Q(LL_RULE_STATIC_4); break;

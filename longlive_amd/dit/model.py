@@ -17,6 +17,7 @@ import torch
 import torch.nn as nn
 
 from .. import _native
+from ..fouroversix.model.modules.linear import FourOverSixLinear
 from ..utils import kv_cache as kvc
 from ..utils.adaln import adaln_modulate
 from ..utils.rope import build_rope_angles, rope_apply, rope_cos_sin
@@ -62,6 +63,17 @@ class WanLayerNorm(nn.LayerNorm):
         return super().forward(x).type_as(x)
 
 
+def _project_shared(x: torch.Tensor, layers) -> list[torch.Tensor]:
+    """Apply several linear layers to the same input.  Quantized layers with the same activation config
+    share one quantized operand (bit-identical to quantizing per layer, as the reference does)."""
+    first = layers[0]
+    if all(isinstance(m, FourOverSixLinear) for m in layers) and all(
+            m.config.get_activation_config() == first.config.get_activation_config() for m in layers):
+        xq = first.quantize_input(x.reshape(-1, x.shape[-1]))
+        return [m.forward_quantized(xq).reshape(*x.shape[:-1], -1) for m in layers]
+    return [m(x) for m in layers]
+
+
 class CausalSelfAttention(nn.Module):
     def __init__(self, dim: int, num_heads: int, eps: float = 1e-6) -> None:
         super().__init__()
@@ -72,9 +84,10 @@ class CausalSelfAttention(nn.Module):
     def forward(self, x, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size):
         b, s = x.shape[:2]
         n, d = self.num_heads, self.head_dim
-        q = self.norm_q(self.q(x)).view(b, s, n, d)
-        k = self.norm_k(self.k(x)).view(b, s, n, d)
-        v = self.v(x).view(b, s, n, d)
+        q, k, v = _project_shared(x, [self.q, self.k, self.v])
+        q = self.norm_q(q).view(b, s, n, d)
+        k = self.norm_k(k).view(b, s, n, d)
+        v = v.view(b, s, n, d)
         roped_q = rope_apply(q[0], cos, sin).unsqueeze(0)
         roped_k = rope_apply(k[0], cos, sin).unsqueeze(0)
         out, update = kvc.kv_cache_attention(roped_q, roped_k, v, kv_cache, current_start, sink_tokens,
@@ -93,8 +106,9 @@ class CrossAttention(nn.Module):
         b, n, d = x.shape[0], self.num_heads, self.head_dim
         q = self.norm_q(self.q(x)).view(b, -1, n, d)
         # K / V of the text context are recomputed on every call, as the reference does (:229-235)
-        k = self.norm_k(self.k(context)).view(b, -1, n, d)
-        v = self.v(context).view(b, -1, n, d)
+        k, v = _project_shared(context, [self.k, self.v])
+        k = self.norm_k(k).view(b, -1, n, d)
+        v = v.view(b, -1, n, d)
         out = _native.attention_bf16(q[0].contiguous(), k[0].contiguous(), v[0].contiguous(), d ** -0.5)
         return self.o(out.unsqueeze(0).flatten(2))
 

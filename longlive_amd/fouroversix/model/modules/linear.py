@@ -98,9 +98,18 @@ class FourOverSixLinear(nn.Linear):
         return out.reshape(*input.shape[:-1], out.shape[-1])
 
     def _forward_2d(self, x2d: torch.Tensor) -> torch.Tensor:
+        return self.forward_quantized(self.quantize_input(x2d))
+
+    def quantize_input(self, x2d: torch.Tensor) -> QuantizedTensor:
+        """The activation operand exactly as ``forward`` would build it from a 2-D input."""
+        return quantize_to_fp4(x2d, self.config.get_activation_config())
+
+    def forward_quantized(self, xq: QuantizedTensor) -> torch.Tensor:
+        """``forward`` for an input already quantized with :meth:`quantize_input`.  Several layers that read
+        the same tensor with the same activation config (the q / k / v projections) share one quantized
+        operand this way; each would otherwise compute the identical bytes again.  Returns [M, out_features]."""
         weight = self.quantized_weight()
         if not isinstance(weight, QuantizedTensor):
             weight = quantize_to_fp4(weight.data, self.config.get_weight_config())
-        xq = quantize_to_fp4(x2d, self.config.get_activation_config())
         return fp4_matmul(xq, weight, backend=self.config.matmul_backend, out_dtype=self.config.output_dtype,
                           bias=self.bias)
