@@ -250,3 +250,53 @@ def test_streaming_generator_small_end_to_end(gpu):
     # the first chunk only depends on itself: generating just that chunk gives the same latents
     gen3 = StreamingGenerator(cfg, gpu, seed=4)
     assert torch.equal(gen3.generate(noise[:, :2], ctx), out[:, :2])
+
+
+def test_packed_nvfp4_checkpoint_round_trip(gpu, tmp_path):
+    """Export a quantized generator as a packed NVFP4 checkpoint, load it into a fresh bf16 model
+    (utils/inference_utils.py:186-218 order: swap linears, drop master weights, strict load) and check
+    that buffers and outputs are identical; a bf16 checkpoint of the same weights gives the same model."""
+    from types import SimpleNamespace
+
+    from longlive_amd.dit import CausalDiT
+    from longlive_amd.utils import nvfp4_checkpoint as ck
+
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    run_cfg = SimpleNamespace(model_quant_scale_rule="mse")
+    gen = StreamingGenerator(cfg, gpu, seed=7)  # quantized (mse) and materialized
+    path = tmp_path / "model_4o6.pt"
+    saved = ck.save_nvfp4_checkpoint(path, gen.model, scale_rule="mse", model_name="tiny")
+    assert saved["checkpoint_format"] == "longlive_generator_nvfp4" and saved["checkpoint_version"] == 1
+    assert ck.is_nvfp4_state_dict(saved["generator"])
+    assert not any(k.endswith("self_attn.q.weight") for k in saved["generator"])
+    assert any(k.endswith("self_attn.q.quantized_weight_values") for k in saved["generator"])
+
+    def fresh():
+        torch.manual_seed(123)  # different init: everything must come from the checkpoint
+        with torch.device(gpu):
+            m = CausalDiT(cfg)
+        m.rope_angles = m.rope_angles.cpu()
+        return m
+
+    loaded = ck.load_nvfp4_generator(fresh(), str(path), run_cfg).eval()
+    a, b = gen.model.state_dict(), loaded.state_dict()
+    assert a.keys() == b.keys()
+    for k in a:
+        assert torch.equal(a[k].cpu().view(torch.uint8) if a[k].dtype == torch.float8_e4m3fn else a[k].cpu(),
+                           b[k].cpu().view(torch.uint8) if b[k].dtype == torch.float8_e4m3fn else b[k].cpu()), k
+
+    g = torch.Generator().manual_seed(5)
+    noise = torch.randn(1, 4, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    ref = gen.generate(noise, ctx)
+    gen2 = StreamingGenerator(cfg, gpu, seed=99)
+    gen2.model = loaded
+    gen2.model.kv_quant_config = gen2.kv_quant_config
+    assert torch.equal(gen2.generate(noise, ctx), ref)
+
+    # TransformerEngine checkpoints and unknown versions are refused
+    with pytest.raises(ValueError):
+        ck.load_nvfp4_generator(fresh(), {"checkpoint_format": ck.TE_NVFP4_CHECKPOINT_FORMAT, "generator": {}})
+    with pytest.raises(ValueError):
+        ck.load_nvfp4_generator(fresh(), {**saved, "checkpoint_version": 2})

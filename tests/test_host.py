@@ -152,3 +152,22 @@ def test_cache_policy_fill_then_roll_matches_reference_numbers():
     assert info["action"] == "direct_insert" and slots == (0, 1, 2, 3) and info["local_start_index"] == 10560
     with pytest.raises(NotImplementedError):
         kvc.plan_cache_step(_fake_cache(blk, 5), 0, blk // 2, blk)
+
+
+def test_nvfp4_checkpoint_helpers_on_plain_dictionaries():
+    from types import SimpleNamespace
+
+    from longlive_amd.utils import nvfp4_checkpoint as ck
+
+    assert ck.is_nvfp4_state_dict({"blocks.0.ffn.0.quantized_weight_values": 1})
+    assert not ck.is_nvfp4_state_dict({"blocks.0.ffn.0.weight": 1}) and not ck.is_nvfp4_state_dict(3)
+    ckpt = {"generator": {"a": 1}, "generator_ema": {"a": 2}}
+    assert ck.unwrap_generator_state_dict(ckpt) == {"a": 1}
+    assert ck.unwrap_generator_state_dict(ckpt, use_ema=True) == {"a": 2}
+    assert ck.unwrap_generator_state_dict({"model": {"b": 1}}) == {"b": 1}
+    assert ck.unwrap_generator_state_dict({"c": 1}) == {"c": 1}
+    assert ck.clean_fsdp_state_dict_keys({"m._fsdp_wrapped_module.w": 0}) == {"m.w": 0}
+    assert ck.is_te_nvfp4_checkpoint({"checkpoint_format": "longlive_generator_te_nvfp4"})
+    cfg = ck.build_model_quantization_config(SimpleNamespace(model_quant_scale_rule="mse"))
+    assert cfg.scale_rule.value == "mse" and cfg.activation_scale_rule.value == "mse" and not cfg.keep_master_weights
+    assert ck.build_model_quantization_config(None).scale_rule.value == "static_6"
