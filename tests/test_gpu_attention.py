@@ -184,3 +184,35 @@ def test_rms_norm_against_oracle(gpu):
     ref = o.rms_norm(x.float().numpy(), w.float().numpy())
     diff = np.abs(got - ref)
     assert diff.max() <= 2 ** -5 and (diff != 0).mean() < 5e-3
+
+
+def test_config3_full_size_fused_decode_equals_attention_over_the_dequantized_cache(gpu):
+    """Benchmark shape (24 heads, 2640 queries, 4 FP4 slots of 2640 tokens + the bf16 chunk = 13200 keys):
+    the kernel that decodes FP4 on load must agree with plain bf16 attention over the cache dequantized by
+    ll_kv_dequantize_blocks (a different kernel path), and with the oracle on a sample of queries.  Also a
+    row-sum property at full size: with V = const the output is that constant."""
+    H, T = 24, 2640
+    g = torch.Generator().manual_seed(2)
+    cache = kvc.initialize_kv_cache(1, T, 5, H, 128, CFG, gpu)[0]
+    for c in range(4):
+        q, k, v = (torch.randn(1, T, H, 128, generator=g).bfloat16().to(gpu) for _ in range(3))
+        _, (ce, le, info) = kvc.kv_cache_attention(q, k, v, cache, c * T, sink_tokens=T)
+        kvc.apply_cache_update(cache, ce, le, info, CFG)
+    q, k, v = (torch.randn(1, T, H, 128, generator=g).bfloat16().to(gpu) for _ in range(3))
+    out, _ = kvc.kv_cache_attention(q, k, v, cache, 4 * T, sink_tokens=T)
+    kd = dequantize_kv_cache(cache["k"], 4, H, T, torch.bfloat16, gpu)[0]
+    vd = dequantize_kv_cache(cache["v"], 4, H, T, torch.bfloat16, gpu)[0]
+    from longlive_amd.utils.quant import k_smooth
+    k_all = torch.cat([kd, k_smooth(k)[0]]).contiguous()
+    v_all = torch.cat([vd, v[0]]).contiguous()
+    assert k_all.shape == (5 * T, H, 128)
+    ref = _native.attention_bf16(q[0].contiguous(), k_all, v_all, 128 ** -0.5)
+    assert (out[0].float() - ref.float()).abs().max().item() <= 4e-3  # same bf16 operands, other summation order
+    # oracle (fp64 softmax) on the first 16 queries of three heads
+    for h in (0, 11, 23):
+        want = o.attention(q[0, :16, h:h + 1].float().cpu().numpy(), k_all[:, h:h + 1].float().cpu().numpy(),
+                           v_all[:, h:h + 1].float().cpu().numpy())
+        assert np.abs(out[0, :16, h:h + 1].float().cpu().numpy() - want).max() <= 2e-2
+    # rows of the softmax sum to one at full size
+    out_c = _native.attention_bf16(q[0].contiguous(), k_all, torch.full_like(v_all, 0.75), 128 ** -0.5)
+    assert (out_c.float() - 0.75).abs().max().item() <= 2 ** -7
