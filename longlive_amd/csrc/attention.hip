@@ -11,8 +11,6 @@
 // S^T = K Q^T and O^T = V^T P^T (v_mfma_f32_32x32x16_bf16), so every lane owns one query column:
 // row max / row sum need no cross-lane traffic beyond one swap between the wave halves, and the
 // online-softmax rescale is a per-lane scalar.
-#include <type_traits>
-
 #include "ll_common.h"
 
 namespace ll {
@@ -365,27 +363,15 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     store_v4(vf, kind, gs, src, smem + stage * kStageBytes + 2 * kKTileBytes + v_tile * kVTileBytes, v_blk * 16, v_chunk);
   };
 
-  // One iteration handles the wave's 64-key tile as two 32-key halves: S half -> running max -> P, PV half.
-  // S^T of one half (32 keys x 64 queries).  kDecode = 1: convert the prefetched FP4 K row (8 dwords, one
-  // per MFMA step) between the MFMAs; kDecode = 2: convert the prefetched FP4 V data (4 keys x 16 elements,
-  // one quarter every second step); 0: nothing.
+  // Plain loop: the wave's 64-key tile is handled as two 32-key halves: S half -> running max -> P, PV half.
+  // S^T of one half (32 keys x 64 queries).
   float16v s[2];
-  auto s_half = [&](const uint8_t* kt_base, int kt, auto decode_tag, uint8_t* dst) __attribute__((always_inline)) {
-    constexpr int kDecode = decltype(decode_tag)::value;
-    float gs = 0.0f, sfv[4] = {0.f, 0.f, 0.f, 0.f};
-    if constexpr (kDecode == 1) gs = tab.kg[k_slot];
-    if constexpr (kDecode == 2) {
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk)
-        sfv[kk] = fp8_byte_to_f32(vf[kk].scale, 0) * tab.vg[v_slot + (v_off + kk >= p.bts ? 1 : 0)];
-    }
-    const uint32_t w[8] = {kf.v0.x, kf.v0.y, kf.v0.z, kf.v0.w, kf.v1.x, kf.v1.y, kf.v1.z, kf.v1.w};
+  auto s_half = [&](const uint8_t* kt_base, int kt) __attribute__((always_inline)) {
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt)
 #pragma unroll
       for (int i = 0; i < 16; ++i) s[qt][i] = 0.0f;
-    // K fragments are read two steps ahead of their MFMAs, and in program order before the LDS stores of
-    // the interleaved conversion (the compiler cannot prove those stores go to the other stage).
+    // K fragments are read two steps ahead of their MFMAs
     const uint8_t* krow = kt_base + (kt * 32 + l32) * kKPitch + lh * 16;
     uint4 afrag[8];
     afrag[0] = *reinterpret_cast<const uint4*>(krow);
@@ -397,36 +383,6 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       const bf16x8 a = __builtin_bit_cast(bf16x8, afrag[ks]);
 #pragma unroll
       for (int qt = 0; qt < 2; ++qt) s[qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[qt][ks], s[qt], 0, 0, 0);
-      if constexpr (kDecode == 1) {
-        const float sf = fp8_byte_to_f32(kf.scales, ks >> 1) * gs;
-        float v8[8];
-        fp4x8_to_f32(w[ks], sf, v8);
-        reinterpret_cast<uint4*>(dst)[ks] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
-                                                        pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
-      }
-      if constexpr (kDecode == 2) {
-        if (ks & 1) {
-          // piece: elements 4 * piece .. + 3 of the thread's 16, for its 4 keys
-          const int piece = ks >> 1;
-          float e[4][4];
-#pragma unroll
-          for (int kk = 0; kk < 4; ++kk) {
-            const uint32_t word = (piece & 2) ? vf[kk].v.y : vf[kk].v.x;
-            const float2v lo = (piece & 1) ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2)
-                                           : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0);
-            const float2v hi = (piece & 1) ? __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3)
-                                           : __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1);
-            e[kk][0] = lo[0] * sfv[kk];
-            e[kk][1] = lo[1] * sfv[kk];
-            e[kk][2] = hi[0] * sfv[kk];
-            e[kk][3] = hi[1] * sfv[kk];
-          }
-#pragma unroll
-          for (int j = 0; j < 4; ++j)
-            *reinterpret_cast<uint2*>(dst + (4 * piece + j) * kVPitch) =
-                make_uint2(pack_bf16(e[0][j], e[1][j]), pack_bf16(e[2][j], e[3][j]));
-        }
-      }
     }
   };
 
@@ -502,10 +458,6 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) l_run[qt] += sum[qt];
   };
-  using Tag0 = std::integral_constant<int, 0>;
-  using Tag1 = std::integral_constant<int, 1>;
-  using Tag2 = std::integral_constant<int, 2>;
-
   // prologue: stage 0 <- iteration 0, raw registers <- iteration 1
   fetch_k_next();
   fetch_v_next();
@@ -707,7 +659,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     for (int kt = 0; kt < 2; ++kt) {
       const int half_base = tile_base + kt * 32;
       if (half_base < Lk_i) {
-        s_half(kt_base, kt, Tag0{}, nullptr);
+        s_half(kt_base, kt);
         if (half_base + 32 > Lk_i) {  // mask keys beyond the end (only in the last tile)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
