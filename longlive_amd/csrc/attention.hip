@@ -792,7 +792,8 @@ extern "C" int ll_kv_attention(const void* q, int64_t Lq, int num_heads, const u
   p.vv_ptrs = v_values_ptrs; p.vs_ptrs = v_scales_ptrs; p.va_ptrs = v_amax_ptrs;
   p.n_cached = n_cached;
   p.n_new = n_new;
-  p.bts = block_token_size > 0 ? block_token_size : 1;
+  // without cached tokens the slot size only feeds the (unused) position bookkeeping: make it never wrap
+  p.bts = n_cached > 0 ? block_token_size : (1 << 30);
   p.n_slots = n_slots;
   p.inv_denom = n_cached > 0 ? 1.0f / (e2m1_max * e4m3_max) : 0.f;
   p.k_new = static_cast<const uint16_t*>(k_new);
