@@ -34,6 +34,7 @@ enum {
 };
 
 enum { LL_RULE_STATIC_6 = 0, LL_RULE_STATIC_4 = 1, LL_RULE_MAE = 2, LL_RULE_MSE = 3, LL_RULE_ABS_MAX = 4 };
+enum { LL_ACT_NONE = 0, LL_ACT_GELU_TANH = 1 };
 enum { LL_DTYPE_BF16 = 0, LL_DTYPE_F16 = 1, LL_DTYPE_F32 = 2 }; /* utils/kernel/kv_dequant.py:18-25 */
 
 const char* ll_last_error(void);
@@ -78,6 +79,16 @@ int ll_nvfp4_gemm_tnt(const uint8_t* A_values, const uint8_t* A_scales, const ui
                       const uint8_t* B_scales, const float* alpha, const float* amax_a, const float* amax_b,
                       float denom_a, float denom_b, int64_t M, int64_t N, int64_t Mp, int64_t Np, int64_t Kp,
                       void* D, int64_t ldd, const void* bias, void* stream);
+
+/*
+ * ll_nvfp4_gemm_tnt with an activation applied to the bf16 result (after the bias) in the epilogue, for the
+ * Linear -> GELU(tanh) pair of the DiT feed-forward (wan_5b/modules/causal_model.py:822-824):
+ *   D = bf16(act(f32(bf16(bf16(alpha * acc) + bias))));  activation: LL_ACT_NONE or LL_ACT_GELU_TANH.
+ */
+int ll_nvfp4_gemm_tnt_act(const uint8_t* A_values, const uint8_t* A_scales, const uint8_t* B_values,
+                          const uint8_t* B_scales, const float* alpha, const float* amax_a, const float* amax_b,
+                          float denom_a, float denom_b, int64_t M, int64_t N, int64_t Mp, int64_t Np, int64_t Kp,
+                          void* D, int64_t ldd, const void* bias, int activation, void* stream);
 
 /*
  * Replaces torch.ops.longlive_kernels.dequantize_kv_cache_fp4 (utils/kernel/kv_dequant.cpp:14,

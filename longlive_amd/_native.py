@@ -19,6 +19,7 @@ HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "ll_nvfp4.h")
 
 RULE_IDS = {"static_6": 0, "static_4": 1, "mae": 2, "mse": 3, "abs_max": 4}
 DTYPE_CODES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+ACTIVATION_IDS = {"gelu_tanh": 1}
 
 _lib = None
 
@@ -33,6 +34,9 @@ _SIGNATURES = {
     "ll_nvfp4_gemm_tnt": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                   c_float, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p,
                                   c_void_p]),
+    "ll_nvfp4_gemm_tnt_act": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                      c_float, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64,
+                                      c_void_p, c_int, c_void_p]),
     "ll_kv_dequantize_blocks": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float,
                                         c_void_p, c_void_p]),
     "ll_kv_attention": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -162,7 +166,9 @@ def dequantize(values, scales, amax, rule: str, padded, original, dtype: torch.d
 
 # --------------------------------------------------------------------------- GEMM
 def gemm(a_values, a_scales, b_values, b_scales, M: int, N: int, *, alpha=None, amax_a=None, amax_b=None,
-         denom_a: float = 1536.0, denom_b: float = 1536.0, bias=None, out=None) -> torch.Tensor:
+         denom_a: float = 1536.0, denom_b: float = 1536.0, bias=None, out=None, activation=None) -> torch.Tensor:
+    if activation is not None and activation not in ACTIVATION_IDS:
+        raise ValueError(f"unknown epilogue activation {activation!r}")
     _require_cuda(a_values, a_scales, b_values, b_scales, alpha, amax_a, amax_b, bias)
     Mp, Kb = a_values.shape
     Np, Kb2 = b_values.shape
@@ -173,9 +179,13 @@ def gemm(a_values, a_scales, b_values, b_scales, M: int, N: int, *, alpha=None, 
     if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N or not bias.is_contiguous()):
         raise ValueError("bias must be a contiguous bfloat16 vector of length N")
     with torch.cuda.device(a_values.device):
-        code = load().ll_nvfp4_gemm_tnt(a_values.data_ptr(), a_scales.data_ptr(), b_values.data_ptr(),
-                                        b_scales.data_ptr(), _ptr(alpha), _ptr(amax_a), _ptr(amax_b), denom_a, denom_b,
-                                        M, N, Mp, Np, Kb * 2, out.data_ptr(), out.stride(0), _ptr(bias), _stream())
+        args = (a_values.data_ptr(), a_scales.data_ptr(), b_values.data_ptr(), b_scales.data_ptr(), _ptr(alpha),
+                _ptr(amax_a), _ptr(amax_b), denom_a, denom_b, M, N, Mp, Np, Kb * 2, out.data_ptr(), out.stride(0),
+                _ptr(bias))
+        if activation is None:
+            code = load().ll_nvfp4_gemm_tnt(*args, _stream())
+        else:
+            code = load().ll_nvfp4_gemm_tnt_act(*args, ACTIVATION_IDS[activation], _stream())
     _check(code, "ll_nvfp4_gemm_tnt")
     return out
 

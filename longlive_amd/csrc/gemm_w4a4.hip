@@ -54,12 +54,18 @@ struct GemmSmem {
   static constexpr int kStage = kAVals + kBVals + kAScales + kBScales;
 };
 
+// 0.5 x (1 + tanh(u)) = x / (1 + exp(-2u)),  u = sqrt(2/pi) (x + 0.044715 x^3)  (nn.GELU(approximate="tanh"))
+__device__ __forceinline__ float gelu_tanh_f32(float x) {
+  const float u2 = x * (1.5957691216057308f + 0.07135481627260025f * (x * x));  // 2u
+  return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * u2));
+}
+
 template <int FA, int FB>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
     const uint8_t* __restrict__ Av, const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bv,
     const uint8_t* __restrict__ Bs, const float* __restrict__ alpha_ptr, const float* __restrict__ amax_a,
     const float* __restrict__ amax_b, float inv_denom_a, float inv_denom_b, int M, int N, int Mp, int Np, int Kp,
-    uint16_t* __restrict__ D, int64_t ldd, const uint16_t* __restrict__ bias, int tiles_m, int tiles_n) {
+    uint16_t* __restrict__ D, int64_t ldd, const uint16_t* __restrict__ bias, int tiles_m, int tiles_n, int act) {
   using S = GemmSmem<FA, FB>;
   constexpr int BM = S::BM, BN = S::BN;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -297,6 +303,14 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
             w[i] = lo | (hi << 16);
           }
         }
+        if (act == LL_ACT_GELU_TANH) {  // GELU (tanh form) of the bf16 value, computed in fp32, rounded to bf16
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const uint32_t lo = f32_to_bf16_bits(gelu_tanh_f32(__uint_as_float(w[i] << 16)));
+            const uint32_t hi = f32_to_bf16_bits(gelu_tanh_f32(__uint_as_float(w[i] & 0xFFFF0000u)));
+            w[i] = lo | (hi << 16);
+          }
+        }
         uint16_t* dst = D + (int64_t)m * ldd + n_lane;
         if (vec_ok && n_lane + 8 <= N) {
           *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
@@ -312,7 +326,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
 template <int FA, int FB>
 int launch_gemm(const uint8_t* Av, const uint8_t* As, const uint8_t* Bv, const uint8_t* Bs, const float* alpha,
                 const float* amax_a, const float* amax_b, float denom_a, float denom_b, int M, int N, int Mp, int Np,
-                int Kp, void* D, int64_t ldd, const void* bias, hipStream_t stream) {
+                int Kp, void* D, int64_t ldd, const void* bias, int act, hipStream_t stream) {
   using S = GemmSmem<FA, FB>;
   const int tiles_m = (M + S::BM - 1) / S::BM, tiles_n = (N + S::BN - 1) / S::BN;
   const size_t smem = 2 * S::kStage;
@@ -328,7 +342,7 @@ int launch_gemm(const uint8_t* Av, const uint8_t* As, const uint8_t* Bv, const u
   }
   hipLaunchKernelGGL((gemm_w4a4_kernel<FA, FB>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kGemmThreads), smem, stream,
                      Av, As, Bv, Bs, alpha, amax_a, amax_b, 1.0f / denom_a, 1.0f / denom_b, M, N, Mp, Np, Kp,
-                     static_cast<uint16_t*>(D), ldd, static_cast<const uint16_t*>(bias), tiles_m, tiles_n);
+                     static_cast<uint16_t*>(D), ldd, static_cast<const uint16_t*>(bias), tiles_m, tiles_n, act);
   LL_CHECK_LAUNCH("gemm_w4a4_kernel");
   return LL_OK;
 }
@@ -339,7 +353,18 @@ extern "C" int ll_nvfp4_gemm_tnt(const uint8_t* A_values, const uint8_t* A_scale
                                  const uint8_t* B_scales, const float* alpha, const float* amax_a,
                                  const float* amax_b, float denom_a, float denom_b, int64_t M, int64_t N, int64_t Mp,
                                  int64_t Np, int64_t Kp, void* D, int64_t ldd, const void* bias, void* stream) {
+  return ll_nvfp4_gemm_tnt_act(A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, M, N,
+                               Mp, Np, Kp, D, ldd, bias, LL_ACT_NONE, stream);
+}
+
+extern "C" int ll_nvfp4_gemm_tnt_act(const uint8_t* A_values, const uint8_t* A_scales, const uint8_t* B_values,
+                                     const uint8_t* B_scales, const float* alpha, const float* amax_a,
+                                     const float* amax_b, float denom_a, float denom_b, int64_t M, int64_t N,
+                                     int64_t Mp, int64_t Np, int64_t Kp, void* D, int64_t ldd, const void* bias,
+                                     int activation, void* stream) {
   using namespace ll;
+  LL_REQUIRE(activation == LL_ACT_NONE || activation == LL_ACT_GELU_TANH, "ll_nvfp4_gemm_tnt: unknown activation %d",
+             activation);
   LL_REQUIRE(A_values && A_scales && B_values && B_scales && D, "ll_nvfp4_gemm_tnt: null pointer");
   LL_REQUIRE(alpha || (amax_a && amax_b && denom_a > 0.f && denom_b > 0.f),
              "ll_nvfp4_gemm_tnt: pass alpha, or both amax pointers with positive denominators");
@@ -378,7 +403,7 @@ extern "C" int ll_nvfp4_gemm_tnt(const uint8_t* A_values, const uint8_t* A_scale
     if (f >= 0 && f < 3) best = f;
   }
 #define LL_GEMM_ARGS A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, (int)M, (int)N, \
-                     (int)Mp, (int)Np, (int)Kp, D, ldd, bias, s
+                     (int)Mp, (int)Np, (int)Kp, D, ldd, bias, activation, s
   switch (best) {
     case 0: return launch_gemm<4, 2>(LL_GEMM_ARGS);
     case 1: return launch_gemm<2, 4>(LL_GEMM_ARGS);

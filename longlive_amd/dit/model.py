@@ -125,6 +125,14 @@ class DiTBlock(nn.Module):
         self.ffn = nn.Sequential(nn.Linear(dim, ffn_dim), nn.GELU(approximate="tanh"), nn.Linear(ffn_dim, dim))
         self.modulation = nn.Parameter(torch.randn(1, 6, dim) / dim ** 0.5)
 
+    def _feed_forward(self, y: torch.Tensor) -> torch.Tensor:
+        """Linear -> GELU(tanh) -> Linear; with a quantized first layer the GELU runs in its GEMM epilogue."""
+        up, act, down = self.ffn
+        if isinstance(up, FourOverSixLinear) and getattr(act, "approximate", None) == "tanh":
+            h = up.forward_quantized(up.quantize_input(y.reshape(-1, y.shape[-1])), activation="gelu_tanh")
+            return down(h.reshape(*y.shape[:-1], -1))
+        return self.ffn(y)
+
     def forward(self, x, e, cos, sin, context, kv_cache, current_start, sink_tokens, max_attention_size=None):
         """x [1, L, C]; e [1, F, 6, C]; returns (x, (current_end, local_end_index, cache_update_info))."""
         num_frames, frame_seqlen = e.shape[1], x.shape[1] // e.shape[1]
@@ -133,7 +141,7 @@ class DiTBlock(nn.Module):
         y, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size)
         x = x + (y.unflatten(1, (num_frames, frame_seqlen)) * e[2]).flatten(1, 2)
         x = x + self.cross_attn(self.norm3(x), context)
-        y = self.ffn(adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps))
+        y = self._feed_forward(adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps))
         x = x + (y.unflatten(1, (num_frames, frame_seqlen)) * e[5]).flatten(1, 2)
         return x, update
 

@@ -17,12 +17,14 @@ def fp4_matmul(
     other_config: QuantizationConfig | None = None,
     out_dtype: DataType = DataType.bfloat16,
     bias: torch.Tensor | None = None,
+    activation: str | None = None,
 ) -> torch.Tensor:
     """``input @ other.T`` of two NVFP4 tensors with fp32 accumulation (W4A4 GEMM).
 
     High-precision operands are quantized first with ``input_config`` / ``other_config``.
     ``backend`` is accepted for compatibility; the gfx950 kernel always runs.  ``bias`` (bfloat16
-    [N], an extension) is added to the bfloat16 result inside the kernel epilogue.
+    [N], an extension) is added to the bfloat16 result inside the kernel epilogue; ``activation``
+    (``"gelu_tanh"``, an extension) is then applied to that bfloat16 value, also in the epilogue.
     """
     if isinstance(backend, str):
         backend = MatmulBackend(backend)
@@ -47,4 +49,5 @@ def fp4_matmul(
         denom_a=float(input.scale_rule.max_allowed_e2m1_value() * input.scale_rule.max_allowed_e4m3_value()),
         denom_b=float(other.scale_rule.max_allowed_e2m1_value() * other.scale_rule.max_allowed_e4m3_value()),
         bias=bias,
+        activation=activation,
     )

@@ -104,12 +104,13 @@ class FourOverSixLinear(nn.Linear):
         """The activation operand exactly as ``forward`` would build it from a 2-D input."""
         return quantize_to_fp4(x2d, self.config.get_activation_config())
 
-    def forward_quantized(self, xq: QuantizedTensor) -> torch.Tensor:
+    def forward_quantized(self, xq: QuantizedTensor, activation: str | None = None) -> torch.Tensor:
         """``forward`` for an input already quantized with :meth:`quantize_input`.  Several layers that read
         the same tensor with the same activation config (the q / k / v projections) share one quantized
-        operand this way; each would otherwise compute the identical bytes again.  Returns [M, out_features]."""
+        operand this way; each would otherwise compute the identical bytes again.  ``activation`` ("gelu_tanh")
+        is applied to the bfloat16 result in the GEMM epilogue.  Returns [M, out_features]."""
         weight = self.quantized_weight()
         if not isinstance(weight, QuantizedTensor):
             weight = quantize_to_fp4(weight.data, self.config.get_weight_config())
         return fp4_matmul(xq, weight, backend=self.config.matmul_backend, out_dtype=self.config.output_dtype,
-                          bias=self.bias)
+                          bias=self.bias, activation=activation)

@@ -141,3 +141,30 @@ def test_linear_module_with_bias_matches_reference_semantics(gpu):
     fresh.load_state_dict(model.state_dict(), strict=True)
     with torch.no_grad():
         assert torch.equal(fresh[0](x), y)
+
+
+def test_gelu_epilogue_matches_separate_gelu(gpu):
+    """The GEMM with the GELU(tanh) epilogue against the plain GEMM followed by torch's GELU on the bf16
+    result: the same function evaluated as x / (1 + exp(-2u)) instead of 0.5 x (1 + tanh(u)), so results may
+    differ by one bf16 ulp on a small fraction of the elements."""
+    from longlive_amd.fouroversix import QuantizationConfig, fp4_matmul, quantize_to_fp4
+    cfg = QuantizationConfig(scale_rule="mse")
+    x = activations((300, 512), 31).to(gpu)
+    w = (weights((640, 512), 32) * 40).to(gpu)  # outputs spread over roughly [-8, 8]
+    bias = (torch.randn(640, generator=torch.Generator().manual_seed(33)) * 0.5).bfloat16().to(gpu)
+    xq, wq = quantize_to_fp4(x, cfg), quantize_to_fp4(w, cfg)
+    plain = fp4_matmul(xq, wq, bias=bias)
+    fused = fp4_matmul(xq, wq, bias=bias, activation="gelu_tanh")
+    want = torch.nn.functional.gelu(plain, approximate="tanh")
+    assert plain.float().abs().max() > 4
+    # one bf16 ulp where the result is not tiny; far in the negative tail 1 + tanh cancels in torch's formula
+    # and the two evaluations differ relatively (not absolutely): results there are below 1e-5
+    f, w_ = fused.float(), want.float()
+    assert bool(((f - w_).abs() <= torch.maximum(w_.abs() * 2 ** -7, torch.tensor(2e-6, device=gpu))).all())
+    body = plain.float().abs() < 3
+    assert float((f[body] != w_[body]).float().mean()) < 0.02
+    # the oracle's formula in float64
+    ref = o.gelu_tanh(plain.float().cpu().numpy().astype(np.float64))
+    assert np.abs(fused.float().cpu().numpy() - ref).max() <= 2 ** -8 * max(1.0, np.abs(ref).max())
+    with pytest.raises(ValueError):
+        fp4_matmul(xq, wq, activation="relu")
