@@ -140,6 +140,14 @@ int ll_adaln_modulate(const void* x, int64_t B, int64_t L, int C, const void* sc
                       int64_t scale_stride_b, int64_t scale_stride_f, int64_t shift_stride_b, int64_t shift_stride_f,
                       int64_t frame_seqlen, float eps, int add_one_to_scale, void* out, void* stream);
 
+/*
+ * Gated residual of the DiT block (wan_5b/modules/causal_model.py:889, 919-920):
+ *   out = bf16(x + bf16(y * gate[b, l / frame_seqlen, :]));  x, y, out bf16 [B, L, C] contiguous, gate bf16 with
+ *   the given strides (elements).  out may alias x.
+ */
+int ll_gate_residual(const void* x, const void* y, int64_t B, int64_t L, int C, const void* gate,
+                     int64_t gate_stride_b, int64_t gate_stride_f, int64_t frame_seqlen, void* out, void* stream);
+
 /* WanRMSNorm (wan_5b/modules/model.py:82-98): y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) over the
  * last dim C of x bf16 [rows, C]; w bf16 [C]. */
 int ll_rms_norm(const void* x, int64_t rows, int C, const void* weight, float eps, void* out, void* stream);

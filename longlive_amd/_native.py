@@ -47,6 +47,8 @@ _SIGNATURES = {
                               c_void_p, c_void_p]),
     "ll_adaln_modulate": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p, c_void_p]),
+    "ll_gate_residual": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_int64, c_int64,
+                                 c_void_p, c_void_p]),
     "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
     "ll_debug_convert": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
 }
@@ -263,6 +265,24 @@ def adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps=1e-6, add_one_to_scale
                                         e_scale.stride(0), e_scale.stride(1), e_shift.stride(0), e_shift.stride(1),
                                         frame_seqlen, float(eps), int(add_one_to_scale), out.data_ptr(), _stream())
     _check(code, "ll_adaln_modulate")
+    return out
+
+
+def gate_residual(x, y, gate, frame_seqlen):
+    """x + y * gate, x / y bf16 [B, L, C] contiguous, gate bf16 [B, F, 1, C] (per frame)."""
+    _require_cuda(x, y, gate)
+    if x.ndim != 3 or x.dtype != torch.bfloat16 or y.dtype != torch.bfloat16 or x.shape != y.shape \
+            or not (x.is_contiguous() and y.is_contiguous()):
+        raise ValueError("x and y must be contiguous bfloat16 [B, L, C] tensors of the same shape")
+    B, L, C = x.shape
+    F = L // frame_seqlen
+    if gate.shape != (B, F, 1, C) or gate.dtype != torch.bfloat16 or gate.stride(3) != 1:
+        raise ValueError(f"gate must be bfloat16 [B, F, 1, C] = {(B, F, 1, C)}, got {tuple(gate.shape)}")
+    out = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        code = load().ll_gate_residual(x.data_ptr(), y.data_ptr(), B, L, C, gate.data_ptr(), gate.stride(0),
+                                       gate.stride(1), frame_seqlen, out.data_ptr(), _stream())
+    _check(code, "ll_gate_residual")
     return out
 
 

@@ -167,6 +167,32 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(const uint16_t* __
   }
 }
 
+
+// ----------------------------------------------------------------------------- gated residual
+// x + y * gate of the DiT block (wan_5b/modules/causal_model.py:889, 919-920): the product is rounded to
+// bf16, then the sum, as the two separate bf16 operations of the reference do.  gate is indexed
+// [b, l / frame_seqlen, :].  One thread = 8 consecutive channels.
+__global__ __launch_bounds__(256) void gate_residual_kernel(const uint16_t* __restrict__ x,
+                                                           const uint16_t* __restrict__ y,
+                                                           const uint16_t* __restrict__ gate, int64_t L, int C,
+                                                           int64_t g_sb, int64_t g_sf, int64_t frame_seqlen,
+                                                           int64_t total_chunks, uint16_t* __restrict__ out) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= total_chunks) return;
+  const int cpr = C >> 3;  // chunks per row
+  const int64_t row = idx / cpr;
+  const int c = (int)(idx - row * cpr);
+  const int64_t b = row / L, l = row - b * L, f = l / frame_seqlen;
+  float xv[8], yv[8], gv[8];
+  unpack8(*reinterpret_cast<const uint4*>(x + row * (int64_t)C + c * 8), xv);
+  unpack8(*reinterpret_cast<const uint4*>(y + row * (int64_t)C + c * 8), yv);
+  unpack8(*reinterpret_cast<const uint4*>(gate + b * g_sb + f * g_sf + c * 8), gv);
+  float r[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) r[j] = xv[j] + round_to_bf16(yv[j] * gv[j]);
+  *reinterpret_cast<uint4*>(out + row * (int64_t)C + c * 8) = pack8(r);
+}
+
 }  // namespace ll
 
 extern "C" int ll_rope_apply(const void* x, int64_t S, int N, int D, int64_t x_stride_s, int64_t x_stride_n,
@@ -224,5 +250,26 @@ extern "C" int ll_rms_norm(const void* x, int64_t rows, int C, const void* weigh
                      static_cast<const uint16_t*>(x), C, static_cast<const uint16_t*>(weight), eps,
                      static_cast<uint16_t*>(out));
   LL_CHECK_LAUNCH("rmsnorm_kernel");
+  return LL_OK;
+}
+
+extern "C" int ll_gate_residual(const void* x, const void* y, int64_t B, int64_t L, int C, const void* gate,
+                                int64_t gate_stride_b, int64_t gate_stride_f, int64_t frame_seqlen, void* out,
+                                void* stream) {
+  using namespace ll;
+  LL_REQUIRE(x && y && gate && out, "ll_gate_residual: null pointer");
+  LL_REQUIRE(B > 0 && L > 0 && C > 0 && C % 8 == 0 && frame_seqlen > 0, "ll_gate_residual: bad shape B=%lld L=%lld C=%d",
+             (long long)B, (long long)L, C);
+  LL_REQUIRE(gate_stride_b % 8 == 0 && gate_stride_f % 8 == 0 &&
+                 ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) | reinterpret_cast<uintptr_t>(gate) |
+                   reinterpret_cast<uintptr_t>(out)) & 15) == 0,
+             "ll_gate_residual: pointers must be 16-byte aligned and strides multiples of 8 elements");
+  const int64_t chunks = B * L * (C >> 3);
+  LL_REQUIRE((chunks + 255) / 256 <= 0x7FFFFFFF, "ll_gate_residual: tensor too large");
+  hipLaunchKernelGGL(gate_residual_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x),
+                     static_cast<const uint16_t*>(y), static_cast<const uint16_t*>(gate), L, C, gate_stride_b,
+                     gate_stride_f, frame_seqlen, chunks, static_cast<uint16_t*>(out));
+  LL_CHECK_LAUNCH("gate_residual_kernel");
   return LL_OK;
 }

@@ -19,7 +19,7 @@ import torch.nn as nn
 from .. import _native
 from ..fouroversix.model.modules.linear import FourOverSixLinear
 from ..utils import kv_cache as kvc
-from ..utils.adaln import adaln_modulate
+from ..utils.adaln import adaln_modulate, gate_residual
 from ..utils.rope import build_rope_angles, rope_apply, rope_cos_sin
 
 
@@ -139,10 +139,10 @@ class DiTBlock(nn.Module):
         e = (self.modulation.unsqueeze(1) + e).chunk(6, dim=2)
         y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.eps)
         y, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size)
-        x = x + (y.unflatten(1, (num_frames, frame_seqlen)) * e[2]).flatten(1, 2)
+        x = gate_residual(x, y.contiguous(), e[2], frame_seqlen)
         x = x + self.cross_attn(self.norm3(x), context)
         y = self._feed_forward(adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps))
-        x = x + (y.unflatten(1, (num_frames, frame_seqlen)) * e[5]).flatten(1, 2)
+        x = gate_residual(x, y.contiguous(), e[5], frame_seqlen)
         return x, update
 
 

@@ -14,3 +14,10 @@ def adaln_modulate(x: torch.Tensor, e_scale: torch.Tensor, e_shift: torch.Tensor
 
 
 adaln_modulate_triton = adaln_modulate
+
+
+def gate_residual(x: torch.Tensor, y: torch.Tensor, gate: torch.Tensor, frame_seqlen: int) -> torch.Tensor:
+    """``x + (y.unflatten(1, (F, frame_seqlen)) * gate).flatten(1, 2)`` of the DiT block
+    (wan_5b/modules/causal_model.py:889, 919-920) in one pass; product and sum are each rounded to bf16
+    like the two eager operations."""
+    return _native.gate_residual(x, y, gate, frame_seqlen)

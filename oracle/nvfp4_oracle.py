@@ -396,6 +396,14 @@ def adaln_modulate(x, scale, shift, frame_seqlen, eps=1e-6):
     return round_bf16(prod + shift[fidx].astype(F32))
 
 
+def gate_residual(x, y, gate, frame_seqlen):
+    """wan_5b/modules/causal_model.py:889, 919-920: x + y * gate with the product and the sum each rounded
+    to bf16.  x, y [L,C] and gate [F,C] hold bf16 values."""
+    fidx = np.arange(x.shape[0]) // frame_seqlen
+    prod = round_bf16(y.astype(F32) * gate[fidx].astype(F32))
+    return round_bf16(x.astype(F32) + prod)
+
+
 def rms_norm(x, weight, eps=1e-6):
     """wan_5b/modules/model.py:82-98: fp32 x*rsqrt(mean(x^2)+eps) -> bf16, times bf16 weight -> bf16."""
     x = x.astype(F32)

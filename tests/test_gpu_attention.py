@@ -216,3 +216,18 @@ def test_config3_full_size_fused_decode_equals_attention_over_the_dequantized_ca
     # rows of the softmax sum to one at full size
     out_c = _native.attention_bf16(q[0].contiguous(), k_all, torch.full_like(v_all, 0.75), 128 ** -0.5)
     assert (out_c.float() - 0.75).abs().max().item() <= 2 ** -7
+
+
+def test_gate_residual_bit_exact_against_oracle_and_eager(gpu):
+    from longlive_amd.utils.adaln import gate_residual
+    L, C, fs = 48, 3072, 16
+    x, y = _randn((1, L, C), 41), _randn((1, L, C), 42, 3.0)
+    e = _randn((1, L // fs, 6, C), 43)          # modulation tensor; the gate is a strided view of it
+    gate = e.chunk(6, dim=2)[2]
+    got = gate_residual(x.to(gpu), y.to(gpu), e.to(gpu).chunk(6, dim=2)[2], fs)
+    want = o.gate_residual(x[0].float().numpy(), y[0].float().numpy(), gate[0, :, 0].float().numpy(), fs)
+    assert np.array_equal(got[0].float().cpu().numpy(), want)
+    eager = x + (y.unflatten(1, (L // fs, fs)) * gate).flatten(1, 2)
+    assert torch.equal(got.cpu(), eager)
+    with pytest.raises(ValueError):
+        gate_residual(x.to(gpu), y.to(gpu)[:, :, :8], e.to(gpu).chunk(6, dim=2)[2], fs)

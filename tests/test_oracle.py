@@ -287,3 +287,13 @@ def test_rms_norm_matches_torch():
     ref = ((xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16() * w).float().numpy()
     diff = np.abs(got - ref)
     assert diff.max() <= 2 ** -6 and (diff != 0).mean() < 0.01
+
+
+def test_gate_residual_equals_two_bf16_operations():
+    import torch
+    g = torch.Generator().manual_seed(9)
+    x, y = torch.randn(12, 64, generator=g).bfloat16(), (torch.randn(12, 64, generator=g) * 4).bfloat16()
+    gate = torch.randn(3, 64, generator=g).bfloat16()
+    want = x + y * gate.repeat_interleave(4, dim=0)      # two bf16 eager operations
+    got = o.gate_residual(x.float().numpy(), y.float().numpy(), gate.float().numpy(), 4)
+    assert np.array_equal(got, want.float().numpy())
