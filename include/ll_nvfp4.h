@@ -152,6 +152,16 @@ int ll_gate_residual(const void* x, const void* y, int64_t B, int64_t L, int C, 
  * last dim C of x bf16 [rows, C]; w bf16 [C]. */
 int ll_rms_norm(const void* x, int64_t rows, int C, const void* weight, float eps, void* out, void* stream);
 
+/*
+ * q / k path between the projections and attention in one pass (wan_5b/modules/causal_model.py:362-368,
+ * 477-487; utils/quant.py:797-798): WanRMSNorm over rows of num_heads*128 channels, then the rotary embedding
+ * per head (rows < seq_len; cos/sin f32 [seq_len, 64]), with the roundings of ll_rms_norm followed by
+ * ll_rope_apply.  out bf16 [rows, num_heads, 128]; out_smooth (may be NULL) receives
+ * bf16(out - bf16(mean of out over the 128 channels of the head)), the K handed to attention for the current chunk.
+ */
+int ll_qk_norm_rope(const void* x, int64_t rows, int num_heads, const void* weight, float eps, const float* cos,
+                    const float* sin, int64_t seq_len, void* out, void* out_smooth, void* stream);
+
 /* Test hooks: hardware fp32->e4m3 / fp32->e2m1 conversions applied to n floats (used by the GPU tests to
  * check the instructions the fast paths rely on against the software codecs). mode 0: e4m3, 1: e2m1. */
 int ll_debug_convert(const float* in, int64_t n, int mode, uint8_t* out, void* stream);

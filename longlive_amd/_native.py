@@ -47,6 +47,8 @@ _SIGNATURES = {
                               c_void_p, c_void_p]),
     "ll_adaln_modulate": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p, c_void_p]),
+    "ll_qk_norm_rope": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p, c_int64, c_void_p,
+                                c_void_p, c_void_p]),
     "ll_gate_residual": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_int64, c_int64,
                                  c_void_p, c_void_p]),
     "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
@@ -248,6 +250,29 @@ def rope_apply(x, cos, sin, seq_len=None):
                                     seq_len, out.data_ptr(), _stream())
     _check(code, "ll_rope_apply")
     return out
+
+
+def qk_norm_rope(x, weight, eps, cos, sin, num_heads, seq_len=None, smooth=False):
+    """RMSNorm over rows of x bf16 [S, num_heads*128], RoPE per head -> bf16 [S, num_heads, 128]; with
+    ``smooth`` also returns that tensor minus its per-head mean over the 128 channels."""
+    _require_cuda(x, weight, cos, sin)
+    if x.ndim != 2 or x.dtype != torch.bfloat16 or not x.is_contiguous() or x.shape[1] != num_heads * 128:
+        raise ValueError("x must be a contiguous bfloat16 [S, num_heads * 128] tensor")
+    if weight.dtype != torch.bfloat16 or weight.numel() != x.shape[1]:
+        raise ValueError("weight must be bfloat16 with one entry per channel")
+    S = x.shape[0]
+    seq_len = S if seq_len is None else seq_len
+    if cos.shape != (seq_len, 64) or sin.shape != cos.shape or cos.dtype != torch.float32:
+        raise ValueError(f"cos/sin must be float32 [{seq_len}, 64]")
+    cos = cos.contiguous()
+    sin = sin.contiguous()
+    out = torch.empty((S, num_heads, 128), dtype=x.dtype, device=x.device)
+    out_s = torch.empty_like(out) if smooth else None
+    with torch.cuda.device(x.device):
+        code = load().ll_qk_norm_rope(x.data_ptr(), S, num_heads, weight.contiguous().data_ptr(), float(eps),
+                                      cos.data_ptr(), sin.data_ptr(), seq_len, out.data_ptr(), _ptr(out_s), _stream())
+    _check(code, "ll_qk_norm_rope")
+    return (out, out_s) if smooth else out
 
 
 def adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps=1e-6, add_one_to_scale=True):

@@ -168,6 +168,76 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(const uint16_t* __
 }
 
 
+// ----------------------------------------------------------------------------- RMSNorm + RoPE (+ K smoothing)
+// q / k path after the projections (wan_5b/modules/causal_model.py:362-368, 477-487): WanRMSNorm over the
+// whole row, then the 3-D rotary embedding per head of 128, each with the roundings of the separate kernels
+// above; optionally also k - mean(k over the head dimension) (utils/quant.py:797-798) as a second output,
+// mean and difference rounded to bf16 like the two eager operations.  One workgroup = one token row; a head
+// is held by 16 consecutive threads.
+__global__ __launch_bounds__(kRowThreads) void qk_norm_rope_kernel(const uint16_t* __restrict__ x, int C,
+                                                                   const uint16_t* __restrict__ w, float eps,
+                                                                   const float* __restrict__ cosp,
+                                                                   const float* __restrict__ sinp, int64_t seq_len,
+                                                                   uint16_t* __restrict__ out,
+                                                                   uint16_t* __restrict__ out_smooth) {
+  __shared__ float sm[kRowThreads / 64];
+  const int64_t row = blockIdx.x;
+  const uint16_t* xr = x + row * (int64_t)C;
+  const int nchunks = C >> 3;
+  float v[kMaxChunks][8];
+  float sq = 0.0f;
+#pragma unroll
+  for (int i = 0; i < kMaxChunks; ++i) {
+    const int c = threadIdx.x + i * kRowThreads;
+    if (c < nchunks) {
+      unpack8(*reinterpret_cast<const uint4*>(xr + c * 8), v[i]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sq += v[i][j] * v[i][j];
+    }
+  }
+  const float ms = block_sum<kRowThreads>(sq, sm) / (float)C;
+  const float r = 1.0f / sqrtf(ms + eps);
+  const bool rotate = row < seq_len;
+#pragma unroll
+  for (int i = 0; i < kMaxChunks; ++i) {
+    const int c = threadIdx.x + i * kRowThreads;  // uniform over each group of 16 threads: c < nchunks or not
+    if (c < nchunks) {
+      float w8[8], y[8], o8[8];
+      unpack8(*reinterpret_cast<const uint4*>(w + c * 8), w8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = round_to_bf16(round_to_bf16(v[i][j] * r) * w8[j]);
+      if (rotate) {
+        const int pair0 = (c & 15) * 4;  // first rotation pair of this chunk inside its head
+        const float4 cs = *reinterpret_cast<const float4*>(cosp + row * 64 + pair0);
+        const float4 sn = *reinterpret_cast<const float4*>(sinp + row * 64 + pair0);
+        const float cc[4] = {cs.x, cs.y, cs.z, cs.w}, ss[4] = {sn.x, sn.y, sn.z, sn.w};
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+          const float a = y[2 * p], b = y[2 * p + 1];
+          o8[2 * p] = round_to_bf16(a * cc[p] - b * ss[p]);
+          o8[2 * p + 1] = round_to_bf16(a * ss[p] + b * cc[p]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o8[j] = y[j];
+      }
+      *reinterpret_cast<uint4*>(out + row * (int64_t)C + c * 8) = pack8(o8);
+      if (out_smooth) {
+        float part = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) part += o8[j];
+#pragma unroll
+        for (int m = 1; m < 16; m <<= 1) part += __shfl_xor(part, m, 64);
+        const float mean = round_to_bf16(part * (1.0f / 128.0f));
+        float s8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s8[j] = o8[j] - mean;
+        *reinterpret_cast<uint4*>(out_smooth + row * (int64_t)C + c * 8) = pack8(s8);
+      }
+    }
+  }
+}
+
 // ----------------------------------------------------------------------------- gated residual
 // x + y * gate of the DiT block (wan_5b/modules/causal_model.py:889, 919-920): the product is rounded to
 // bf16, then the sum, as the two separate bf16 operations of the reference do.  gate is indexed
@@ -271,5 +341,25 @@ extern "C" int ll_gate_residual(const void* x, const void* y, int64_t B, int64_t
                      static_cast<const uint16_t*>(y), static_cast<const uint16_t*>(gate), L, C, gate_stride_b,
                      gate_stride_f, frame_seqlen, chunks, static_cast<uint16_t*>(out));
   LL_CHECK_LAUNCH("gate_residual_kernel");
+  return LL_OK;
+}
+
+extern "C" int ll_qk_norm_rope(const void* x, int64_t rows, int num_heads, const void* weight, float eps,
+                               const float* cos, const float* sin, int64_t seq_len, void* out, void* out_smooth,
+                               void* stream) {
+  using namespace ll;
+  LL_REQUIRE(x && weight && cos && sin && out, "ll_qk_norm_rope: null pointer");
+  const int64_t C = (int64_t)num_heads * 128;
+  LL_REQUIRE(rows > 0 && rows <= 0x7FFFFFFF && num_heads > 0 && C <= kRowThreads * kMaxChunks * 8 && seq_len >= 0,
+             "ll_qk_norm_rope: bad shape rows=%lld heads=%d", (long long)rows, num_heads);
+  LL_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out) |
+               reinterpret_cast<uintptr_t>(out_smooth) | reinterpret_cast<uintptr_t>(cos) |
+               reinterpret_cast<uintptr_t>(sin)) & 15) == 0,
+             "ll_qk_norm_rope: pointers must be 16-byte aligned");
+  hipLaunchKernelGGL(qk_norm_rope_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x), (int)C,
+                     static_cast<const uint16_t*>(weight), eps, cos, sin, seq_len, static_cast<uint16_t*>(out),
+                     static_cast<uint16_t*>(out_smooth));
+  LL_CHECK_LAUNCH("qk_norm_rope_kernel");
   return LL_OK;
 }

@@ -85,13 +85,21 @@ class CausalSelfAttention(nn.Module):
         b, s = x.shape[:2]
         n, d = self.num_heads, self.head_dim
         q, k, v = _project_shared(x, [self.q, self.k, self.v])
-        q = self.norm_q(q).view(b, s, n, d)
-        k = self.norm_k(k).view(b, s, n, d)
         v = v.view(b, s, n, d)
-        roped_q = rope_apply(q[0], cos, sin).unsqueeze(0)
-        roped_k = rope_apply(k[0], cos, sin).unsqueeze(0)
+        if b == 1 and d == 128:
+            # RMSNorm -> RoPE (-> K smoothing) of the reference in one pass per tensor
+            roped_q = _native.qk_norm_rope(q[0], self.norm_q.weight.data, self.norm_q.eps, cos, sin, n).unsqueeze(0)
+            roped_k, smooth_k = _native.qk_norm_rope(k[0], self.norm_k.weight.data, self.norm_k.eps, cos, sin, n,
+                                                     smooth=True)
+            roped_k, smooth_k = roped_k.unsqueeze(0), smooth_k.unsqueeze(0)
+        else:
+            q = self.norm_q(q).view(b, s, n, d)
+            k = self.norm_k(k).view(b, s, n, d)
+            roped_q = rope_apply(q[0], cos, sin).unsqueeze(0)
+            roped_k = rope_apply(k[0], cos, sin).unsqueeze(0)
+            smooth_k = None
         out, update = kvc.kv_cache_attention(roped_q, roped_k, v, kv_cache, current_start, sink_tokens,
-                                             max_attention_size=max_attention_size)
+                                             max_attention_size=max_attention_size, smoothed_key=smooth_k)
         return self.o(out.flatten(2)), update
 
 

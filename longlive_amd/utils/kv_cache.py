@@ -104,20 +104,22 @@ def plan_cache_step(cache: dict, current_start: int, num_new_tokens: int, sink_t
 
 def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Tensor, cache: dict,
                        current_start: int, sink_tokens: int, softmax_scale: float | None = None,
-                       max_attention_size: int | None = None):
+                       max_attention_size: int | None = None, smoothed_key: torch.Tensor | None = None):
     """Self-attention of one chunk against the FP4 cache.
 
     q, key_to_cache (RoPE'd, un-smoothed), v: bf16 [1, S, H, 128].  Attends
     [selected FP4 slots | k_smooth(key_to_cache), v] without a mask and returns
     ``(out [1, S, H, 128], (current_end, local_end_index, cache_update_info))`` exactly like the
     reference's attention module, with ``new_k`` / ``new_v`` = the un-smoothed chunk to be written.
+    ``smoothed_key`` = k_smooth(key_to_cache) [1, S, H, 128] when the caller has it already (the fused
+    norm + RoPE kernel produces it as a second output).
     """
     if q.shape[0] != 1:
         raise ValueError("the quantized KV cache holds one sequence (batch size 1)")
     S, H, D = q.shape[1:]
     slot_ids, info, local_end = plan_cache_step(cache, current_start, S, sink_tokens, max_attention_size)
     info["new_k"], info["new_v"] = key_to_cache, v
-    k_new = k_smooth(key_to_cache)[0]
+    k_new = (k_smooth(key_to_cache) if smoothed_key is None else smoothed_key)[0]
     scale = D ** -0.5 if softmax_scale is None else softmax_scale
     rule = cache["k"][0].scale_rule
     if slot_ids:

@@ -231,3 +231,26 @@ def test_gate_residual_bit_exact_against_oracle_and_eager(gpu):
     assert torch.equal(got.cpu(), eager)
     with pytest.raises(ValueError):
         gate_residual(x.to(gpu), y.to(gpu)[:, :, :8], e.to(gpu).chunk(6, dim=2)[2], fs)
+
+
+def test_fused_norm_rope_equals_the_separate_kernels(gpu):
+    """ll_qk_norm_rope against ll_rms_norm followed by ll_rope_apply (bit-exact) and, for the smoothed K,
+    against torch's k - k.mean(-1) on the bf16 tensor (same roundings; the fp32 summation order of the mean
+    may differ, so a value may move by one bf16 ulp in rare cases)."""
+    S, H = 96, 3
+    x = _randn((S, H * 128), 51, 2.0).to(gpu)
+    w = (1 + 0.1 * torch.randn(H * 128, generator=torch.Generator().manual_seed(52))).bfloat16().to(gpu)
+    cos, sin = rope_cos_sin(build_rope_angles(128), 2, 6, 8, 3, gpu)  # 96 rows
+    want = rope_apply(_native.rms_norm(x, w, 1e-6).view(S, H, 128), cos, sin)
+    got = _native.qk_norm_rope(x, w, 1e-6, cos, sin, H)
+    assert torch.equal(got, want)
+    got2, smooth = _native.qk_norm_rope(x, w, 1e-6, cos, sin, H, smooth=True)
+    assert torch.equal(got2, want)
+    eager = want - want.mean(dim=-1, keepdim=True)
+    d = (smooth.float() - eager.float()).abs()
+    assert float(d.max()) <= 2 ** -7 * float(eager.float().abs().max())
+    assert float((d != 0).float().mean()) < 0.01
+    # rows beyond seq_len are normalized but not rotated
+    part = _native.qk_norm_rope(x, w, 1e-6, cos[:64], sin[:64], H, seq_len=64)
+    assert torch.equal(part[:64], want[:64])
+    assert torch.equal(part[64:], _native.rms_norm(x, w, 1e-6).view(S, H, 128)[64:])
