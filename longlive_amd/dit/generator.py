@@ -19,7 +19,7 @@ from .model import CausalDiT, DiTConfig
 
 class StreamingGenerator:
     def __init__(self, cfg: DiTConfig, device, timesteps=(1000.0, 750.0, 500.0, 250.0), seed: int = 0,
-                 model_quant: dict | None = None, kv_scale_rule: str = "mse") -> None:
+                 model_quant: dict | None = None, kv_scale_rule: str = "mse", cache_text_kv: bool = True) -> None:
         self.cfg, self.device = cfg, torch.device(device)
         self.timesteps = [float(t) for t in timesteps]
         torch.manual_seed(seed)
@@ -35,6 +35,7 @@ class StreamingGenerator:
         self.kv_quant_config = LongLiveQuantizationConfig(scale_rule=kv_scale_rule, backend="cuda", type="kv")
         self.model.kv_quant_config = self.kv_quant_config
         self.kv_cache = None
+        self.cache_text_kv = cache_text_kv
 
     def reset_cache(self, frame_seq_length: int) -> None:
         cfg = self.cfg
@@ -54,17 +55,20 @@ class StreamingGenerator:
             self.reset_cache(fs)
         out = torch.empty_like(noise)
         nb = cfg.num_frame_per_block
+        # projected text K / V per layer: one prompt per call, so they are computed by the first forward only
+        xcache = [{"is_init": False} for _ in range(cfg.num_layers)] if self.cache_text_kv else None
         sigmas = [t / 1000.0 for t in self.timesteps] + [0.0]
         for ci, start in enumerate(range(0, F, nb)):
             x = noise[0, start:start + nb].transpose(0, 1).contiguous()  # [C, f, H, W]
             f = x.shape[1]
             for si, t in enumerate(self.timesteps):
                 tt = torch.full((1, f), t, device=self.device, dtype=torch.float32)
-                flow = self.model(x, tt, context, self.kv_cache, start * fs)
+                flow = self.model(x, tt, context, self.kv_cache, start * fs, crossattn_cache=xcache)
                 x = (x.float() + (sigmas[si + 1] - sigmas[si]) * flow.float()).to(noise.dtype)
             out[0, start:start + f] = x.transpose(0, 1)
             # clean-context pass: rewrites this chunk's K / V in the cache
-            self.model(x, torch.zeros((1, f), device=self.device), context, self.kv_cache, start * fs)
+            self.model(x, torch.zeros((1, f), device=self.device), context, self.kv_cache, start * fs,
+                       crossattn_cache=xcache)
             if on_chunk is not None:
                 on_chunk(ci)
         return out

@@ -110,13 +110,21 @@ class CrossAttention(nn.Module):
         self.q, self.k, self.v, self.o = (nn.Linear(dim, dim) for _ in range(4))
         self.norm_q, self.norm_k = WanRMSNorm(dim, eps), WanRMSNorm(dim, eps)
 
-    def forward(self, x, context):
+    def forward(self, x, context, crossattn_cache: dict | None = None):
+        """``crossattn_cache`` ({"is_init": bool, "k": ..., "v": ...}, the reference's interface,
+        wan_5b/modules/causal_model.py:199-206) keeps the projected K / V of a prompt's text context between
+        calls; the reference has the argument but recomputes on every call (:229-235), which gives the same
+        tensors.  Without a cache K / V are recomputed here too."""
         b, n, d = x.shape[0], self.num_heads, self.head_dim
         q = self.norm_q(self.q(x)).view(b, -1, n, d)
-        # K / V of the text context are recomputed on every call, as the reference does (:229-235)
-        k, v = _project_shared(context, [self.k, self.v])
-        k = self.norm_k(k).view(b, -1, n, d)
-        v = v.view(b, -1, n, d)
+        if crossattn_cache is not None and crossattn_cache.get("is_init"):
+            k, v = crossattn_cache["k"], crossattn_cache["v"]
+        else:
+            k, v = _project_shared(context, [self.k, self.v])
+            k = self.norm_k(k).view(b, -1, n, d)
+            v = v.view(b, -1, n, d)
+            if crossattn_cache is not None:
+                crossattn_cache.update(is_init=True, k=k, v=v)
         out = _native.attention_bf16(q[0].contiguous(), k[0].contiguous(), v[0].contiguous(), d ** -0.5)
         return self.o(out.unsqueeze(0).flatten(2))
 
@@ -141,14 +149,15 @@ class DiTBlock(nn.Module):
             return down(h.reshape(*y.shape[:-1], -1))
         return self.ffn(y)
 
-    def forward(self, x, e, cos, sin, context, kv_cache, current_start, sink_tokens, max_attention_size=None):
+    def forward(self, x, e, cos, sin, context, kv_cache, current_start, sink_tokens, max_attention_size=None,
+                crossattn_cache=None):
         """x [1, L, C]; e [1, F, 6, C]; returns (x, (current_end, local_end_index, cache_update_info))."""
         num_frames, frame_seqlen = e.shape[1], x.shape[1] // e.shape[1]
         e = (self.modulation.unsqueeze(1) + e).chunk(6, dim=2)
         y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.eps)
         y, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size)
         x = gate_residual(x, y.contiguous(), e[2], frame_seqlen)
-        x = x + self.cross_attn(self.norm3(x), context)
+        x = x + self.cross_attn(self.norm3(x), context, crossattn_cache)
         y = self._feed_forward(adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps))
         x = gate_residual(x, y.contiguous(), e[5], frame_seqlen)
         return x, update
@@ -223,10 +232,12 @@ class CausalDiT(nn.Module):
 
     @torch.no_grad()
     def forward(self, x: torch.Tensor, t: torch.Tensor, context: torch.Tensor, kv_cache: list[dict],
-                current_start: int, apply_cache_updates: bool = True) -> torch.Tensor:
+                current_start: int, apply_cache_updates: bool = True,
+                crossattn_cache: list[dict] | None = None) -> torch.Tensor:
         """x [C_in, F, H, W] latents of one chunk, t [1, F] timesteps, context [L, text_dim];
         returns the flow prediction [C_out, F, H, W] and updates the KV cache like the reference
-        (all layers' updates applied after the last block)."""
+        (all layers' updates applied after the last block).  ``crossattn_cache``: one dictionary per layer
+        holding the projected text K / V of the current prompt (filled on first use)."""
         cfg = self.cfg
         x = self.patch_embedding(x.unsqueeze(0))
         f, h, w = x.shape[2:]
@@ -242,7 +253,8 @@ class CausalDiT(nn.Module):
         max_attn = cfg.local_attn_size * frame_seqlen
         updates = []
         for i, block in enumerate(self.blocks):
-            x, upd = block(x, e0, cos, sin, ctx, kv_cache[i], current_start, sink_tokens, max_attn)
+            x, upd = block(x, e0, cos, sin, ctx, kv_cache[i], current_start, sink_tokens, max_attn,
+                           None if crossattn_cache is None else crossattn_cache[i])
             updates.append(upd)
         if apply_cache_updates:
             for i, (cur_end, loc_end, info) in enumerate(updates):

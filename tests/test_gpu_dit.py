@@ -300,3 +300,16 @@ def test_packed_nvfp4_checkpoint_round_trip(gpu, tmp_path):
         ck.load_nvfp4_generator(fresh(), {"checkpoint_format": ck.TE_NVFP4_CHECKPOINT_FORMAT, "generator": {}})
     with pytest.raises(ValueError):
         ck.load_nvfp4_generator(fresh(), {**saved, "checkpoint_version": 2})
+
+
+def test_text_kv_cache_gives_identical_latents(gpu):
+    """The per-prompt cache of the projected text K / V (crossattn_cache of the reference's interface) must not
+    change a single bit of the output."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    g = torch.Generator().manual_seed(8)
+    noise = torch.randn(1, 6, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    a = StreamingGenerator(cfg, gpu, seed=4, cache_text_kv=True).generate(noise, ctx)
+    b = StreamingGenerator(cfg, gpu, seed=4, cache_text_kv=False).generate(noise, ctx)
+    assert torch.equal(a, b)
