@@ -161,7 +161,7 @@ def run_e2e(torch, dev):
     return {"latent_frames_per_s": 30.0 / dt, "seconds_30_frames": dt, "steady_chunk_ms": 1e3 * min(per[5:]),
             "steady_latent_frames_per_s": 3.0 / min(per[5:]), "finite": bool(torch.isfinite(out.float()).all().item()),
             "workload": "configs[4]: 30-block NVFP4 generator, 10 chunks x (4 denoising + 1 recache) forwards, FP4 KV cache "
-                        "sink 3 + window 12 frames, text K/V projected once per prompt; first chunk includes one-time warm-up"}
+                        "sink 3 + window 12 frames, text K/V projected once per prompt, cache written by the recache forward only (the denoising forwards' writes are dead stores); first chunk includes one-time warm-up"}
 
 
 def main() -> None:

@@ -19,7 +19,8 @@ from .model import CausalDiT, DiTConfig
 
 class StreamingGenerator:
     def __init__(self, cfg: DiTConfig, device, timesteps=(1000.0, 750.0, 500.0, 250.0), seed: int = 0,
-                 model_quant: dict | None = None, kv_scale_rule: str = "mse", cache_text_kv: bool = True) -> None:
+                 model_quant: dict | None = None, kv_scale_rule: str = "mse", cache_text_kv: bool = True,
+                 skip_dead_cache_writes: bool = True) -> None:
         self.cfg, self.device = cfg, torch.device(device)
         self.timesteps = [float(t) for t in timesteps]
         torch.manual_seed(seed)
@@ -36,6 +37,7 @@ class StreamingGenerator:
         self.model.kv_quant_config = self.kv_quant_config
         self.kv_cache = None
         self.cache_text_kv = cache_text_kv
+        self.skip_dead_cache_writes = skip_dead_cache_writes
 
     def reset_cache(self, frame_seq_length: int) -> None:
         cfg = self.cfg
@@ -63,7 +65,11 @@ class StreamingGenerator:
             f = x.shape[1]
             for si, t in enumerate(self.timesteps):
                 tt = torch.full((1, f), t, device=self.device, dtype=torch.float32)
-                flow = self.model(x, tt, context, self.kv_cache, start * fs, crossattn_cache=xcache)
+                # The K / V a denoising forward would write into the chunk's slot are overwritten by the next
+                # forward before anything reads them (the chunk attends its own K / V in bf16), so only the
+                # clean-context pass below writes; the cache after the chunk is the same either way.
+                flow = self.model(x, tt, context, self.kv_cache, start * fs, crossattn_cache=xcache,
+                                  apply_cache_updates=not self.skip_dead_cache_writes)
                 x = (x.float() + (sigmas[si + 1] - sigmas[si]) * flow.float()).to(noise.dtype)
             out[0, start:start + f] = x.transpose(0, 1)
             # clean-context pass: rewrites this chunk's K / V in the cache

@@ -313,3 +313,13 @@ def test_text_kv_cache_gives_identical_latents(gpu):
     a = StreamingGenerator(cfg, gpu, seed=4, cache_text_kv=True).generate(noise, ctx)
     b = StreamingGenerator(cfg, gpu, seed=4, cache_text_kv=False).generate(noise, ctx)
     assert torch.equal(a, b)
+    # so must leaving out the cache writes of the denoising forwards, which the clean pass overwrites
+    gen_c = StreamingGenerator(cfg, gpu, seed=4, skip_dead_cache_writes=False)
+    c = gen_c.generate(noise, ctx)
+    assert torch.equal(a, c)
+    gen_a = StreamingGenerator(cfg, gpu, seed=4)
+    gen_a.generate(noise, ctx)
+    for la, lc in zip(gen_a.kv_cache, gen_c.kv_cache):
+        assert la["_global_end"] == lc["_global_end"] and la["_local_end"] == lc["_local_end"]
+        for sa, sc in zip(la["k"] + la["v"], lc["k"] + lc["v"]):
+            assert torch.equal(sa.values, sc.values) and torch.equal(sa.amax, sc.amax)
