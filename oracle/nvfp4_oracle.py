@@ -34,6 +34,13 @@ Pinning status (what independent evidence fixes each function):
 * dequantize / matmul         exhaustive code x scale table; fp64 brute force; integer special case
 * attention / RoPE / adaLN    fp64 textbook forms, torch library routines (layer_norm,
                               complex multiply), norm preservation
+* gate_residual / gelu_tanh   the two eager bf16 operations / torch.nn.functional.gelu(approximate="tanh")
+
+Parity unpinned: the reference's production matmul is a CUTLASS kernel (fouroversix/.gitmodules, submodule
+absent, no pinned commit) and its attention is flash-attn 2.8.3 (not installed); neither result is
+recorded anywhere in the reference's tests.  ``fp4_matmul`` and ``attention`` here follow the reference's
+PyTorch matmul backend (pinned by one golden matmul) and the textbook softmax; agreement with the
+third-party kernels themselves is not pinned.
 """
 from __future__ import annotations
 
