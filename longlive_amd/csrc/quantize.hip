@@ -328,14 +328,15 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
 
   const bool vec = ((ldx & 7) == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
   uint8_t* s_bytes = reinterpret_cast<uint8_t*>(s_scales);
-  const int64_t tiles_x = Kp >> 6;
+  const uint32_t tiles_x = (uint32_t)(Kp >> 6);
 
   // Tiles are dealt to the resident workgroups round-robin, so the prologue above (amax reduction,
   // scale table) is paid once per workgroup and not once per tile.
 #pragma unroll 1
-  for (int64_t tile = blockIdx.x; tile < total_tiles; tile += gridDim.x) {
-  const int64_t row0 = (tile / tiles_x) * 128;
-  const int64_t col0 = (tile % tiles_x) * 64;
+  for (uint32_t tile = blockIdx.x; tile < (uint32_t)total_tiles; tile += gridDim.x) {  // 32-bit: cheap division
+  const uint32_t tile_y = tile / tiles_x;
+  const int64_t row0 = (int64_t)tile_y * 128;
+  const int64_t col0 = (int64_t)(tile - tile_y * tiles_x) * 64;
 #pragma unroll 1
   for (int it = 0; it < 2; ++it) {
     const int b = threadIdx.x + it * kThreads;  // block within the tile
@@ -362,7 +363,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
     s_bytes[(r & 31) * 16 + (r >> 5) * 4 + cb] = (uint8_t)sb;
   }
   __syncthreads();
-  if (threadIdx.x < 128) reinterpret_cast<uint32_t*>(scales)[tile * 128 + threadIdx.x] = s_scales[threadIdx.x];
+  if (threadIdx.x < 128) reinterpret_cast<uint32_t*>(scales)[(int64_t)tile * 128 + threadIdx.x] = s_scales[threadIdx.x];
   __syncthreads();  // the staged scale tile is rewritten by the next tile
   }
 }
@@ -395,6 +396,7 @@ extern "C" int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ld
              "ll_nvfp4_quantize: outputs must be 8-byte (values) / 4-byte (scales) aligned");
   const int64_t Mp = round_up(M, 128), Kp = round_up(K, 64);
   const int64_t total_tiles = (Kp / 64) * (Mp / 128);
+  LL_REQUIRE(total_tiles < (1ll << 31), "ll_nvfp4_quantize: tensor too large for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const uint16_t* xp = static_cast<const uint16_t*>(x);
   if (!amax_given) {
