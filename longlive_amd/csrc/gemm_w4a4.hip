@@ -167,14 +167,16 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
 #pragma unroll
   for (int f = 0; f < FA; ++f) {
     const int r = wm * 32 * FA + 32 * f + l32;
+    const int rs = r + (row0 & 127);  // row inside the staged 128-row scale blocks (64-row tiles start mid-block)
     a_voff[f] = r * kLdsRow + 16 * lh;
-    a_soff[f] = S::kAVals + S::kBVals + (r >> 7) * 1024 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + 2 * lh;
+    a_soff[f] = S::kAVals + S::kBVals + (rs >> 7) * 1024 + (rs & 31) * 16 + ((rs & 127) >> 5) * 4 + 2 * lh;
   }
 #pragma unroll
   for (int f = 0; f < FB; ++f) {
     const int r = wn * 32 * FB + 32 * f + l32;
+    const int rs = r + (col0 & 127);
     b_voff[f] = S::kAVals + r * kLdsRow + 16 * lh;
-    b_soff[f] = S::kAVals + S::kBVals + S::kAScales + (r >> 7) * 1024 + (r & 31) * 16 + ((r & 127) >> 5) * 4 + 2 * lh;
+    b_soff[f] = S::kAVals + S::kBVals + S::kAScales + (rs >> 7) * 1024 + (rs & 31) * 16 + ((rs & 127) >> 5) * 4 + 2 * lh;
   }
 
   float16v acc[FB][FA];
@@ -398,16 +400,22 @@ extern "C" int ll_nvfp4_gemm_tnt_act(const uint8_t* A_values, const uint8_t* A_s
       best = i;
     }
   }
-  if (const char* force = getenv("LL_GEMM_TILE")) {  // tuning aid: 0..3 selects a tile configuration
+  // Small problems: when even 128x128 tiles would occupy at most half of the CUs, 64x64 tiles (more decode
+  // work per MFMA, but four times the workgroups) finish sooner.  Configuration 3 (64x128) is only reachable
+  // through the override below.
+  if (((M + 127) / 128) * ((N + 127) / 128) <= 128) best = 4;
+  if (const char* force = getenv("LL_GEMM_TILE")) {  // tuning aid: 0..4 selects a tile configuration
     const int f = atoi(force);
-    if (f >= 0 && f < 3) best = f;
+    if (f >= 0 && f < 5) best = f;
   }
 #define LL_GEMM_ARGS A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, (int)M, (int)N, \
                      (int)Mp, (int)Np, (int)Kp, D, ldd, bias, activation, s
   switch (best) {
     case 0: return launch_gemm<4, 2>(LL_GEMM_ARGS);
     case 1: return launch_gemm<2, 4>(LL_GEMM_ARGS);
-    default: return launch_gemm<2, 2>(LL_GEMM_ARGS);
+    case 2: return launch_gemm<2, 2>(LL_GEMM_ARGS);
+    case 3: return launch_gemm<1, 2>(LL_GEMM_ARGS);
+    default: return launch_gemm<1, 1>(LL_GEMM_ARGS);
   }
 #undef LL_GEMM_ARGS
 }
