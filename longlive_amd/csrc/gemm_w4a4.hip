@@ -240,17 +240,22 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
     load_step(0);
     store_step(0);
     __syncthreads();
+    // A wave whose rows (or columns) all lie beyond M (N) only helps with the staging: in the last row of
+    // tiles of M = 2640 with 256-row tiles that is half of the waves.
+    const bool wave_has_output = row0 + wm * 32 * FA < M && col0 + wn * 32 * FB < N;
     for (int t = 0; t < nk; ++t) {
       load_step(min(t + 1, nk - 1));
+      if (wave_has_output) {
 #pragma unroll
-      for (int cc = 0; cc < 2; ++cc) {
-        Half h;
-        read_half(h, t & 1, cc);
+        for (int cc = 0; cc < 2; ++cc) {
+          Half h;
+          read_half(h, t & 1, cc);
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          Operands o;
-          decode(o, h, j);
-          mma(o);
+          for (int j = 0; j < 4; ++j) {
+            Operands o;
+            decode(o, h, j);
+            mma(o);
+          }
         }
       }
       store_step((t + 1) & 1);
