@@ -23,7 +23,7 @@ __device__ __forceinline__ void store8(void* out, int64_t off, const float (&v)[
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (DT == LL_DTYPE_BF16) {
-        w[i] = f32_to_bf16_bits(v[2 * i]) | (f32_to_bf16_bits(v[2 * i + 1]) << 16);
+        w[i] = pack_bf16x2(v[2 * i], v[2 * i + 1]);
       } else {
         const __half2 h = __floats2half2_rn(v[2 * i], v[2 * i + 1]);
         w[i] = *reinterpret_cast<const uint32_t*>(&h);

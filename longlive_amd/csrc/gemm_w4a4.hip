@@ -288,11 +288,9 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
     for (int g = 0; g < FB; ++g)
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
-        uint32_t o[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = f32_to_bf16_bits(acc[g][f][4 * rg + i] * alpha);
         *reinterpret_cast<uint2*>(ebuf + l32 * kEpiPitch + (32 * g + 8 * rg + 4 * lh) * 2) =
-            make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+            make_uint2(pack_bf16x2(acc[g][f][4 * rg] * alpha, acc[g][f][4 * rg + 1] * alpha),
+                       pack_bf16x2(acc[g][f][4 * rg + 2] * alpha, acc[g][f][4 * rg + 3] * alpha));
       }
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -305,17 +303,15 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
         if (bias) {  // bf16 result + bf16 bias, rounded to bf16 (the separate add of the reference)
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const uint32_t lo = f32_to_bf16_bits(__uint_as_float(w[i] << 16) + bias_f[2 * i]);
-            const uint32_t hi = f32_to_bf16_bits(__uint_as_float(w[i] & 0xFFFF0000u) + bias_f[2 * i + 1]);
-            w[i] = lo | (hi << 16);
+            w[i] = pack_bf16x2(__uint_as_float(w[i] << 16) + bias_f[2 * i],
+                               __uint_as_float(w[i] & 0xFFFF0000u) + bias_f[2 * i + 1]);
           }
         }
         if (act == LL_ACT_GELU_TANH) {  // GELU (tanh form) of the bf16 value, computed in fp32, rounded to bf16
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
-            const uint32_t lo = f32_to_bf16_bits(gelu_tanh_f32(__uint_as_float(w[i] << 16)));
-            const uint32_t hi = f32_to_bf16_bits(gelu_tanh_f32(__uint_as_float(w[i] & 0xFFFF0000u)));
-            w[i] = lo | (hi << 16);
+            w[i] = pack_bf16x2(gelu_tanh_f32(__uint_as_float(w[i] << 16)),
+                               gelu_tanh_f32(__uint_as_float(w[i] & 0xFFFF0000u)));
           }
         }
         uint16_t* dst = D + (int64_t)m * ldd + n_lane;

@@ -33,11 +33,17 @@ inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 // ----------------------------------------------------------------------------- formats
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
 
-// fp32 -> bf16 bits, round to nearest even (NaN stays NaN).
+// fp32 -> bf16 bits, round to nearest even, with the hardware conversion of gfx950 (v_cvt_pk_bf16_f32;
+// NaN becomes a quiet NaN).
+typedef __bf16 bf16x2_hw __attribute__((ext_vector_type(2)));
+typedef float f32x2_hw __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u >> 16) | 0x40u;
-  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+  return (uint32_t)__builtin_bit_cast(uint16_t, static_cast<__bf16>(f));
+}
+// Two values at once: lo in bits 0-15, hi in bits 16-31.
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  const f32x2_hw v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_hw));
 }
 __device__ __forceinline__ float round_to_bf16(float f) { return __uint_as_float(f32_to_bf16_bits(f) << 16); }
 
