@@ -650,11 +650,32 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     }
     __syncthreads();
   }
+  typedef __attribute__((address_space(1))) const void* gptr_t;
+  typedef __attribute__((address_space(3))) void* lptr_t;
   for (; it < n_iter; ++it) {
     const uint8_t* cur = smem + (it & 1) * kStageBytes;
     const uint8_t* kt_base = cur + kp * kKTileBytes;
     const uint8_t* vt_base = cur + 2 * kKTileBytes + kp * kVTileBytes;
     const int tile_base = it * kIterKeys + kp * kTileKeys;
+    // A successor that lies wholly in the bf16 chunk is brought in ahead of the MFMAs: its K rows go
+    // straight from global memory into the other stage (one 256-byte row per wave instruction, 32 rows per
+    // wave), its V pieces are requested now and transposed into LDS after the PV phase.
+    const bool next_is_chunk = iter_base >= n_cached && iter_base + kIterKeys <= Lk_i;  // iter_base = first key of tile it + 1
+    uint4 vraw[4][2];
+    if (next_is_chunk) {
+      uint8_t* nxt = smem + ((it + 1) & 1) * kStageBytes;
+      const uint16_t* ksrc = p.k_new + ((int64_t)(iter_base + wave * 32 - n_cached) * p.H + head) * kHeadDim + lane * 2;
+      uint8_t* kdst = nxt + (wave >> 1) * kKTileBytes + ((wave & 1) * 32) * kKPitch;
+#pragma unroll
+      for (int r = 0; r < 32; ++r)
+        __builtin_amdgcn_global_load_lds((gptr_t)(ksrc + (int64_t)r * p.H * kHeadDim), (lptr_t)(kdst + r * kKPitch), 4, 0, 0);
+#pragma unroll
+      for (int kk = 0; kk < 4; ++kk) {
+        const uint16_t* vsrc = p.v_new + ((int64_t)(iter_base + v_local + kk - n_cached) * p.H + head) * kHeadDim + v_blk * 16;
+        vraw[kk][0] = load_global_b128(vsrc);
+        vraw[kk][1] = load_global_b128(vsrc + 8);
+      }
+    }
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
       const int half_base = tile_base + kt * 32;
@@ -674,7 +695,25 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
         pv_half(vt_base, kt);
       }
     }
-    if (it + 1 < n_iter) {
+    if (next_is_chunk) {
+      uint8_t* vdst = smem + ((it + 1) & 1) * kStageBytes + v_dst_off;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {  // elements 2 i, 2 i + 1 of the thread's 16, for its 4 keys -> two rows of V^T
+        uint32_t w[4];
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+          const uint4 q = vraw[kk][i >> 2];
+          w[kk] = (i & 3) == 0 ? q.x : (i & 3) == 1 ? q.y : (i & 3) == 2 ? q.z : q.w;
+        }
+        // v_perm_b32: bytes 0-3 come from the second operand, 4-7 from the first
+        *reinterpret_cast<uint2*>(vdst + (2 * i) * kVPitch) =
+            make_uint2(__builtin_amdgcn_perm(w[1], w[0], 0x05040100u), __builtin_amdgcn_perm(w[3], w[2], 0x05040100u));
+        *reinterpret_cast<uint2*>(vdst + (2 * i + 1) * kVPitch) =
+            make_uint2(__builtin_amdgcn_perm(w[1], w[0], 0x07060302u), __builtin_amdgcn_perm(w[3], w[2], 0x07060302u));
+      }
+      iter_base += kIterKeys;  // the slot bookkeeping of advance() has no use beyond the cache
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K rows have landed in LDS
+    } else if (it + 1 < n_iter) {
       decode_k_any((it + 1) & 1);
       decode_v_any((it + 1) & 1);
       advance();
