@@ -58,6 +58,28 @@ int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ldx, int rule
                       float* workspace, void* stream);
 
 /*
+ * Amax sink.  The tensor-wide absolute maximum that NVFP4 quantization starts from
+ * (quantize/pytorch/reference.py:242-255, x.abs().max()) costs a pass over the tensor.  A kernel of this
+ * library that writes the tensor can leave the maximum behind instead: it raises LL_AMAX_PARTS 64-bit slots,
+ * each (epoch << 32) | float bits, with atomic max.  A newer epoch beats every older value, so the buffer is
+ * zeroed once when it is allocated and never again; every producer call on a buffer passes an epoch greater
+ * than all earlier ones (1, 2, 3, ...; clear the buffer before wrapping around), and
+ * ll_nvfp4_quantize_from_sink reads the slots of that epoch.  Calls that share a buffer must be ordered
+ * (one stream).
+ */
+#define LL_AMAX_PARTS 1024
+typedef struct ll_amax_sink {
+  uint64_t* parts;   /* device memory, LL_AMAX_PARTS entries, 8-byte aligned */
+  uint32_t epoch;    /* > 0 */
+} ll_amax_sink;
+
+/* ll_nvfp4_quantize whose tensor amax comes from an amax sink that the producer of x has filled with the
+ * same epoch; amax (f32[1]) is written.  The bytes equal those of ll_nvfp4_quantize with amax_given == 0. */
+int ll_nvfp4_quantize_from_sink(const void* x, int64_t M, int64_t K, int64_t ldx, int rule,
+                                uint8_t* values, uint8_t* scales, float* amax,
+                                const ll_amax_sink* amax_sink, void* stream);
+
+/*
  * Replaces QuantizedTensor.dequantize (fouroversix/src/fouroversix/quantize/quantized_tensor.py:184-214):
  * out[r, c] = cast(((e2m1 * e4m3) * amax) / (e2m1_max * e4m3_max)) for r < M, c < K; ldo in elements.
  */
@@ -91,6 +113,33 @@ int ll_nvfp4_gemm_tnt_act(const uint8_t* A_values, const uint8_t* A_scales, cons
                           void* D, int64_t ldd, const void* bias, int activation, void* stream);
 
 /*
+ * ll_nvfp4_gemm_tnt with the element-wise operations that follow a projection in the DiT block folded into
+ * the epilogue.  With y = bf16(alpha * acc) the steps are, in this order and each optional:
+ *   y = bf16(y + bias[n])                                   (model/modules/linear.py:73-74)
+ *   y = bf16(act(y))                                         (causal_model.py:822-824, nn.GELU(approximate="tanh"))
+ *   y = bf16(y * gate[m / gate_rows, n])   only with residual (causal_model.py:889, 919-920: y * e[2] / e[5])
+ *   y = bf16(residual[m, n] + y)                             (causal_model.py:889, 906, 919-920: x + ...)
+ *   max |y| goes to amax_sink (see ll_amax_sink) when amax_sink.parts is not NULL.
+ * Every rounding is the one the separate bf16 operations of the reference perform.
+ *   gate bf16, row stride gate_stride elements; residual bf16 [M, N], row stride ldr; both 16-byte aligned,
+ *   strides multiples of 8, and N a multiple of 8 when a residual is given.  residual may alias D.
+ */
+typedef struct ll_gemm_epilogue {
+  const void* bias;       /* bf16 [N] or NULL */
+  int activation;         /* LL_ACT_NONE or LL_ACT_GELU_TANH */
+  const void* gate;       /* bf16 or NULL (needs residual) */
+  int64_t gate_rows;      /* rows of D that share one gate row */
+  int64_t gate_stride;
+  const void* residual;   /* bf16 [M, N] or NULL */
+  int64_t ldr;
+  ll_amax_sink amax_sink; /* parts == NULL: none */
+} ll_gemm_epilogue;
+int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A_scales, const uint8_t* B_values,
+                            const uint8_t* B_scales, const float* alpha, const float* amax_a, const float* amax_b,
+                            float denom_a, float denom_b, int64_t M, int64_t N, int64_t Mp, int64_t Np, int64_t Kp,
+                            void* D, int64_t ldd, const ll_gemm_epilogue* epilogue, void* stream);
+
+/*
  * Replaces torch.ops.longlive_kernels.dequantize_kv_cache_fp4 (utils/kernel/kv_dequant.cpp:14,
  * utils/kernel/kv_dequant_cuda.cu:59-239) and the Triton fp4_dequantize it falls back to
  * (utils/nvfp4_kernel.py:40-176): n_blocks cache slots, each NVFP4 [rows_padded, 128] holding
@@ -119,6 +168,15 @@ int ll_kv_attention(const void* q, int64_t Lq, int num_heads,
                     const void* k_new, const void* v_new, int64_t n_new,
                     float softmax_scale, void* out, void* stream);
 
+/* ll_kv_attention that also leaves max |out| in amax_sink (may be NULL), for the quantization in front of the
+ * output projection (causal_model.py:783-785 feeds FourOverSixLinear.forward, model/modules/linear.py:243-270). */
+int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads,
+                         const uint64_t* k_values_ptrs, const uint64_t* k_scales_ptrs, const uint64_t* k_amax_ptrs,
+                         const uint64_t* v_values_ptrs, const uint64_t* v_scales_ptrs, const uint64_t* v_amax_ptrs,
+                         int64_t n_cached, int block_token_size, float e2m1_max, float e4m3_max,
+                         const void* k_new, const void* v_new, int64_t n_new,
+                         float softmax_scale, void* out, const ll_amax_sink* amax_sink, void* stream);
+
 /* Plain bf16 attention (cross-attention to the text context; wan_5b/modules/causal_model.py:197-262):
  * q [Lq,H,128], k/v [Lk,H,128], out [Lq,H,128], no mask. */
 int ll_attention_bf16(const void* q, const void* k, const void* v, int64_t Lq, int64_t Lk, int num_heads,
@@ -139,6 +197,13 @@ int ll_rope_apply(const void* x, int64_t S, int N, int D, int64_t x_stride_s, in
 int ll_adaln_modulate(const void* x, int64_t B, int64_t L, int C, const void* scale, const void* shift,
                       int64_t scale_stride_b, int64_t scale_stride_f, int64_t shift_stride_b, int64_t shift_stride_f,
                       int64_t frame_seqlen, float eps, int add_one_to_scale, void* out, void* stream);
+
+/* ll_adaln_modulate that also leaves max |y| in amax_sink (may be NULL), for the quantization that follows
+ * (causal_model.py:869-878, 909-918). */
+int ll_adaln_modulate_amax(const void* x, int64_t B, int64_t L, int C, const void* scale, const void* shift,
+                           int64_t scale_stride_b, int64_t scale_stride_f, int64_t shift_stride_b,
+                           int64_t shift_stride_f, int64_t frame_seqlen, float eps, int add_one_to_scale, void* out,
+                           const ll_amax_sink* amax_sink, void* stream);
 
 /*
  * Gated residual of the DiT block (wan_5b/modules/causal_model.py:889, 919-920):

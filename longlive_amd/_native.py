@@ -29,6 +29,8 @@ _SIGNATURES = {
     "ll_nvfp4_quantize_workspace_floats": (c_size_t, []),
     "ll_nvfp4_quantize": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                   c_void_p, c_void_p]),
+    "ll_nvfp4_quantize_from_sink": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p,
+                                            c_void_p, c_void_p]),
     "ll_nvfp4_dequantize": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,
                                     c_void_p, c_int, c_int64, c_void_p]),
     "ll_nvfp4_gemm_tnt": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
@@ -37,16 +39,24 @@ _SIGNATURES = {
     "ll_nvfp4_gemm_tnt_act": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                       c_float, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64,
                                       c_void_p, c_int, c_void_p]),
+    "ll_nvfp4_gemm_tnt_fused": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
+                                        c_float, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64,
+                                        c_void_p, c_void_p]),
     "ll_kv_dequantize_blocks": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float,
                                         c_void_p, c_void_p]),
     "ll_kv_attention": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                 c_int64, c_int, c_float, c_float, c_void_p, c_void_p, c_int64, c_float, c_void_p,
                                 c_void_p]),
+    "ll_kv_attention_amax": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                     c_void_p, c_int64, c_int, c_float, c_float, c_void_p, c_void_p, c_int64, c_float,
+                                     c_void_p, c_void_p, c_void_p]),
     "ll_attention_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_float, c_void_p, c_void_p]),
     "ll_rope_apply": (c_int, [c_void_p, c_int64, c_int, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int64,
                               c_void_p, c_void_p]),
     "ll_adaln_modulate": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64,
                                   c_int64, c_int64, c_float, c_int, c_void_p, c_void_p]),
+    "ll_adaln_modulate_amax": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int64,
+                                       c_int64, c_int64, c_int64, c_float, c_int, c_void_p, c_void_p, c_void_p]),
     "ll_qk_norm_rope": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p, c_int64, c_void_p,
                                 c_void_p, c_void_p]),
     "ll_gate_residual": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_int64, c_int64,
@@ -120,10 +130,61 @@ def padded_shape(shape: tuple[int, int]) -> tuple[int, int]:
     return (-(-shape[0] // 128) * 128, -(-shape[1] // 64) * 64)
 
 
+# --------------------------------------------------------------------------- amax sink
+AMAX_PARTS = 1024
+
+
+class AmaxSinkStruct(ctypes.Structure):
+    """struct ll_amax_sink of include/ll_nvfp4.h."""
+    _fields_ = [("parts", c_void_p), ("epoch", ctypes.c_uint32)]
+
+
+class AmaxTicket:
+    """One use of a device's amax sink: handed to the kernel that writes a tensor (``amax_out=``) and then to
+    the quantization of that tensor (``amax=``), which reads the maximum the producer left."""
+
+    __slots__ = ("parts", "epoch")
+
+    def __init__(self, parts: torch.Tensor, epoch: int) -> None:
+        self.parts, self.epoch = parts, epoch
+
+    def struct(self) -> AmaxSinkStruct:
+        return AmaxSinkStruct(self.parts.data_ptr(), self.epoch)
+
+
+_sinks: dict = {}
+
+
+def amax_ticket(device: torch.device) -> AmaxTicket:
+    """A fresh epoch on the device's amax sink buffer.  Epochs only grow, which is what lets the buffer go
+    uncleared between uses; producer and consumer must run on one stream, in that order."""
+    device = torch.device(device)
+    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    entry = _sinks.get(key)
+    if entry is None or entry[1] >= 0xFFFFFFFE:
+        entry = [torch.zeros(AMAX_PARTS, dtype=torch.int64, device=device), 0]
+        _sinks[key] = entry
+    entry[1] += 1
+    return AmaxTicket(entry[0], entry[1])
+
+
+def _sink_struct(ticket):
+    if ticket is None:
+        return AmaxSinkStruct(None, 0)
+    if not isinstance(ticket, AmaxTicket):
+        raise TypeError("amax_out must be an AmaxTicket (see amax_ticket)")
+    return ticket.struct()
+
+
 # --------------------------------------------------------------------------- quantize / dequantize
 def quantize(x: torch.Tensor, rule: str, amax: torch.Tensor | None = None, out=None):
     """x bf16 [M, K] -> (values u8 [Mp, Kp/2], scales float8_e4m3fn [Mp*Kp/16] blocked, amax f32[1]).
-    ``out`` = (values, scale_factors, amax) buffers of exactly those shapes to write into (KV slots)."""
+    ``out`` = (values, scale_factors, amax) buffers of exactly those shapes to write into (KV slots).
+    ``amax``: a float32[1] tensor to quantize against, or the :class:`AmaxTicket` the producer of ``x`` was
+    given, in which case the bytes equal those of ``amax=None``."""
+    ticket = amax if isinstance(amax, AmaxTicket) else None
+    if ticket is not None:
+        amax = None
     _require_cuda(x, amax)
     if x.ndim != 2:
         raise ValueError("quantize expects a 2-D tensor")
@@ -147,10 +208,16 @@ def quantize(x: torch.Tensor, rule: str, amax: torch.Tensor | None = None, out=N
         scales = torch.empty(Mp * Kp // 16, dtype=torch.uint8, device=x.device)
         amax_t = amax.reshape(1).to(torch.float32).contiguous() if given else torch.empty(
             1, dtype=torch.float32, device=x.device)
-    ws = None if given else _workspace(x.device)
+    ws = None if given or ticket is not None else _workspace(x.device)
     with torch.cuda.device(x.device):
-        code = load().ll_nvfp4_quantize(x.data_ptr(), M, K, x.stride(0), RULE_IDS[rule], values.data_ptr(),
-                                        scales.data_ptr(), amax_t.data_ptr(), int(given), _ptr(ws), _stream())
+        if ticket is not None:
+            sink = ticket.struct()
+            code = load().ll_nvfp4_quantize_from_sink(x.data_ptr(), M, K, x.stride(0), RULE_IDS[rule],
+                                                      values.data_ptr(), scales.data_ptr(), amax_t.data_ptr(),
+                                                      ctypes.byref(sink), _stream())
+        else:
+            code = load().ll_nvfp4_quantize(x.data_ptr(), M, K, x.stride(0), RULE_IDS[rule], values.data_ptr(),
+                                            scales.data_ptr(), amax_t.data_ptr(), int(given), _ptr(ws), _stream())
     _check(code, "ll_nvfp4_quantize")
     if out is not None:
         return out
@@ -169,11 +236,21 @@ def dequantize(values, scales, amax, rule: str, padded, original, dtype: torch.d
 
 
 # --------------------------------------------------------------------------- GEMM
+class GemmEpilogue(ctypes.Structure):
+    """struct ll_gemm_epilogue of include/ll_nvfp4.h."""
+    _fields_ = [("bias", c_void_p), ("activation", c_int), ("gate", c_void_p), ("gate_rows", c_int64),
+                ("gate_stride", c_int64), ("residual", c_void_p), ("ldr", c_int64), ("amax_sink", AmaxSinkStruct)]
+
+
 def gemm(a_values, a_scales, b_values, b_scales, M: int, N: int, *, alpha=None, amax_a=None, amax_b=None,
-         denom_a: float = 1536.0, denom_b: float = 1536.0, bias=None, out=None, activation=None) -> torch.Tensor:
+         denom_a: float = 1536.0, denom_b: float = 1536.0, bias=None, out=None, activation=None,
+         residual=None, gate=None, gate_rows: int = 0, amax_out=None) -> torch.Tensor:
+    """D = A @ B^T with the epilogue of ll_nvfp4_gemm_tnt_fused: bias, activation, then
+    ``residual + y * gate[m // gate_rows]`` (gate [G, N], rows may be strided) or ``residual + y``, and the
+    absolute maximum of the result left in ``amax_out`` (an :class:`AmaxTicket`)."""
     if activation is not None and activation not in ACTIVATION_IDS:
         raise ValueError(f"unknown epilogue activation {activation!r}")
-    _require_cuda(a_values, a_scales, b_values, b_scales, alpha, amax_a, amax_b, bias)
+    _require_cuda(a_values, a_scales, b_values, b_scales, alpha, amax_a, amax_b, bias, residual, gate)
     Mp, Kb = a_values.shape
     Np, Kb2 = b_values.shape
     if Kb != Kb2:
@@ -182,14 +259,24 @@ def gemm(a_values, a_scales, b_values, b_scales, M: int, N: int, *, alpha=None, 
         out = torch.empty((M, N), dtype=torch.bfloat16, device=a_values.device)
     if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N or not bias.is_contiguous()):
         raise ValueError("bias must be a contiguous bfloat16 vector of length N")
+    epi = GemmEpilogue(_ptr(bias), ACTIVATION_IDS[activation] if activation else 0, None, 0, 0, None, 0,
+                       _sink_struct(amax_out))
+    if residual is not None:
+        if residual.dtype != torch.bfloat16 or residual.shape != (M, N) or residual.stride(1) != 1:
+            raise ValueError("residual must be bfloat16 [M, N] with contiguous rows")
+        epi.residual, epi.ldr = residual.data_ptr(), residual.stride(0)
+        if gate is not None:
+            if gate.dtype != torch.bfloat16 or gate.dim() != 2 or gate.shape[1] != N or gate.stride(1) != 1 \
+                    or gate_rows <= 0 or gate.shape[0] * gate_rows < M:
+                raise ValueError("gate must be bfloat16 [G, N] with contiguous rows and G * gate_rows >= M")
+            epi.gate, epi.gate_rows, epi.gate_stride = gate.data_ptr(), gate_rows, gate.stride(0)
+    elif gate is not None:
+        raise ValueError("a gate needs a residual")
     with torch.cuda.device(a_values.device):
-        args = (a_values.data_ptr(), a_scales.data_ptr(), b_values.data_ptr(), b_scales.data_ptr(), _ptr(alpha),
-                _ptr(amax_a), _ptr(amax_b), denom_a, denom_b, M, N, Mp, Np, Kb * 2, out.data_ptr(), out.stride(0),
-                _ptr(bias))
-        if activation is None:
-            code = load().ll_nvfp4_gemm_tnt(*args, _stream())
-        else:
-            code = load().ll_nvfp4_gemm_tnt_act(*args, ACTIVATION_IDS[activation], _stream())
+        code = load().ll_nvfp4_gemm_tnt_fused(
+            a_values.data_ptr(), a_scales.data_ptr(), b_values.data_ptr(), b_scales.data_ptr(), _ptr(alpha),
+            _ptr(amax_a), _ptr(amax_b), denom_a, denom_b, M, N, Mp, Np, Kb * 2, out.data_ptr(), out.stride(0),
+            ctypes.byref(epi), _stream())
     _check(code, "ll_nvfp4_gemm_tnt")
     return out
 
@@ -206,9 +293,12 @@ def kv_dequantize_blocks(values_ptrs, scales_ptrs, amax_ptrs, n_blocks, num_head
     return out
 
 
-def kv_attention(q, tables, n_cached, block_token_size, e2m1_max, e4m3_max, k_new, v_new, softmax_scale):
-    """q [Lq, H, 128] bf16; tables = six int64 device tensors of slot pointers (or None when n_cached == 0)."""
+def kv_attention(q, tables, n_cached, block_token_size, e2m1_max, e4m3_max, k_new, v_new, softmax_scale,
+                 amax_out=None):
+    """q [Lq, H, 128] bf16; tables = six int64 device tensors of slot pointers (or None when n_cached == 0).
+    ``amax_out`` (an :class:`AmaxTicket`) receives the absolute maximum of the result."""
     _require_cuda(q, k_new, v_new)
+    sink = _sink_struct(amax_out)
     if q.dtype != torch.bfloat16 or q.ndim != 3 or q.shape[-1] != 128 or not q.is_contiguous():
         raise ValueError("q must be a contiguous bfloat16 [Lq, H, 128] tensor")
     Lq, H, _ = q.shape
@@ -222,15 +312,15 @@ def kv_attention(q, tables, n_cached, block_token_size, e2m1_max, e4m3_max, k_ne
     out = torch.empty_like(q)
     t = [None] * 6 if tables is None else [x.data_ptr() for x in tables]
     with torch.cuda.device(q.device):
-        code = load().ll_kv_attention(q.data_ptr(), Lq, H, *t, n_cached, block_token_size, float(e2m1_max),
-                                      float(e4m3_max), _ptr(k_new), _ptr(v_new), n_new, float(softmax_scale),
-                                      out.data_ptr(), _stream())
+        code = load().ll_kv_attention_amax(q.data_ptr(), Lq, H, *t, n_cached, block_token_size, float(e2m1_max),
+                                           float(e4m3_max), _ptr(k_new), _ptr(v_new), n_new, float(softmax_scale),
+                                           out.data_ptr(), ctypes.byref(sink), _stream())
     _check(code, "ll_kv_attention")
     return out
 
 
-def attention_bf16(q, k, v, softmax_scale):
-    return kv_attention(q, None, 0, 0, 6.0, 256.0, k, v, softmax_scale)
+def attention_bf16(q, k, v, softmax_scale, amax_out=None):
+    return kv_attention(q, None, 0, 0, 6.0, 256.0, k, v, softmax_scale, amax_out=amax_out)
 
 
 # --------------------------------------------------------------------------- elementwise
@@ -275,8 +365,10 @@ def qk_norm_rope(x, weight, eps, cos, sin, num_heads, seq_len=None, smooth=False
     return (out, out_s) if smooth else out
 
 
-def adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps=1e-6, add_one_to_scale=True):
+def adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps=1e-6, add_one_to_scale=True, amax_out=None):
+    """``amax_out`` (an :class:`AmaxTicket`) receives the absolute maximum of the result."""
     _require_cuda(x, e_scale, e_shift)
+    sink = _sink_struct(amax_out)
     if x.ndim != 3 or x.dtype != torch.bfloat16 or not x.is_contiguous():
         raise ValueError("x must be a contiguous bfloat16 [B, L, C] tensor")
     B, L, C = x.shape
@@ -286,9 +378,10 @@ def adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps=1e-6, add_one_to_scale
             raise ValueError(f"{name} must be bfloat16 [B, F, 1, C] = {(B, F, 1, C)}, got {tuple(e.shape)}")
     out = torch.empty_like(x)
     with torch.cuda.device(x.device):
-        code = load().ll_adaln_modulate(x.data_ptr(), B, L, C, e_scale.data_ptr(), e_shift.data_ptr(),
-                                        e_scale.stride(0), e_scale.stride(1), e_shift.stride(0), e_shift.stride(1),
-                                        frame_seqlen, float(eps), int(add_one_to_scale), out.data_ptr(), _stream())
+        code = load().ll_adaln_modulate_amax(x.data_ptr(), B, L, C, e_scale.data_ptr(), e_shift.data_ptr(),
+                                             e_scale.stride(0), e_scale.stride(1), e_shift.stride(0),
+                                             e_shift.stride(1), frame_seqlen, float(eps), int(add_one_to_scale),
+                                             out.data_ptr(), ctypes.byref(sink), _stream())
     _check(code, "ll_adaln_modulate")
     return out
 

@@ -42,6 +42,7 @@ struct AttnParams {
   const uint16_t *k_new, *v_new;
   float scale_log2;  // softmax scale * log2(e)
   uint16_t* out;
+  AmaxSink sink;  // receives max |out| when sink.parts is not null
   int n_qtiles;
 };
 
@@ -746,6 +747,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   }
   __syncthreads();
   if (kp == 0) {
+    float out_max = 0.0f;
 #pragma unroll
     for (int qt = 0; qt < 2; ++qt) {
       const float m1 = xm[(qh * 2 + qt) * 64 + lane], l1 = xl[(qh * 2 + qt) * 64 + lane];
@@ -767,9 +769,15 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
               v[i] = (o[dt][qt][4 * rg + i] * a0 + o1 * a1) * inv_l;
             }
             const int d = dt * 32 + 8 * rg + 4 * lh;
-            *reinterpret_cast<uint2*>(dst + d) = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+            const uint2 packed = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+            *reinterpret_cast<uint2*>(dst + d) = packed;
+            out_max = abs_max_bf16x8(make_uint4(packed.x, packed.y, 0u, 0u), out_max);
           }
       }
+    }
+    if (p.sink.parts) {
+      out_max = wave_max(out_max);
+      if (lane == 0) amax_sink_update(p.sink, blockIdx.x * 2 + qh, out_max);
     }
   }
 }
@@ -801,6 +809,18 @@ extern "C" int ll_kv_attention(const void* q, int64_t Lq, int num_heads, const u
                                const uint64_t* v_amax_ptrs, int64_t n_cached, int block_token_size, float e2m1_max,
                                float e4m3_max, const void* k_new, const void* v_new, int64_t n_new,
                                float softmax_scale, void* out, void* stream) {
+  return ll_kv_attention_amax(q, Lq, num_heads, k_values_ptrs, k_scales_ptrs, k_amax_ptrs, v_values_ptrs,
+                              v_scales_ptrs, v_amax_ptrs, n_cached, block_token_size, e2m1_max, e4m3_max, k_new, v_new,
+                              n_new, softmax_scale, out, nullptr, stream);
+}
+
+extern "C" int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads, const uint64_t* k_values_ptrs,
+                                    const uint64_t* k_scales_ptrs, const uint64_t* k_amax_ptrs,
+                                    const uint64_t* v_values_ptrs, const uint64_t* v_scales_ptrs,
+                                    const uint64_t* v_amax_ptrs, int64_t n_cached, int block_token_size,
+                                    float e2m1_max, float e4m3_max, const void* k_new, const void* v_new,
+                                    int64_t n_new, float softmax_scale, void* out, const ll_amax_sink* amax_sink,
+                                    void* stream) {
   using namespace ll;
   LL_REQUIRE(q && out, "ll_kv_attention: null q/out");
   LL_REQUIRE(Lq > 0 && num_heads > 0 && n_cached >= 0 && n_new >= 0 && n_cached + n_new > 0,
@@ -839,6 +859,12 @@ extern "C" int ll_kv_attention(const void* q, int64_t Lq, int num_heads, const u
   p.v_new = static_cast<const uint16_t*>(v_new);
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.out = static_cast<uint16_t*>(out);
+  if (amax_sink && amax_sink->parts) {
+    LL_REQUIRE((reinterpret_cast<uintptr_t>(amax_sink->parts) & 7) == 0 && amax_sink->epoch != 0,
+               "ll_kv_attention_amax: amax sink needs 8-byte alignment and a non-zero epoch");
+    p.sink.parts = reinterpret_cast<unsigned long long*>(amax_sink->parts);
+    p.sink.epoch = amax_sink->epoch;
+  }
   return launch_attention(p, static_cast<hipStream_t>(stream));
 }
 

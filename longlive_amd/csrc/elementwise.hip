@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kRowThreads) void adaln_kernel(const uint16_t* __re
                                                             const uint16_t* __restrict__ shift, int64_t sc_sb,
                                                             int64_t sc_sf, int64_t sh_sb, int64_t sh_sf,
                                                             int64_t frame_seqlen, float eps, int add_one,
-                                                            uint16_t* __restrict__ out) {
+                                                            uint16_t* __restrict__ out, AmaxSink sink) {
   __shared__ float sm[kRowThreads / 64];
   const int64_t row = blockIdx.x;
   const int64_t b = row / L, l = row - b * L, f = l / frame_seqlen;
@@ -112,6 +112,7 @@ __global__ __launch_bounds__(kRowThreads) void adaln_kernel(const uint16_t* __re
   const uint16_t* scr = scale + b * sc_sb + f * sc_sf;
   const uint16_t* shr = shift + b * sh_sb + f * sh_sf;
   uint16_t* orow = out + row * (int64_t)C;
+  float out_max = 0.0f;
 #pragma unroll
   for (int i = 0; i < kMaxChunks; ++i) {
     const int c = threadIdx.x + i * kRowThreads;
@@ -126,8 +127,14 @@ __global__ __launch_bounds__(kRowThreads) void adaln_kernel(const uint16_t* __re
         const float prod = round_to_bf16(xn * s);
         y[j] = prod + h8[j];
       }
-      *reinterpret_cast<uint4*>(orow + c * 8) = pack8(y);
+      const uint4 packed = pack8(y);
+      *reinterpret_cast<uint4*>(orow + c * 8) = packed;
+      out_max = abs_max_bf16x8(packed, out_max);
     }
+  }
+  if (sink.parts) {
+    out_max = wave_max(out_max);
+    if ((threadIdx.x & 63) == 0) amax_sink_update(sink, blockIdx.x * (kRowThreads / 64) + (threadIdx.x >> 6), out_max);
   }
 }
 
@@ -288,7 +295,22 @@ extern "C" int ll_adaln_modulate(const void* x, int64_t B, int64_t L, int C, con
                                  int64_t scale_stride_b, int64_t scale_stride_f, int64_t shift_stride_b,
                                  int64_t shift_stride_f, int64_t frame_seqlen, float eps, int add_one_to_scale,
                                  void* out, void* stream) {
+  return ll_adaln_modulate_amax(x, B, L, C, scale, shift, scale_stride_b, scale_stride_f, shift_stride_b,
+                                shift_stride_f, frame_seqlen, eps, add_one_to_scale, out, nullptr, stream);
+}
+
+extern "C" int ll_adaln_modulate_amax(const void* x, int64_t B, int64_t L, int C, const void* scale,
+                                      const void* shift, int64_t scale_stride_b, int64_t scale_stride_f,
+                                      int64_t shift_stride_b, int64_t shift_stride_f, int64_t frame_seqlen, float eps,
+                                      int add_one_to_scale, void* out, const ll_amax_sink* amax_sink, void* stream) {
   using namespace ll;
+  AmaxSink sink{};
+  if (amax_sink && amax_sink->parts) {
+    LL_REQUIRE((reinterpret_cast<uintptr_t>(amax_sink->parts) & 7) == 0 && amax_sink->epoch != 0,
+               "ll_adaln_modulate_amax: amax sink needs 8-byte alignment and a non-zero epoch");
+    sink.parts = reinterpret_cast<unsigned long long*>(amax_sink->parts);
+    sink.epoch = amax_sink->epoch;
+  }
   LL_REQUIRE(x && scale && shift && out, "ll_adaln_modulate: null pointer");
   LL_REQUIRE(B > 0 && L > 0 && C > 0 && C % 8 == 0 && C <= kRowThreads * kMaxChunks * 8 && frame_seqlen > 0 &&
                  L % frame_seqlen == 0,
@@ -302,7 +324,7 @@ extern "C" int ll_adaln_modulate(const void* x, int64_t B, int64_t L, int C, con
   hipLaunchKernelGGL(adaln_kernel, dim3((unsigned)(B * L)), dim3(kRowThreads), 0, static_cast<hipStream_t>(stream),
                      static_cast<const uint16_t*>(x), L, C, static_cast<const uint16_t*>(scale),
                      static_cast<const uint16_t*>(shift), scale_stride_b, scale_stride_f, shift_stride_b,
-                     shift_stride_f, frame_seqlen, eps, add_one_to_scale, static_cast<uint16_t*>(out));
+                     shift_stride_f, frame_seqlen, eps, add_one_to_scale, static_cast<uint16_t*>(out), sink);
   LL_CHECK_LAUNCH("adaln_kernel");
   return LL_OK;
 }

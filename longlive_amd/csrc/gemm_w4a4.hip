@@ -60,13 +60,29 @@ __device__ __forceinline__ float gelu_tanh_f32(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * u2));
 }
 
+// What the epilogue does to y = bf16(alpha * acc), in this order (each step optional):
+//   y = bf16(y + bias[n]);  y = bf16(act(y));  y = bf16(y * gate[m / gate_rows, n]) (only with residual);
+//   y = bf16(residual[m, n] + y);  max |y| goes to the amax sink.
+struct GemmEpilogue {
+  const uint16_t* bias;
+  int act;
+  const uint16_t* gate;
+  int gate_rows;
+  int64_t gate_stride;
+  const uint16_t* residual;
+  int64_t ldr;
+  AmaxSink sink;
+};
+
 template <int FA, int FB>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
     const uint8_t* __restrict__ Av, const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bv,
     const uint8_t* __restrict__ Bs, const float* __restrict__ alpha_ptr, const float* __restrict__ amax_a,
     const float* __restrict__ amax_b, float inv_denom_a, float inv_denom_b, int M, int N, int Mp, int Np, int Kp,
-    uint16_t* __restrict__ D, int64_t ldd, const uint16_t* __restrict__ bias, int tiles_m, int tiles_n, int act) {
+    uint16_t* __restrict__ D, int64_t ldd, int tiles_m, int tiles_n, GemmEpilogue epi) {
   using S = GemmSmem<FA, FB>;
+  const uint16_t* __restrict__ bias = epi.bias;
+  const int act = epi.act;
   constexpr int BM = S::BM, BN = S::BN;
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
 
@@ -279,6 +295,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
   const int ch = lane % kChunksPerRow;      // this lane's chunk column, the same in every pass
   const int n_lane = col0 + wn * 32 * FB + 8 * ch;
   const bool vec_ok = ((ldd & 7) == 0) && ((reinterpret_cast<uintptr_t>(D) & 15) == 0);
+  float out_max = 0.0f;
   float bias_f[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) bias_f[i] = (bias && n_lane + i < N) ? bf16_bits_to_f32(bias[n_lane + i]) : 0.0f;
@@ -314,6 +331,30 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
                                gelu_tanh_f32(__uint_as_float(w[i] & 0xFFFF0000u)));
           }
         }
+        if (epi.residual) {  // host side guarantees 16-byte aligned rows and N % 8 == 0 for this path
+          const uint4 rv = *reinterpret_cast<const uint4*>(epi.residual + (int64_t)m * epi.ldr + n_lane);
+          const uint32_t r[4] = {rv.x, rv.y, rv.z, rv.w};
+          if (epi.gate) {
+            const uint4 gv = *reinterpret_cast<const uint4*>(epi.gate + (int64_t)(m / epi.gate_rows) * epi.gate_stride + n_lane);
+            const uint32_t g[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              w[i] = pack_bf16x2(__uint_as_float(w[i] << 16) * __uint_as_float(g[i] << 16),
+                                 __uint_as_float(w[i] & 0xFFFF0000u) * __uint_as_float(g[i] & 0xFFFF0000u));
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            w[i] = pack_bf16x2(__uint_as_float(r[i] << 16) + __uint_as_float(w[i] << 16),
+                               __uint_as_float(r[i] & 0xFFFF0000u) + __uint_as_float(w[i] & 0xFFFF0000u));
+        }
+        if (epi.sink.parts) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const bool lo_ok = n_lane + 2 * i < N, hi_ok = n_lane + 2 * i + 1 < N;
+            if (lo_ok) out_max = fmaxf(out_max, fabsf(__uint_as_float(w[i] << 16)));
+            if (hi_ok) out_max = fmaxf(out_max, fabsf(__uint_as_float(w[i] & 0xFFFF0000u)));
+          }
+        }
         uint16_t* dst = D + (int64_t)m * ldd + n_lane;
         if (vec_ok && n_lane + 8 <= N) {
           *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
@@ -324,12 +365,16 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
     }
     __builtin_amdgcn_wave_barrier();
   }
+  if (epi.sink.parts) {  // one atomic per wave
+    out_max = wave_max(out_max);
+    if (lane == 0) amax_sink_update(epi.sink, blockIdx.x * 4 + wave, out_max);
+  }
 }
 
 template <int FA, int FB>
 int launch_gemm(const uint8_t* Av, const uint8_t* As, const uint8_t* Bv, const uint8_t* Bs, const float* alpha,
                 const float* amax_a, const float* amax_b, float denom_a, float denom_b, int M, int N, int Mp, int Np,
-                int Kp, void* D, int64_t ldd, const void* bias, int act, hipStream_t stream) {
+                int Kp, void* D, int64_t ldd, const GemmEpilogue& epi, hipStream_t stream) {
   using S = GemmSmem<FA, FB>;
   const int tiles_m = (M + S::BM - 1) / S::BM, tiles_n = (N + S::BN - 1) / S::BN;
   const size_t smem = 2 * S::kStage;
@@ -345,7 +390,7 @@ int launch_gemm(const uint8_t* Av, const uint8_t* As, const uint8_t* Bv, const u
   }
   hipLaunchKernelGGL((gemm_w4a4_kernel<FA, FB>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kGemmThreads), smem, stream,
                      Av, As, Bv, Bs, alpha, amax_a, amax_b, 1.0f / denom_a, 1.0f / denom_b, M, N, Mp, Np, Kp,
-                     static_cast<uint16_t*>(D), ldd, static_cast<const uint16_t*>(bias), tiles_m, tiles_n, act);
+                     static_cast<uint16_t*>(D), ldd, tiles_m, tiles_n, epi);
   LL_CHECK_LAUNCH("gemm_w4a4_kernel");
   return LL_OK;
 }
@@ -365,9 +410,50 @@ extern "C" int ll_nvfp4_gemm_tnt_act(const uint8_t* A_values, const uint8_t* A_s
                                      const float* amax_b, float denom_a, float denom_b, int64_t M, int64_t N,
                                      int64_t Mp, int64_t Np, int64_t Kp, void* D, int64_t ldd, const void* bias,
                                      int activation, void* stream) {
+  ll_gemm_epilogue e = {};
+  e.bias = bias;
+  e.activation = activation;
+  return ll_nvfp4_gemm_tnt_fused(A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, M,
+                                 N, Mp, Np, Kp, D, ldd, &e, stream);
+}
+
+extern "C" int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A_scales, const uint8_t* B_values,
+                                       const uint8_t* B_scales, const float* alpha, const float* amax_a,
+                                       const float* amax_b, float denom_a, float denom_b, int64_t M, int64_t N,
+                                       int64_t Mp, int64_t Np, int64_t Kp, void* D, int64_t ldd,
+                                       const ll_gemm_epilogue* epilogue, void* stream) {
   using namespace ll;
+  LL_REQUIRE(epilogue, "ll_nvfp4_gemm_tnt_fused: null epilogue");
+  const int activation = epilogue->activation;
+  const void* bias = epilogue->bias;
   LL_REQUIRE(activation == LL_ACT_NONE || activation == LL_ACT_GELU_TANH, "ll_nvfp4_gemm_tnt: unknown activation %d",
              activation);
+  GemmEpilogue epi{};
+  epi.bias = static_cast<const uint16_t*>(bias);
+  epi.act = activation;
+  if (epilogue->amax_sink.parts) {
+    LL_REQUIRE((reinterpret_cast<uintptr_t>(epilogue->amax_sink.parts) & 7) == 0 && epilogue->amax_sink.epoch != 0,
+               "ll_nvfp4_gemm_tnt_fused: amax sink needs 8-byte alignment and a non-zero epoch");
+    epi.sink.parts = reinterpret_cast<unsigned long long*>(epilogue->amax_sink.parts);
+    epi.sink.epoch = epilogue->amax_sink.epoch;
+  }
+  if (epilogue->residual) {
+    LL_REQUIRE(N % 8 == 0 && epilogue->ldr % 8 == 0 && epilogue->ldr >= N &&
+                   (reinterpret_cast<uintptr_t>(epilogue->residual) & 15) == 0,
+               "ll_nvfp4_gemm_tnt_fused: residual needs N %% 8 == 0, ldr %% 8 == 0 and 16-byte alignment");
+    epi.residual = static_cast<const uint16_t*>(epilogue->residual);
+    epi.ldr = epilogue->ldr;
+    if (epilogue->gate) {
+      LL_REQUIRE(epilogue->gate_rows > 0 && epilogue->gate_rows < (1ll << 31) && epilogue->gate_stride % 8 == 0 &&
+                     (reinterpret_cast<uintptr_t>(epilogue->gate) & 15) == 0,
+                 "ll_nvfp4_gemm_tnt_fused: gate needs gate_rows > 0, gate_stride %% 8 == 0 and 16-byte alignment");
+      epi.gate = static_cast<const uint16_t*>(epilogue->gate);
+      epi.gate_rows = (int)epilogue->gate_rows;
+      epi.gate_stride = epilogue->gate_stride;
+    }
+  } else {
+    LL_REQUIRE(!epilogue->gate, "ll_nvfp4_gemm_tnt_fused: a gate needs a residual");
+  }
   LL_REQUIRE(A_values && A_scales && B_values && B_scales && D, "ll_nvfp4_gemm_tnt: null pointer");
   LL_REQUIRE(alpha || (amax_a && amax_b && denom_a > 0.f && denom_b > 0.f),
              "ll_nvfp4_gemm_tnt: pass alpha, or both amax pointers with positive denominators");
@@ -410,7 +496,7 @@ extern "C" int ll_nvfp4_gemm_tnt_act(const uint8_t* A_values, const uint8_t* A_s
     if (f >= 0 && f < 5) best = f;
   }
 #define LL_GEMM_ARGS A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, (int)M, (int)N, \
-                     (int)Mp, (int)Np, (int)Kp, D, ldd, bias, activation, s
+                     (int)Mp, (int)Np, (int)Kp, D, ldd, epi, s
   switch (best) {
     case 0: return launch_gemm<4, 2>(LL_GEMM_ARGS);
     case 1: return launch_gemm<2, 4>(LL_GEMM_ARGS);

@@ -102,4 +102,31 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// max(m, |v|) over the 8 bf16 values of a packed 16-byte group
+__device__ __forceinline__ float abs_max_bf16x8(const uint4& v, float m) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    m = fmaxf(m, fabsf(__uint_as_float(w[i] << 16)));
+    m = fmaxf(m, fabsf(__uint_as_float(w[i] & 0xFFFF0000u)));
+  }
+  return m;
+}
+// Amax sink: a kernel that writes a tensor leaves partial absolute maxima of it in LL_AMAX_PARTS 64-bit
+// slots, each holding (epoch << 32) | float bits and raised with a 64-bit atomic max.  A value of a newer
+// epoch beats every older one, so the slots never need clearing; the reader ignores slots of other epochs.
+// (The bit patterns of non-negative floats order like unsigned integers.)
+constexpr int kAmaxParts = LL_AMAX_PARTS;
+struct AmaxSink {
+  unsigned long long* parts;  // null: no sink
+  uint32_t epoch;
+};
+__device__ __forceinline__ void amax_sink_update(const AmaxSink& sink, uint32_t slot, float v) {
+  atomicMax(sink.parts + (slot & (kAmaxParts - 1)), ((unsigned long long)sink.epoch << 32) | __float_as_uint(v));
+}
+__device__ __forceinline__ float amax_sink_read(const unsigned long long* parts, uint32_t epoch, int slot) {
+  const unsigned long long v = parts[slot];
+  return (uint32_t)(v >> 32) == epoch ? __uint_as_float((uint32_t)v) : 0.0f;
+}
+
 }  // namespace ll

@@ -11,7 +11,6 @@
 
 namespace ll {
 
-constexpr int kAmaxParts = 1024;  // partial maxima written by the amax kernel
 constexpr int kThreads = 256;
 
 // ----------------------------------------------------------------------------- amax
@@ -283,7 +282,9 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
                                                             int64_t ldx, int64_t Kp, uint8_t* __restrict__ values,
                                                             uint8_t* __restrict__ scales, float* __restrict__ amax_io,
                                                             const float* __restrict__ parts, int amax_given,
-                                                            int64_t total_tiles) {
+                                                            int64_t total_tiles,
+                                                            const unsigned long long* __restrict__ sink_parts,
+                                                            uint32_t sink_epoch) {
   __shared__ float s_red[kThreads / 64];
   __shared__ float s_amax;
   __shared__ uint32_t s_scales[128];  // 512 bytes in blocked order
@@ -292,7 +293,15 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
   if (amax_given) {
     if (threadIdx.x == 0) s_amax = amax_io[0];
   } else {
-    const float4 p = reinterpret_cast<const float4*>(parts)[threadIdx.x];  // kAmaxParts == 4 * kThreads
+    float4 p;  // kAmaxParts == 4 * kThreads
+    if (sink_parts) {
+      p = make_float4(amax_sink_read(sink_parts, sink_epoch, 4 * threadIdx.x),
+                      amax_sink_read(sink_parts, sink_epoch, 4 * threadIdx.x + 1),
+                      amax_sink_read(sink_parts, sink_epoch, 4 * threadIdx.x + 2),
+                      amax_sink_read(sink_parts, sink_epoch, 4 * threadIdx.x + 3));
+    } else {
+      p = reinterpret_cast<const float4*>(parts)[threadIdx.x];
+    }
     float m = wave_max(fmaxf(fmaxf(p.x, p.y), fmaxf(p.z, p.w)));
     if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = m;
     __syncthreads();
@@ -384,14 +393,16 @@ __global__ void debug_convert_kernel(const float* __restrict__ in, int64_t n, in
 
 extern "C" size_t ll_nvfp4_quantize_workspace_floats(void) { return ll::kAmaxParts; }
 
-extern "C" int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ldx, int rule, uint8_t* values,
-                                 uint8_t* scales, float* amax, int amax_given, float* workspace, void* stream) {
+static int quantize_impl(const void* x, int64_t M, int64_t K, int64_t ldx, int rule, uint8_t* values, uint8_t* scales,
+                         float* amax, int amax_given, float* workspace, const ll_amax_sink* sink, void* stream) {
   using namespace ll;
   LL_REQUIRE(x && values && scales && amax, "ll_nvfp4_quantize: null pointer");
   LL_REQUIRE(M > 0 && K > 0 && ldx >= K, "ll_nvfp4_quantize: bad shape M=%lld K=%lld ldx=%lld", (long long)M,
              (long long)K, (long long)ldx);
   LL_REQUIRE(rule >= 0 && rule <= 4, "ll_nvfp4_quantize: unknown scale rule %d", rule);
-  LL_REQUIRE(amax_given || workspace, "ll_nvfp4_quantize: workspace required to compute amax");
+  LL_REQUIRE(amax_given || workspace || sink, "ll_nvfp4_quantize: workspace required to compute amax");
+  LL_REQUIRE(!sink || (sink->parts && (reinterpret_cast<uintptr_t>(sink->parts) & 7) == 0 && sink->epoch != 0),
+             "ll_nvfp4_quantize_from_sink: amax sink needs an 8-byte aligned buffer and a non-zero epoch");
   LL_REQUIRE((reinterpret_cast<uintptr_t>(values) & 7) == 0 && (reinterpret_cast<uintptr_t>(scales) & 3) == 0,
              "ll_nvfp4_quantize: outputs must be 8-byte (values) / 4-byte (scales) aligned");
   const int64_t Mp = round_up(M, 128), Kp = round_up(K, 64);
@@ -399,17 +410,19 @@ extern "C" int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ld
   LL_REQUIRE(total_tiles < (1ll << 31), "ll_nvfp4_quantize: tensor too large for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const uint16_t* xp = static_cast<const uint16_t*>(x);
-  if (!amax_given) {
+  if (!amax_given && !sink) {
     hipLaunchKernelGGL(amax_partial_kernel, dim3(kAmaxParts), dim3(kThreads), 0, s, xp, M, K, ldx, workspace);
     LL_CHECK_LAUNCH("amax_partial_kernel");
   }
+  const unsigned long long* sink_parts = sink ? reinterpret_cast<const unsigned long long*>(sink->parts) : nullptr;
+  const uint32_t sink_epoch = sink ? sink->epoch : 0u;
   // one workgroup per tile up to what the chip holds at once (256 CUs x 8 for the static rules,
   // x 4 for the rules that evaluate two candidates and need twice the registers)
   const int64_t resident = (rule == LL_RULE_STATIC_6 || rule == LL_RULE_STATIC_4) ? 2048 : 1024;
   const dim3 grid((unsigned)(total_tiles < resident ? total_tiles : resident));
 #define LL_LAUNCH_Q(R)                                                                                          \
   hipLaunchKernelGGL(quantize_kernel<R>, grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales, amax, \
-                     workspace, amax_given, total_tiles)
+                     workspace, amax_given, total_tiles, sink_parts, sink_epoch)
   switch (rule) {
     case LL_RULE_STATIC_6: LL_LAUNCH_Q(LL_RULE_STATIC_6); break;
     case LL_RULE_STATIC_4: LL_LAUNCH_Q(LL_RULE_STATIC_4); break;
@@ -420,6 +433,19 @@ extern "C" int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ld
 #undef LL_LAUNCH_Q
   LL_CHECK_LAUNCH("quantize_kernel");
   return LL_OK;
+}
+
+extern "C" int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ldx, int rule, uint8_t* values,
+                                 uint8_t* scales, float* amax, int amax_given, float* workspace, void* stream) {
+  return quantize_impl(x, M, K, ldx, rule, values, scales, amax, amax_given, workspace, nullptr, stream);
+}
+
+extern "C" int ll_nvfp4_quantize_from_sink(const void* x, int64_t M, int64_t K, int64_t ldx, int rule,
+                                           uint8_t* values, uint8_t* scales, float* amax,
+                                           const ll_amax_sink* amax_sink, void* stream) {
+  using namespace ll;
+  LL_REQUIRE(amax_sink, "ll_nvfp4_quantize_from_sink: null amax sink");
+  return quantize_impl(x, M, K, ldx, rule, values, scales, amax, 0, nullptr, amax_sink, stream);
 }
 
 extern "C" int ll_debug_convert(const float* in, int64_t n, int mode, uint8_t* out, void* stream) {

@@ -63,15 +63,52 @@ class WanLayerNorm(nn.LayerNorm):
         return super().forward(x).type_as(x)
 
 
-def _project_shared(x: torch.Tensor, layers) -> list[torch.Tensor]:
+def _project_shared(x: torch.Tensor, layers, amax: torch.Tensor | None = None) -> list[torch.Tensor]:
     """Apply several linear layers to the same input.  Quantized layers with the same activation config
-    share one quantized operand (bit-identical to quantizing per layer, as the reference does)."""
+    share one quantized operand (bit-identical to quantizing per layer, as the reference does).  ``amax`` is
+    the amax ticket that the kernel which produced ``x`` was given."""
     first = layers[0]
     if all(isinstance(m, FourOverSixLinear) for m in layers) and all(
             m.config.get_activation_config() == first.config.get_activation_config() for m in layers):
-        xq = first.quantize_input(x.reshape(-1, x.shape[-1]))
+        xq = first.quantize_input(x.reshape(-1, x.shape[-1]), amax=amax)
         return [m.forward_quantized(xq).reshape(*x.shape[:-1], -1) for m in layers]
     return [m(x) for m in layers]
+
+
+def _fused_linear(layer, x: torch.Tensor, *, amax: torch.Tensor | None = None, activation: str | None = None,
+                  residual: torch.Tensor | None = None, gate: torch.Tensor | None = None, gate_rows: int = 0,
+                  amax_out: torch.Tensor | None = None) -> torch.Tensor | None:
+    """``layer(x)`` of a quantized layer with the GEMM epilogue extensions (``residual + y * gate`` etc.);
+    ``None`` when the layer is not quantized or the shapes rule the fused epilogue out, so that the caller
+    runs the separate operations."""
+    if not isinstance(layer, FourOverSixLinear) or layer.out_features % 8 != 0:
+        return None
+    x2d = x.reshape(-1, x.shape[-1])
+    if residual is not None:
+        residual = residual.reshape(-1, residual.shape[-1])
+        if residual.data_ptr() % 16 or residual.stride(0) % 8 or (gate is not None and (
+                gate.data_ptr() % 16 or gate.stride(0) % 8)):
+            return None
+    out = layer.forward_quantized(layer.quantize_input(x2d, amax=amax), activation, residual=residual, gate=gate,
+                                  gate_rows=gate_rows, amax_out=amax_out)
+    return out.reshape(*x.shape[:-1], -1)
+
+
+def _project_out(layer, y: torch.Tensor, amax, residual, gate, gate_rows: int) -> torch.Tensor:
+    """``layer(y)``, or ``residual + layer(y) * gate`` (gate [G, C], row ``m // gate_rows``; plain sum without a
+    gate) when a residual is given: in the GEMM epilogue for a quantized layer, else as separate operations
+    with the same roundings."""
+    if residual is None:
+        out = _fused_linear(layer, y, amax=amax)
+        return layer(y) if out is None else out
+    out = _fused_linear(layer, y, amax=amax, residual=residual, gate=gate, gate_rows=gate_rows)
+    if out is not None:
+        return out
+    out = layer(y)
+    if gate is None:
+        return residual + out
+    b, l, c = residual.shape
+    return gate_residual(residual, out.contiguous(), gate.view(b, -1, 1, c), gate_rows)
 
 
 class CausalSelfAttention(nn.Module):
@@ -81,10 +118,14 @@ class CausalSelfAttention(nn.Module):
         self.q, self.k, self.v, self.o = (nn.Linear(dim, dim) for _ in range(4))
         self.norm_q, self.norm_k = WanRMSNorm(dim, eps), WanRMSNorm(dim, eps)
 
-    def forward(self, x, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size):
+    def forward(self, x, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size, *, input_amax=None,
+                residual=None, gate=None, gate_rows=0):
+        """``input_amax``: the amax ticket the producer of ``x`` was given, if any.
+        ``residual`` [B, L, C] (with ``gate`` [B*F, C], ``gate_rows`` tokens per gate row) turns the result into
+        ``residual + out * gate``, folded into the output projection."""
         b, s = x.shape[:2]
         n, d = self.num_heads, self.head_dim
-        q, k, v = _project_shared(x, [self.q, self.k, self.v])
+        q, k, v = _project_shared(x, [self.q, self.k, self.v], amax=input_amax)
         v = v.view(b, s, n, d)
         if b == 1 and d == 128:
             # RMSNorm -> RoPE (-> K smoothing) of the reference in one pass per tensor
@@ -98,9 +139,11 @@ class CausalSelfAttention(nn.Module):
             roped_q = rope_apply(q[0], cos, sin).unsqueeze(0)
             roped_k = rope_apply(k[0], cos, sin).unsqueeze(0)
             smooth_k = None
+        out_amax = _native.amax_ticket(x.device) if isinstance(self.o, FourOverSixLinear) else None
         out, update = kvc.kv_cache_attention(roped_q, roped_k, v, kv_cache, current_start, sink_tokens,
-                                             max_attention_size=max_attention_size, smoothed_key=smooth_k)
-        return self.o(out.flatten(2)), update
+                                             max_attention_size=max_attention_size, smoothed_key=smooth_k,
+                                             amax_out=out_amax)
+        return _project_out(self.o, out.flatten(2), out_amax, residual, gate, gate_rows), update
 
 
 class CrossAttention(nn.Module):
@@ -110,8 +153,9 @@ class CrossAttention(nn.Module):
         self.q, self.k, self.v, self.o = (nn.Linear(dim, dim) for _ in range(4))
         self.norm_q, self.norm_k = WanRMSNorm(dim, eps), WanRMSNorm(dim, eps)
 
-    def forward(self, x, context, crossattn_cache: dict | None = None):
-        """``crossattn_cache`` ({"is_init": bool, "k": ..., "v": ...}, the reference's interface,
+    def forward(self, x, context, crossattn_cache: dict | None = None, *, residual=None):
+        """``residual`` [B, L, C] turns the result into ``residual + out`` (folded into the output projection).
+        ``crossattn_cache`` ({"is_init": bool, "k": ..., "v": ...}, the reference's interface,
         wan_5b/modules/causal_model.py:199-206) keeps the projected K / V of a prompt's text context between
         calls; the reference has the argument but recomputes on every call (:229-235), which gives the same
         tensors.  Without a cache K / V are recomputed here too."""
@@ -125,8 +169,10 @@ class CrossAttention(nn.Module):
             v = v.view(b, -1, n, d)
             if crossattn_cache is not None:
                 crossattn_cache.update(is_init=True, k=k, v=v)
-        out = _native.attention_bf16(q[0].contiguous(), k[0].contiguous(), v[0].contiguous(), d ** -0.5)
-        return self.o(out.unsqueeze(0).flatten(2))
+        out_amax = _native.amax_ticket(x.device) if isinstance(self.o, FourOverSixLinear) else None
+        out = _native.attention_bf16(q[0].contiguous(), k[0].contiguous(), v[0].contiguous(), d ** -0.5,
+                                     amax_out=out_amax)
+        return _project_out(self.o, out.unsqueeze(0).flatten(2), out_amax, residual, None, 0)
 
 
 class DiTBlock(nn.Module):
@@ -141,25 +187,35 @@ class DiTBlock(nn.Module):
         self.ffn = nn.Sequential(nn.Linear(dim, ffn_dim), nn.GELU(approximate="tanh"), nn.Linear(ffn_dim, dim))
         self.modulation = nn.Parameter(torch.randn(1, 6, dim) / dim ** 0.5)
 
-    def _feed_forward(self, y: torch.Tensor) -> torch.Tensor:
-        """Linear -> GELU(tanh) -> Linear; with a quantized first layer the GELU runs in its GEMM epilogue."""
+    def _feed_forward(self, y, y_amax, residual, gate, gate_rows: int) -> torch.Tensor:
+        """``residual + ffn(y) * gate`` with ffn = Linear -> GELU(tanh) -> Linear.  With quantized layers the
+        GELU runs in the first GEMM's epilogue (which also yields the amax of its result) and the gated
+        residual in the second's."""
         up, act, down = self.ffn
         if isinstance(up, FourOverSixLinear) and getattr(act, "approximate", None) == "tanh":
-            h = up.forward_quantized(up.quantize_input(y.reshape(-1, y.shape[-1])), activation="gelu_tanh")
-            return down(h.reshape(*y.shape[:-1], -1))
-        return self.ffn(y)
+            h_amax = _native.amax_ticket(y.device) if isinstance(down, FourOverSixLinear) else None
+            h = up.forward_quantized(up.quantize_input(y.reshape(-1, y.shape[-1]), amax=y_amax),
+                                     activation="gelu_tanh", amax_out=h_amax).reshape(*y.shape[:-1], -1)
+        else:
+            h, h_amax = act(up(y)), None
+        return _project_out(down, h, h_amax, residual, gate, gate_rows)
 
     def forward(self, x, e, cos, sin, context, kv_cache, current_start, sink_tokens, max_attention_size=None,
                 crossattn_cache=None):
-        """x [1, L, C]; e [1, F, 6, C]; returns (x, (current_end, local_end_index, cache_update_info))."""
+        """x [1, L, C]; e [1, F, 6, C]; returns (x, (current_end, local_end_index, cache_update_info)).
+        The tensor amax that each activation quantization needs is produced by the kernel that writes the
+        activation wherever that kernel is one of this package's."""
         num_frames, frame_seqlen = e.shape[1], x.shape[1] // e.shape[1]
         e = (self.modulation.unsqueeze(1) + e).chunk(6, dim=2)
-        y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.eps)
-        y, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size)
-        x = gate_residual(x, y.contiguous(), e[2], frame_seqlen)
-        x = x + self.cross_attn(self.norm3(x), context, crossattn_cache)
-        y = self._feed_forward(adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps))
-        x = gate_residual(x, y.contiguous(), e[5], frame_seqlen)
+        gates = [g.reshape(-1, g.shape[-1]) for g in (e[2], e[5])]  # [B*F, C] views, one row per frame
+        y_amax = _native.amax_ticket(x.device) if isinstance(self.self_attn.q, FourOverSixLinear) else None
+        y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.eps, amax_out=y_amax)
+        x, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size,
+                                   input_amax=y_amax, residual=x, gate=gates[0], gate_rows=frame_seqlen)
+        x = self.cross_attn(self.norm3(x), context, crossattn_cache, residual=x)
+        y_amax = _native.amax_ticket(x.device) if isinstance(self.ffn[0], FourOverSixLinear) else None
+        y = adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps, amax_out=y_amax)
+        x = self._feed_forward(y, y_amax, x, gates[1], frame_seqlen)
         return x, update
 
 

@@ -18,6 +18,10 @@ def fp4_matmul(
     out_dtype: DataType = DataType.bfloat16,
     bias: torch.Tensor | None = None,
     activation: str | None = None,
+    residual: torch.Tensor | None = None,
+    gate: torch.Tensor | None = None,
+    gate_rows: int = 0,
+    amax_out=None,
 ) -> torch.Tensor:
     """``input @ other.T`` of two NVFP4 tensors with fp32 accumulation (W4A4 GEMM).
 
@@ -25,6 +29,10 @@ def fp4_matmul(
     ``backend`` is accepted for compatibility; the gfx950 kernel always runs.  ``bias`` (bfloat16
     [N], an extension) is added to the bfloat16 result inside the kernel epilogue; ``activation``
     (``"gelu_tanh"``, an extension) is then applied to that bfloat16 value, also in the epilogue.
+    ``residual`` (bfloat16 [M, N]) with an optional ``gate`` (bfloat16 [G, N], row ``m // gate_rows``)
+    makes the result ``residual + y * gate`` (each step rounded to bfloat16 like the separate
+    operations); ``amax_out`` (an amax ticket, ``_native.amax_ticket``) receives the absolute maximum of
+    the result.  All of these are extensions.
     """
     if isinstance(backend, str):
         backend = MatmulBackend(backend)
@@ -50,4 +58,8 @@ def fp4_matmul(
         denom_b=float(other.scale_rule.max_allowed_e2m1_value() * other.scale_rule.max_allowed_e4m3_value()),
         bias=bias,
         activation=activation,
+        residual=residual,
+        gate=gate,
+        gate_rows=gate_rows,
+        amax_out=amax_out,
     )

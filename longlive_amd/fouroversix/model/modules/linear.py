@@ -100,17 +100,22 @@ class FourOverSixLinear(nn.Linear):
     def _forward_2d(self, x2d: torch.Tensor) -> torch.Tensor:
         return self.forward_quantized(self.quantize_input(x2d))
 
-    def quantize_input(self, x2d: torch.Tensor) -> QuantizedTensor:
-        """The activation operand exactly as ``forward`` would build it from a 2-D input."""
-        return quantize_to_fp4(x2d, self.config.get_activation_config())
+    def quantize_input(self, x2d: torch.Tensor, amax=None) -> QuantizedTensor:
+        """The activation operand exactly as ``forward`` would build it from a 2-D input.  ``amax`` is
+        the amax ticket of the kernel that produced ``x2d``, if it was given one."""
+        return quantize_to_fp4(x2d, self.config.get_activation_config(), amax=amax)
 
-    def forward_quantized(self, xq: QuantizedTensor, activation: str | None = None) -> torch.Tensor:
+    def forward_quantized(self, xq: QuantizedTensor, activation: str | None = None, *,
+                          residual: torch.Tensor | None = None, gate: torch.Tensor | None = None,
+                          gate_rows: int = 0, amax_out=None) -> torch.Tensor:
         """``forward`` for an input already quantized with :meth:`quantize_input`.  Several layers that read
         the same tensor with the same activation config (the q / k / v projections) share one quantized
-        operand this way; each would otherwise compute the identical bytes again.  ``activation`` ("gelu_tanh")
-        is applied to the bfloat16 result in the GEMM epilogue.  Returns [M, out_features]."""
+        operand this way; each would otherwise compute the identical bytes again.  The keyword arguments are
+        the epilogue extensions of :func:`fp4_matmul` (activation, gated residual, amax of the result).
+        Returns [M, out_features]."""
         weight = self.quantized_weight()
         if not isinstance(weight, QuantizedTensor):
             weight = quantize_to_fp4(weight.data, self.config.get_weight_config())
         return fp4_matmul(xq, weight, backend=self.config.matmul_backend, out_dtype=self.config.output_dtype,
-                          bias=self.bias, activation=activation)
+                          bias=self.bias, activation=activation, residual=residual, gate=gate, gate_rows=gate_rows,
+                          amax_out=amax_out)

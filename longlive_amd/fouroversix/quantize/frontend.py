@@ -29,12 +29,14 @@ def _unsupported(x: torch.Tensor, config: QuantizationConfig) -> str | None:
     return None
 
 
-def quantize_to_fp4(x: torch.Tensor, config: QuantizationConfig | None = None) -> QuantizedTensor:
+def quantize_to_fp4(x: torch.Tensor, config: QuantizationConfig | None = None, *,
+                    amax=None) -> QuantizedTensor:
     """Quantize a 2-D bfloat16 GPU tensor to NVFP4.
 
     Default configuration: block 16 along the last axis, e4m3 block scales, fp32 tensor amax,
     round-to-nearest, four-over-six selection with the mse rule.  The packed bytes equal those of
-    the reference's PyTorch back end.
+    the reference's PyTorch back end.  ``amax`` (an extension) is the amax ticket (``_native.amax_ticket``)
+    that the kernel which produced ``x`` was given; the reduction pass over ``x`` is then skipped.
     """
     if config is None:
         config = QuantizationConfig()
@@ -42,6 +44,6 @@ def quantize_to_fp4(x: torch.Tensor, config: QuantizationConfig | None = None) -
     if why is not None:
         backend = config.backend.value if config.backend is not None else "hip"
         raise ValueError(f"Backend {backend} does not support the given parameters: {why}")
-    values, scales, amax = _native.quantize(x, config.scale_rule.value)
+    values, scales, amax = _native.quantize(x, config.scale_rule.value, amax=amax)
     return QuantizedTensor(values, scales, amax, config.dtype, tuple(x.shape), config.scale_rule,
                            _native.padded_shape(tuple(x.shape)))

@@ -7,10 +7,12 @@ from .. import _native
 
 
 def adaln_modulate(x: torch.Tensor, e_scale: torch.Tensor, e_shift: torch.Tensor, frame_seqlen: int,
-                   eps: float = 1e-6, add_one_to_scale: bool = True) -> torch.Tensor:
+                   eps: float = 1e-6, add_one_to_scale: bool = True,
+                   amax_out=None) -> torch.Tensor:
     """``LayerNorm(x) * (1 + e_scale) + e_shift`` over x [B, F*frame_seqlen, C] with per-frame
-    e_scale / e_shift [B, F, 1, C]; bf16 roundings placed as in the eager graph."""
-    return _native.adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps, add_one_to_scale)
+    e_scale / e_shift [B, F, 1, C]; bf16 roundings placed as in the eager graph.  ``amax_out``
+    (an amax ticket, ``_native.amax_ticket``; an extension) receives the absolute maximum of the result."""
+    return _native.adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps, add_one_to_scale, amax_out=amax_out)
 
 
 adaln_modulate_triton = adaln_modulate

@@ -104,7 +104,8 @@ def plan_cache_step(cache: dict, current_start: int, num_new_tokens: int, sink_t
 
 def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Tensor, cache: dict,
                        current_start: int, sink_tokens: int, softmax_scale: float | None = None,
-                       max_attention_size: int | None = None, smoothed_key: torch.Tensor | None = None):
+                       max_attention_size: int | None = None, smoothed_key: torch.Tensor | None = None,
+                       amax_out=None):
     """Self-attention of one chunk against the FP4 cache.
 
     q, key_to_cache (RoPE'd, un-smoothed), v: bf16 [1, S, H, 128].  Attends
@@ -112,7 +113,8 @@ def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Ten
     ``(out [1, S, H, 128], (current_end, local_end_index, cache_update_info))`` exactly like the
     reference's attention module, with ``new_k`` / ``new_v`` = the un-smoothed chunk to be written.
     ``smoothed_key`` = k_smooth(key_to_cache) [1, S, H, 128] when the caller has it already (the fused
-    norm + RoPE kernel produces it as a second output).
+    norm + RoPE kernel produces it as a second output).  ``amax_out`` (an amax ticket, ``_native.amax_ticket``)
+    receives the absolute maximum of ``out``.
     """
     if q.shape[0] != 1:
         raise ValueError("the quantized KV cache holds one sequence (batch size 1)")
@@ -129,7 +131,7 @@ def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Ten
         tables = None
     out = _native.kv_attention(q[0].contiguous(), tables, len(slot_ids) * cache["block_token_size"],
                                cache["block_token_size"], rule.max_allowed_e2m1_value(),
-                               rule.max_allowed_e4m3_value(), k_new, v[0], scale)
+                               rule.max_allowed_e4m3_value(), k_new, v[0], scale, amax_out=amax_out)
     return out.unsqueeze(0), (current_start + S, local_end, info)
 
 

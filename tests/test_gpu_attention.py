@@ -254,3 +254,29 @@ def test_fused_norm_rope_equals_the_separate_kernels(gpu):
     part = _native.qk_norm_rope(x, w, 1e-6, cos[:64], sin[:64], H, seq_len=64)
     assert torch.equal(part[:64], want[:64])
     assert torch.equal(part[64:], _native.rms_norm(x, w, 1e-6).view(S, H, 128)[64:])
+
+
+def test_amax_sink_of_adaln_and_attention_feeds_the_next_quantization(gpu):
+    """adaLN and attention leave the absolute maximum of their result in the amax sink; the quantization that
+    reads it produces the bytes of a quantization that reduces the tensor itself, also when earlier uses of
+    the sink saw larger values."""
+    L, C, fs, H = 264, 768, 88, 6
+    F = L // fs
+    sc, sh = _randn((1, F, 1, C), 61).to(gpu), _randn((1, F, 1, C), 62).to(gpu)
+    for scale in (50.0, 1.0, 0.02):
+        x = _randn((1, L, C), 63, scale).to(gpu)
+        ticket = _native.amax_ticket(gpu)
+        y = adaln_modulate(x, sc, sh * scale, fs, amax_out=ticket)
+        assert torch.equal(y, adaln_modulate(x, sc, sh * scale, fs))
+        a, b = quantize_to_fp4(y[0], CFG, amax=ticket), quantize_to_fp4(y[0], CFG)
+        assert float(b.amax) == float(y.abs().max()) and torch.equal(a.amax, b.amax)
+        assert torch.equal(a.values, b.values) and np.array_equal(u8(a.scale_factors), u8(b.scale_factors))
+
+        q, k = _randn((L, H, 128), 64).to(gpu), _randn((200, H, 128), 65).to(gpu)
+        v = _randn((200, H, 128), 66, scale).to(gpu)
+        ticket = _native.amax_ticket(gpu)
+        out = _native.attention_bf16(q, k, v, 128 ** -0.5, amax_out=ticket)
+        assert torch.equal(out, _native.attention_bf16(q, k, v, 128 ** -0.5))
+        a, b = quantize_to_fp4(out.flatten(1), CFG, amax=ticket), quantize_to_fp4(out.flatten(1), CFG)
+        assert float(b.amax) == float(out.abs().max()) and torch.equal(a.amax, b.amax)
+        assert torch.equal(a.values, b.values) and np.array_equal(u8(a.scale_factors), u8(b.scale_factors))

@@ -168,3 +168,53 @@ def test_gelu_epilogue_matches_separate_gelu(gpu):
     assert np.abs(fused.float().cpu().numpy() - ref).max() <= 2 ** -8 * max(1.0, np.abs(ref).max())
     with pytest.raises(ValueError):
         fp4_matmul(xq, wq, activation="relu")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M,N,K,frame", [(264, 384, 256, 88), (300, 640, 512, 100), (64, 72, 128, 16)])
+def test_gated_residual_epilogue_is_bit_identical_to_the_separate_operations(gpu, M, N, K, frame):
+    """residual + y * gate and residual + y inside the GEMM epilogue against the GEMM followed by the two
+    bf16 operations of the reference (causal_model.py:889, 906), which the oracle restates."""
+    from longlive_amd.fouroversix import QuantizationConfig, fp4_matmul, quantize_to_fp4
+    cfg = QuantizationConfig(scale_rule="mse")
+    x = activations((M, K), 41).to(gpu)
+    w = weights((N, K), 42).to(gpu)
+    gen = torch.Generator().manual_seed(43)
+    bias = (torch.randn(N, generator=gen) * 0.5).bfloat16().to(gpu)
+    residual = torch.randn(M, N, generator=gen).bfloat16().to(gpu)
+    frames = M // frame
+    e = torch.randn(frames, 6, N, generator=gen).bfloat16().to(gpu)
+    gate = e[:, 2]  # rows strided by 6 N, as the chunked modulation tensor of the block hands them over
+    xq, wq = quantize_to_fp4(x, cfg), quantize_to_fp4(w, cfg)
+    plain = fp4_matmul(xq, wq, bias=bias)
+    fused = fp4_matmul(xq, wq, bias=bias, residual=residual, gate=gate, gate_rows=frame)
+    want = o.gate_residual(residual.float().cpu().numpy(), plain.float().cpu().numpy(), gate.float().cpu().numpy(),
+                           frame)
+    assert np.array_equal(fused.float().cpu().numpy(), want)
+    assert torch.equal(fused, residual + (plain.view(frames, frame, N) * gate[:, None]).view(M, N))
+    summed = fp4_matmul(xq, wq, bias=bias, residual=residual)
+    assert torch.equal(summed, residual + plain)
+    with pytest.raises(ValueError):
+        fp4_matmul(xq, wq, gate=gate, gate_rows=frame)
+
+
+@pytest.mark.gpu
+def test_amax_sink_of_the_epilogue_feeds_the_next_quantization(gpu):
+    """The absolute maximum a GEMM leaves in the amax sink makes the following quantization produce the bytes
+    of a quantization that reduces the tensor itself; a later use of the sink with smaller values is not
+    disturbed by what earlier epochs left there."""
+    from longlive_amd import _native
+    from longlive_amd.fouroversix import QuantizationConfig, fp4_matmul, quantize_to_fp4
+    cfg = QuantizationConfig(scale_rule="mse")
+    x = activations((300, 512), 51).to(gpu)
+    wq = quantize_to_fp4(weights((640, 512), 52).to(gpu), cfg)
+    for scale in (8.0, 1.0, 0.01):  # decreasing maxima: stale slots of older epochs hold larger values
+        xq = quantize_to_fp4(x * scale, cfg)
+        for act in (None, "gelu_tanh"):
+            ticket = _native.amax_ticket(gpu)
+            y = fp4_matmul(xq, wq, activation=act, amax_out=ticket)
+            via_sink = quantize_to_fp4(y, cfg, amax=ticket)
+            direct = quantize_to_fp4(y, cfg)
+            assert torch.equal(via_sink.amax, direct.amax) and float(direct.amax) == float(y.abs().max())
+            assert torch.equal(via_sink.values, direct.values)
+            assert torch.equal(via_sink.scale_factors.view(torch.uint8), direct.scale_factors.view(torch.uint8))

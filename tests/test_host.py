@@ -29,6 +29,17 @@ def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
     assert lib.ll_nvfp4_gemm_tnt(None, None, None, None, None, None, None, 1.0, 1.0, 1, 1, 128, 128, 64, None, 1,
                                  None, None) == -1
     assert lib.ll_rope_apply(None, 1, 1, 16, 16, 16, None, None, 1, None, None) == -1
+    assert lib.ll_nvfp4_gemm_tnt_fused(None, None, None, None, None, None, None, 1.0, 1.0, 1, 1, 128, 128, 64, None,
+                                       1, None, None) == -1
+    assert b"null epilogue" in lib.ll_last_error()
+    assert lib.ll_nvfp4_quantize_from_sink(None, 1, 1, 1, 3, None, None, None, None, None) == -1
+    assert b"null amax sink" in lib.ll_last_error()
+    import ctypes
+    gated = _native.GemmEpilogue(None, 0, 1 << 20, 4, 8, None, 0, _native.AmaxSinkStruct(None, 0))
+    assert lib.ll_nvfp4_gemm_tnt_fused(None, None, None, None, None, None, None, 1.0, 1.0, 1, 1, 128, 128, 64, None,
+                                       1, ctypes.byref(gated), None) == -1
+    assert b"a gate needs a residual" in lib.ll_last_error()
+    assert ctypes.sizeof(_native.GemmEpilogue) == 72 and ctypes.sizeof(_native.AmaxSinkStruct) == 16
 
 
 def test_scale_rule_tables():
