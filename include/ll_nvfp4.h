@@ -227,6 +227,12 @@ int ll_rms_norm(const void* x, int64_t rows, int C, const void* weight, float ep
 int ll_qk_norm_rope(const void* x, int64_t rows, int num_heads, const void* weight, float eps, const float* cos,
                     const float* sin, int64_t seq_len, void* out, void* out_smooth, void* stream);
 
+/* ll_qk_norm_rope for q and k of one attention layer in a single launch (same rows, heads, eps and angles;
+ * one weight each); k_out_smooth may be NULL. */
+int ll_qk_norm_rope_pair(const void* q, const void* k, int64_t rows, int num_heads, const void* q_weight,
+                         const void* k_weight, float eps, const float* cos, const float* sin, int64_t seq_len,
+                         void* q_out, void* k_out, void* k_out_smooth, void* stream);
+
 /* Test hooks: hardware fp32->e4m3 / fp32->e2m1 conversions applied to n floats (used by the GPU tests to
  * check the instructions the fast paths rely on against the software codecs). mode 0: e4m3, 1: e2m1. */
 int ll_debug_convert(const float* in, int64_t n, int mode, uint8_t* out, void* stream);

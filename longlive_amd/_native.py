@@ -59,6 +59,8 @@ _SIGNATURES = {
                                        c_int64, c_int64, c_int64, c_float, c_int, c_void_p, c_void_p, c_void_p]),
     "ll_qk_norm_rope": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p, c_int64, c_void_p,
                                 c_void_p, c_void_p]),
+    "ll_qk_norm_rope_pair": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_float, c_void_p,
+                                     c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ll_gate_residual": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_int64, c_int64,
                                  c_void_p, c_void_p]),
     "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
@@ -363,6 +365,35 @@ def qk_norm_rope(x, weight, eps, cos, sin, num_heads, seq_len=None, smooth=False
                                       cos.data_ptr(), sin.data_ptr(), seq_len, out.data_ptr(), _ptr(out_s), _stream())
     _check(code, "ll_qk_norm_rope")
     return (out, out_s) if smooth else out
+
+
+def qk_norm_rope_pair(q, k, q_weight, k_weight, eps, cos, sin, num_heads, seq_len=None):
+    """:func:`qk_norm_rope` of q and of k (with the smoothed second output) in one launch:
+    returns (roped_q, roped_k, smoothed_k), each bf16 [S, num_heads, 128]."""
+    _require_cuda(q, k, q_weight, k_weight, cos, sin)
+    for x in (q, k):
+        if x.ndim != 2 or x.dtype != torch.bfloat16 or not x.is_contiguous() or x.shape[1] != num_heads * 128:
+            raise ValueError("q and k must be contiguous bfloat16 [S, num_heads * 128] tensors")
+    if q.shape != k.shape:
+        raise ValueError("q and k must have the same shape")
+    for w in (q_weight, k_weight):
+        if w.dtype != torch.bfloat16 or w.numel() != q.shape[1]:
+            raise ValueError("weights must be bfloat16 with one entry per channel")
+    S = q.shape[0]
+    seq_len = S if seq_len is None else seq_len
+    if cos.shape != (seq_len, 64) or sin.shape != cos.shape or cos.dtype != torch.float32:
+        raise ValueError(f"cos/sin must be float32 [{seq_len}, 64]")
+    cos = cos.contiguous()
+    sin = sin.contiguous()
+    out_q = torch.empty((S, num_heads, 128), dtype=q.dtype, device=q.device)
+    out_k, out_s = torch.empty_like(out_q), torch.empty_like(out_q)
+    with torch.cuda.device(q.device):
+        code = load().ll_qk_norm_rope_pair(q.data_ptr(), k.data_ptr(), S, num_heads, q_weight.contiguous().data_ptr(),
+                                           k_weight.contiguous().data_ptr(), float(eps), cos.data_ptr(),
+                                           sin.data_ptr(), seq_len, out_q.data_ptr(), out_k.data_ptr(),
+                                           out_s.data_ptr(), _stream())
+    _check(code, "ll_qk_norm_rope_pair")
+    return out_q, out_k, out_s
 
 
 def adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps=1e-6, add_one_to_scale=True, amax_out=None):

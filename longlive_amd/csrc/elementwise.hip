@@ -53,52 +53,50 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
   *reinterpret_cast<uint4*>(out + (s * N + n) * (int64_t)D + c) = o;
 }
 
-// ----------------------------------------------------------------------------- block reductions
-template <int NT>
-__device__ __forceinline__ float block_sum(float v, float* sm) {
-  v = wave_sum(v);
-  if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
-  __syncthreads();
-  float r = 0.0f;
-#pragma unroll
-  for (int i = 0; i < NT / 64; ++i) r += sm[i];
-  __syncthreads();
-  return r;
-}
-
-constexpr int kRowThreads = 128;
-constexpr int kMaxChunks = 8;  // 8 elements each: C <= 128 * 8 * 8 = 8192
+// Row kernels: one wave per row (no workgroup barrier; a row's sums are wave reductions), four rows per
+// workgroup.  A lane holds NCH groups of 8 elements: NCH = 6 covers C = 3072 exactly, 16 anything up to 8192.
+constexpr int kRowThreads = 256;
+constexpr int kRowsPerWg = kRowThreads / 64;
+constexpr int kMaxChunks = 16;  // 8 elements each: C <= 64 * 16 * 8 = 8192
+constexpr int kMaxRowLength = 64 * kMaxChunks * 8;
 
 // ----------------------------------------------------------------------------- adaLN
 // utils/adaln_triton.py:36-86.  One workgroup = one token row.
-__global__ __launch_bounds__(kRowThreads) void adaln_kernel(const uint16_t* __restrict__ x, int64_t L, int C,
+template <int NCH>
+__global__ __launch_bounds__(kRowThreads) void adaln_kernel(const uint16_t* __restrict__ x, int64_t rows, int64_t L, int C,
                                                             const uint16_t* __restrict__ scale,
                                                             const uint16_t* __restrict__ shift, int64_t sc_sb,
                                                             int64_t sc_sf, int64_t sh_sb, int64_t sh_sf,
                                                             int64_t frame_seqlen, float eps, int add_one,
                                                             uint16_t* __restrict__ out, AmaxSink sink) {
-  __shared__ float sm[kRowThreads / 64];
-  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
+  if (row >= rows) return;
   const int64_t b = row / L, l = row - b * L, f = l / frame_seqlen;
   const uint16_t* xr = x + row * (int64_t)C;
   const int nchunks = C >> 3;
-  float v[kMaxChunks][8];
+  const uint16_t* scr = scale + b * sc_sb + f * sc_sf;
+  const uint16_t* shr = shift + b * sh_sb + f * sh_sf;
+  float v[NCH][8];
+  uint4 sraw[NCH], hraw[NCH];  // requested up front: their latency runs under the two reductions
   float sum = 0.0f;
 #pragma unroll
-  for (int i = 0; i < kMaxChunks; ++i) {
-    const int c = threadIdx.x + i * kRowThreads;
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + i * 64;
     if (c < nchunks) {
       unpack8(*reinterpret_cast<const uint4*>(xr + c * 8), v[i]);
+      sraw[i] = *reinterpret_cast<const uint4*>(scr + c * 8);
+      hraw[i] = *reinterpret_cast<const uint4*>(shr + c * 8);
 #pragma unroll
       for (int j = 0; j < 8; ++j) sum += v[i][j];
     }
   }
   const float inv_c = 1.0f / (float)C;
-  const float mean = block_sum<kRowThreads>(sum, sm) * inv_c;
+  const float mean = wave_sum_dpp(sum) * inv_c;
   float sq = 0.0f;
 #pragma unroll
-  for (int i = 0; i < kMaxChunks; ++i) {
-    const int c = threadIdx.x + i * kRowThreads;
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + i * 64;
     if (c < nchunks) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
@@ -107,19 +105,17 @@ __global__ __launch_bounds__(kRowThreads) void adaln_kernel(const uint16_t* __re
       }
     }
   }
-  const float var = block_sum<kRowThreads>(sq, sm) * inv_c;
+  const float var = wave_sum_dpp(sq) * inv_c;
   const float rstd = 1.0f / sqrtf(var + eps);
-  const uint16_t* scr = scale + b * sc_sb + f * sc_sf;
-  const uint16_t* shr = shift + b * sh_sb + f * sh_sf;
   uint16_t* orow = out + row * (int64_t)C;
   float out_max = 0.0f;
 #pragma unroll
-  for (int i = 0; i < kMaxChunks; ++i) {
-    const int c = threadIdx.x + i * kRowThreads;
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + i * 64;
     if (c < nchunks) {
       float s8[8], h8[8], y[8];
-      unpack8(*reinterpret_cast<const uint4*>(scr + c * 8), s8);
-      unpack8(*reinterpret_cast<const uint4*>(shr + c * 8), h8);
+      unpack8(sraw[i], s8);
+      unpack8(hraw[i], h8);
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float xn = round_to_bf16(v[i][j] * rstd);
@@ -134,36 +130,38 @@ __global__ __launch_bounds__(kRowThreads) void adaln_kernel(const uint16_t* __re
   }
   if (sink.parts) {
     out_max = wave_max(out_max);
-    if ((threadIdx.x & 63) == 0) amax_sink_update(sink, blockIdx.x * (kRowThreads / 64) + (threadIdx.x >> 6), out_max);
+    if (lane == 0) amax_sink_update(sink, (uint32_t)row, out_max);
   }
 }
 
 // ----------------------------------------------------------------------------- RMSNorm
 // wan_5b/modules/model.py:82-98.
-__global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(const uint16_t* __restrict__ x, int C,
+template <int NCH>
+__global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(const uint16_t* __restrict__ x, int64_t rows, int C,
                                                               const uint16_t* __restrict__ w, float eps,
                                                               uint16_t* __restrict__ out) {
-  __shared__ float sm[kRowThreads / 64];
-  const int64_t row = blockIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
+  if (row >= rows) return;
   const uint16_t* xr = x + row * (int64_t)C;
   const int nchunks = C >> 3;
-  float v[kMaxChunks][8];
+  float v[NCH][8];
   float sq = 0.0f;
 #pragma unroll
-  for (int i = 0; i < kMaxChunks; ++i) {
-    const int c = threadIdx.x + i * kRowThreads;
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + i * 64;
     if (c < nchunks) {
       unpack8(*reinterpret_cast<const uint4*>(xr + c * 8), v[i]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) sq += v[i][j] * v[i][j];
     }
   }
-  const float ms = block_sum<kRowThreads>(sq, sm) / (float)C;
+  const float ms = wave_sum_dpp(sq) / (float)C;
   const float r = 1.0f / sqrtf(ms + eps);
   uint16_t* orow = out + row * (int64_t)C;
 #pragma unroll
-  for (int i = 0; i < kMaxChunks; ++i) {
-    const int c = threadIdx.x + i * kRowThreads;
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + i * 64;
     if (c < nchunks) {
       float w8[8], y[8];
       unpack8(*reinterpret_cast<const uint4*>(w + c * 8), w8);
@@ -179,35 +177,49 @@ __global__ __launch_bounds__(kRowThreads) void rmsnorm_kernel(const uint16_t* __
 // q / k path after the projections (wan_5b/modules/causal_model.py:362-368, 477-487): WanRMSNorm over the
 // whole row, then the 3-D rotary embedding per head of 128, each with the roundings of the separate kernels
 // above; optionally also k - mean(k over the head dimension) (utils/quant.py:797-798) as a second output,
-// mean and difference rounded to bf16 like the two eager operations.  One workgroup = one token row; a head
-// is held by 16 consecutive threads.
-__global__ __launch_bounds__(kRowThreads) void qk_norm_rope_kernel(const uint16_t* __restrict__ x, int C,
-                                                                   const uint16_t* __restrict__ w, float eps,
+// mean and difference rounded to bf16 like the two eager operations.  One wave = one token row; a head is
+// held by 16 consecutive lanes.  blockIdx.y selects the tensor (q or k), so that both go in one launch.
+struct QkProblem {  // one tensor of the q / k pair
+  const uint16_t* x;
+  const uint16_t* w;
+  uint16_t* out;
+  uint16_t* out_smooth;  // or null
+};
+struct QkProblems {
+  QkProblem p[2];
+};
+
+template <int NCH>
+__global__ __launch_bounds__(kRowThreads) void qk_norm_rope_kernel(QkProblems problems, int64_t rows, int C, float eps,
                                                                    const float* __restrict__ cosp,
-                                                                   const float* __restrict__ sinp, int64_t seq_len,
-                                                                   uint16_t* __restrict__ out,
-                                                                   uint16_t* __restrict__ out_smooth) {
-  __shared__ float sm[kRowThreads / 64];
-  const int64_t row = blockIdx.x;
+                                                                   const float* __restrict__ sinp, int64_t seq_len) {
+  const QkProblem& pr = problems.p[blockIdx.y];
+  const uint16_t* __restrict__ x = pr.x;
+  const uint16_t* __restrict__ w = pr.w;
+  uint16_t* __restrict__ out = pr.out;
+  uint16_t* __restrict__ out_smooth = pr.out_smooth;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
+  if (row >= rows) return;
   const uint16_t* xr = x + row * (int64_t)C;
   const int nchunks = C >> 3;
-  float v[kMaxChunks][8];
+  float v[NCH][8];
   float sq = 0.0f;
 #pragma unroll
-  for (int i = 0; i < kMaxChunks; ++i) {
-    const int c = threadIdx.x + i * kRowThreads;
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + i * 64;
     if (c < nchunks) {
       unpack8(*reinterpret_cast<const uint4*>(xr + c * 8), v[i]);
 #pragma unroll
       for (int j = 0; j < 8; ++j) sq += v[i][j] * v[i][j];
     }
   }
-  const float ms = block_sum<kRowThreads>(sq, sm) / (float)C;
+  const float ms = wave_sum_dpp(sq) / (float)C;
   const float r = 1.0f / sqrtf(ms + eps);
   const bool rotate = row < seq_len;
 #pragma unroll
-  for (int i = 0; i < kMaxChunks; ++i) {
-    const int c = threadIdx.x + i * kRowThreads;  // uniform over each group of 16 threads: c < nchunks or not
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + i * 64;  // uniform over each group of 16 threads: c < nchunks or not
     if (c < nchunks) {
       float w8[8], y[8], o8[8];
       unpack8(*reinterpret_cast<const uint4*>(w + c * 8), w8);
@@ -312,19 +324,27 @@ extern "C" int ll_adaln_modulate_amax(const void* x, int64_t B, int64_t L, int C
     sink.epoch = amax_sink->epoch;
   }
   LL_REQUIRE(x && scale && shift && out, "ll_adaln_modulate: null pointer");
-  LL_REQUIRE(B > 0 && L > 0 && C > 0 && C % 8 == 0 && C <= kRowThreads * kMaxChunks * 8 && frame_seqlen > 0 &&
+  LL_REQUIRE(B > 0 && L > 0 && C > 0 && C % 8 == 0 && C <= kMaxRowLength && frame_seqlen > 0 &&
                  L % frame_seqlen == 0,
              "ll_adaln_modulate: bad shape B=%lld L=%lld C=%d frame_seqlen=%lld (C %% 8 == 0, C <= %d)", (long long)B,
-             (long long)L, C, (long long)frame_seqlen, kRowThreads * kMaxChunks * 8);
+             (long long)L, C, (long long)frame_seqlen, kMaxRowLength);
   LL_REQUIRE(scale_stride_b % 8 == 0 && scale_stride_f % 8 == 0 && shift_stride_b % 8 == 0 && shift_stride_f % 8 == 0 &&
                  ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(scale) |
                    reinterpret_cast<uintptr_t>(shift) | reinterpret_cast<uintptr_t>(out)) & 15) == 0,
              "ll_adaln_modulate: pointers must be 16-byte aligned and strides multiples of 8 elements");
   LL_REQUIRE(B * L <= 0x7FFFFFFF, "ll_adaln_modulate: too many rows");
-  hipLaunchKernelGGL(adaln_kernel, dim3((unsigned)(B * L)), dim3(kRowThreads), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint16_t*>(x), L, C, static_cast<const uint16_t*>(scale),
-                     static_cast<const uint16_t*>(shift), scale_stride_b, scale_stride_f, shift_stride_b,
-                     shift_stride_f, frame_seqlen, eps, add_one_to_scale, static_cast<uint16_t*>(out), sink);
+  const dim3 grid((unsigned)((B * L + kRowsPerWg - 1) / kRowsPerWg));
+#define LL_LAUNCH_ADALN(NCH)                                                                                    \
+  hipLaunchKernelGGL(adaln_kernel<NCH>, grid, dim3(kRowThreads), 0, static_cast<hipStream_t>(stream),           \
+                     static_cast<const uint16_t*>(x), B * L, L, C, static_cast<const uint16_t*>(scale),         \
+                     static_cast<const uint16_t*>(shift), scale_stride_b, scale_stride_f, shift_stride_b,       \
+                     shift_stride_f, frame_seqlen, eps, add_one_to_scale, static_cast<uint16_t*>(out), sink)
+  if (C <= 64 * 6 * 8) {
+    LL_LAUNCH_ADALN(6);
+  } else {
+    LL_LAUNCH_ADALN(kMaxChunks);
+  }
+#undef LL_LAUNCH_ADALN
   LL_CHECK_LAUNCH("adaln_kernel");
   return LL_OK;
 }
@@ -333,14 +353,22 @@ extern "C" int ll_rms_norm(const void* x, int64_t rows, int C, const void* weigh
                            void* stream) {
   using namespace ll;
   LL_REQUIRE(x && weight && out, "ll_rms_norm: null pointer");
-  LL_REQUIRE(rows > 0 && rows <= 0x7FFFFFFF && C > 0 && C % 8 == 0 && C <= kRowThreads * kMaxChunks * 8,
+  LL_REQUIRE(rows > 0 && rows <= 0x7FFFFFFF && C > 0 && C % 8 == 0 && C <= kMaxRowLength,
              "ll_rms_norm: bad shape rows=%lld C=%d", (long long)rows, C);
   LL_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) |
                reinterpret_cast<uintptr_t>(out)) & 15) == 0,
              "ll_rms_norm: pointers must be 16-byte aligned");
-  hipLaunchKernelGGL(rmsnorm_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0, static_cast<hipStream_t>(stream),
-                     static_cast<const uint16_t*>(x), C, static_cast<const uint16_t*>(weight), eps,
-                     static_cast<uint16_t*>(out));
+  const dim3 grid((unsigned)((rows + kRowsPerWg - 1) / kRowsPerWg));
+#define LL_LAUNCH_RMS(NCH)                                                                                       \
+  hipLaunchKernelGGL(rmsnorm_kernel<NCH>, grid, dim3(kRowThreads), 0, static_cast<hipStream_t>(stream),          \
+                     static_cast<const uint16_t*>(x), rows, C, static_cast<const uint16_t*>(weight), eps,        \
+                     static_cast<uint16_t*>(out))
+  if (C <= 64 * 6 * 8) {
+    LL_LAUNCH_RMS(6);
+  } else {
+    LL_LAUNCH_RMS(kMaxChunks);
+  }
+#undef LL_LAUNCH_RMS
   LL_CHECK_LAUNCH("rmsnorm_kernel");
   return LL_OK;
 }
@@ -366,22 +394,51 @@ extern "C" int ll_gate_residual(const void* x, const void* y, int64_t B, int64_t
   return LL_OK;
 }
 
+static int launch_qk_norm_rope(const ll::QkProblems& problems, int n_problems, int64_t rows, int num_heads, float eps,
+                               const float* cos, const float* sin, int64_t seq_len, void* stream) {
+  using namespace ll;
+  const int64_t C = (int64_t)num_heads * 128;
+  LL_REQUIRE(cos && sin, "ll_qk_norm_rope: null pointer");
+  LL_REQUIRE(rows > 0 && rows <= 0x7FFFFFFF && num_heads > 0 && C <= kMaxRowLength && seq_len >= 0,
+             "ll_qk_norm_rope: bad shape rows=%lld heads=%d", (long long)rows, num_heads);
+  uintptr_t bits = reinterpret_cast<uintptr_t>(cos) | reinterpret_cast<uintptr_t>(sin);
+  for (int i = 0; i < n_problems; ++i) {
+    const QkProblem& q = problems.p[i];
+    LL_REQUIRE(q.x && q.w && q.out, "ll_qk_norm_rope: null pointer");
+    bits |= reinterpret_cast<uintptr_t>(q.x) | reinterpret_cast<uintptr_t>(q.w) | reinterpret_cast<uintptr_t>(q.out) |
+            reinterpret_cast<uintptr_t>(q.out_smooth);
+  }
+  LL_REQUIRE((bits & 15) == 0, "ll_qk_norm_rope: pointers must be 16-byte aligned");
+  const dim3 grid((unsigned)((rows + kRowsPerWg - 1) / kRowsPerWg), (unsigned)n_problems);
+#define LL_LAUNCH_QK(NCH)                                                                                       \
+  hipLaunchKernelGGL(qk_norm_rope_kernel<NCH>, grid, dim3(kRowThreads), 0, static_cast<hipStream_t>(stream),    \
+                     problems, rows, (int)C, eps, cos, sin, seq_len)
+  if (C <= 64 * 6 * 8) {
+    LL_LAUNCH_QK(6);
+  } else {
+    LL_LAUNCH_QK(kMaxChunks);
+  }
+#undef LL_LAUNCH_QK
+  LL_CHECK_LAUNCH("qk_norm_rope_kernel");
+  return LL_OK;
+}
+
 extern "C" int ll_qk_norm_rope(const void* x, int64_t rows, int num_heads, const void* weight, float eps,
                                const float* cos, const float* sin, int64_t seq_len, void* out, void* out_smooth,
                                void* stream) {
-  using namespace ll;
-  LL_REQUIRE(x && weight && cos && sin && out, "ll_qk_norm_rope: null pointer");
-  const int64_t C = (int64_t)num_heads * 128;
-  LL_REQUIRE(rows > 0 && rows <= 0x7FFFFFFF && num_heads > 0 && C <= kRowThreads * kMaxChunks * 8 && seq_len >= 0,
-             "ll_qk_norm_rope: bad shape rows=%lld heads=%d", (long long)rows, num_heads);
-  LL_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(out) |
-               reinterpret_cast<uintptr_t>(out_smooth) | reinterpret_cast<uintptr_t>(cos) |
-               reinterpret_cast<uintptr_t>(sin)) & 15) == 0,
-             "ll_qk_norm_rope: pointers must be 16-byte aligned");
-  hipLaunchKernelGGL(qk_norm_rope_kernel, dim3((unsigned)rows), dim3(kRowThreads), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const uint16_t*>(x), (int)C,
-                     static_cast<const uint16_t*>(weight), eps, cos, sin, seq_len, static_cast<uint16_t*>(out),
-                     static_cast<uint16_t*>(out_smooth));
-  LL_CHECK_LAUNCH("qk_norm_rope_kernel");
-  return LL_OK;
+  ll::QkProblems problems{};
+  problems.p[0] = {static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(weight), static_cast<uint16_t*>(out),
+                   static_cast<uint16_t*>(out_smooth)};
+  return launch_qk_norm_rope(problems, 1, rows, num_heads, eps, cos, sin, seq_len, stream);
+}
+
+extern "C" int ll_qk_norm_rope_pair(const void* q, const void* k, int64_t rows, int num_heads, const void* q_weight,
+                                    const void* k_weight, float eps, const float* cos, const float* sin,
+                                    int64_t seq_len, void* q_out, void* k_out, void* k_out_smooth, void* stream) {
+  ll::QkProblems problems{};
+  problems.p[0] = {static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(q_weight),
+                   static_cast<uint16_t*>(q_out), nullptr};
+  problems.p[1] = {static_cast<const uint16_t*>(k), static_cast<const uint16_t*>(k_weight),
+                   static_cast<uint16_t*>(k_out), static_cast<uint16_t*>(k_out_smooth)};
+  return launch_qk_norm_rope(problems, 2, rows, num_heads, eps, cos, sin, seq_len, stream);
 }

@@ -101,6 +101,22 @@ __device__ __forceinline__ float wave_sum(float v) {
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
   return v;
 }
+// Sum over the wave with data-parallel-primitive moves instead of LDS permutes: partial sums travel down
+// each row of 16 lanes (row_shr 1, 2, 3, then 4 and 8 under bank masks), then across the rows (row_bcast 15
+// and 31), which leaves the total in lane 63; every lane returns that value.  Lanes that a move does not
+// reach contribute 0 (bound_ctrl).
+#define LL_DPP_ADD(v, ctrl, row_mask, bank_mask)                                                                 \
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, row_mask, bank_mask, true))
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+  LL_DPP_ADD(v, 0x111, 0xF, 0xF);  // row_shr:1
+  LL_DPP_ADD(v, 0x112, 0xF, 0xF);  // row_shr:2
+  LL_DPP_ADD(v, 0x114, 0xF, 0xE);  // row_shr:4, lanes 4-15 of each row
+  LL_DPP_ADD(v, 0x118, 0xF, 0xC);  // row_shr:8, lanes 8-15 of each row
+  LL_DPP_ADD(v, 0x142, 0xA, 0xF);  // row_bcast:15 into rows 1 and 3
+  LL_DPP_ADD(v, 0x143, 0xC, 0xF);  // row_bcast:31 into rows 2 and 3
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+#undef LL_DPP_ADD
 
 // max(m, |v|) over the 8 bf16 values of a packed 16-byte group
 __device__ __forceinline__ float abs_max_bf16x8(const uint4& v, float m) {

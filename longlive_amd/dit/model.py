@@ -128,11 +128,15 @@ class CausalSelfAttention(nn.Module):
         q, k, v = _project_shared(x, [self.q, self.k, self.v], amax=input_amax)
         v = v.view(b, s, n, d)
         if b == 1 and d == 128:
-            # RMSNorm -> RoPE (-> K smoothing) of the reference in one pass per tensor
-            roped_q = _native.qk_norm_rope(q[0], self.norm_q.weight.data, self.norm_q.eps, cos, sin, n).unsqueeze(0)
-            roped_k, smooth_k = _native.qk_norm_rope(k[0], self.norm_k.weight.data, self.norm_k.eps, cos, sin, n,
-                                                     smooth=True)
-            roped_k, smooth_k = roped_k.unsqueeze(0), smooth_k.unsqueeze(0)
+            # RMSNorm -> RoPE (-> K smoothing) of the reference in one pass over q and k
+            if self.norm_q.eps == self.norm_k.eps:
+                roped_q, roped_k, smooth_k = _native.qk_norm_rope_pair(
+                    q[0], k[0], self.norm_q.weight.data, self.norm_k.weight.data, self.norm_q.eps, cos, sin, n)
+            else:
+                roped_q = _native.qk_norm_rope(q[0], self.norm_q.weight.data, self.norm_q.eps, cos, sin, n)
+                roped_k, smooth_k = _native.qk_norm_rope(k[0], self.norm_k.weight.data, self.norm_k.eps, cos, sin, n,
+                                                         smooth=True)
+            roped_q, roped_k, smooth_k = roped_q.unsqueeze(0), roped_k.unsqueeze(0), smooth_k.unsqueeze(0)
         else:
             q = self.norm_q(q).view(b, s, n, d)
             k = self.norm_k(k).view(b, s, n, d)

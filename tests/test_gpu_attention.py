@@ -280,3 +280,18 @@ def test_amax_sink_of_adaln_and_attention_feeds_the_next_quantization(gpu):
         a, b = quantize_to_fp4(out.flatten(1), CFG, amax=ticket), quantize_to_fp4(out.flatten(1), CFG)
         assert float(b.amax) == float(out.abs().max()) and torch.equal(a.amax, b.amax)
         assert torch.equal(a.values, b.values) and np.array_equal(u8(a.scale_factors), u8(b.scale_factors))
+
+
+@pytest.mark.parametrize("S,H", [(50, 24), (7, 40)])  # 24 heads: six groups per lane; 40 heads: the generic width
+def test_norm_rope_of_q_and_k_in_one_launch_equals_two_launches(gpu, S, H):
+    C = H * 128
+    q, k = _randn((S, C), 71, 2.0).to(gpu), _randn((S, C), 72, 2.0).to(gpu)
+    wq, wk = (1 + _randn((C,), 73, 0.1)).to(gpu), (1 + _randn((C,), 74, 0.1)).to(gpu)
+    cos, sin = rope_cos_sin(build_rope_angles(128), 1, 5, 10, 0, gpu)
+    cos, sin = cos[:S].contiguous(), sin[:S].contiguous()
+    rq, rk, sk = _native.qk_norm_rope_pair(q, k, wq, wk, 1e-6, cos, sin, H)
+    assert torch.equal(rq, _native.qk_norm_rope(q, wq, 1e-6, cos, sin, H))
+    one_k, one_s = _native.qk_norm_rope(k, wk, 1e-6, cos, sin, H, smooth=True)
+    assert torch.equal(rk, one_k) and torch.equal(sk, one_s)
+    with pytest.raises(ValueError):
+        _native.qk_norm_rope_pair(q, k[:-1], wq, wk, 1e-6, cos, sin, H)
