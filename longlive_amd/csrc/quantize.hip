@@ -186,14 +186,19 @@ struct ScaleEntry {
 
 typedef float float2v __attribute__((ext_vector_type(2)));
 
+// Codes of one candidate (scale entry e) and, for the rules that choose between candidates, a cheap
+// estimate of its error in units of the candidate's own step: sum (q - y)^2, sum |q - y| or max |q - y| with
+// y = x * r the scaled value the codes were rounded from.
 template <int RULE>
-__device__ __forceinline__ float fast_candidate(const float (&X)[16], const ScaleEntry& e, uint32_t& lo,
-                                                uint32_t& hi) {
+__device__ __forceinline__ float encode_candidate(const float (&X)[16], const ScaleEntry& e, uint32_t& lo,
+                                                  uint32_t& hi) {
+  float y[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) y[i] = __builtin_fmaf(X[i], e.r, 0.0f);
   lo = 0;
   hi = 0;
-#define LL_PACK(dst, base, k)                                                                         \
-  dst = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(dst, __builtin_fmaf(X[base + 2 * k], e.r, 0.0f),    \
-                                                 __builtin_fmaf(X[base + 2 * k + 1], e.r, 0.0f), 1.0f, k)
+#define LL_PACK(dst, base, k) \
+  dst = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(dst, y[base + 2 * k], y[base + 2 * k + 1], 1.0f, k)
   LL_PACK(lo, 0, 0);
   LL_PACK(lo, 0, 1);
   LL_PACK(lo, 0, 2);
@@ -205,6 +210,35 @@ __device__ __forceinline__ float fast_candidate(const float (&X)[16], const Scal
 #undef LL_PACK
   constexpr bool kStatic = (RULE == LL_RULE_STATIC_6 || RULE == LL_RULE_STATIC_4);
   if (kStatic) return 0.0f;
+  float acc = 0.0f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    float2v q;
+    switch (k & 3) {
+      case 0: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(k < 4 ? lo : hi, 1.0f, 0); break;
+      case 1: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(k < 4 ? lo : hi, 1.0f, 1); break;
+      case 2: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(k < 4 ? lo : hi, 1.0f, 2); break;
+      default: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(k < 4 ? lo : hi, 1.0f, 3); break;
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const float d = q[h] - y[2 * k + h];
+      if (RULE == LL_RULE_MSE) {
+        acc = __builtin_fmaf(d, d, acc);
+      } else if (RULE == LL_RULE_MAE) {
+        acc += fabsf(d);
+      } else {
+        acc = fmaxf(acc, fabsf(d));
+      }
+    }
+  }
+  return acc;
+}
+
+// The reference's error of a candidate whose codes are lo / hi: dequantize with the reference's operations,
+// subtract, square or take the magnitude, reduce in the reference's order.
+template <int RULE>
+__device__ __forceinline__ float exact_error(const float (&X)[16], const ScaleEntry& e, uint32_t lo, uint32_t hi) {
   float t[16];
 #pragma unroll
   for (int k = 0; k < 8; ++k) {
@@ -236,10 +270,47 @@ __device__ __forceinline__ float fast_candidate(const float (&X)[16], const Scal
   return acc;
 }
 
+// Four-over-six choice.  The reference compares the two candidates' errors as it computes them in fp32
+// (exact_error).  The estimates of encode_candidate, multiplied by the candidate's step d1 (squared for
+// mse), are the same quantities up to rounding: y carries at most 5 roundings (|y| < 7), the reference's
+// dequantized value 2, its difference, square and 16-term sum a few more.  With u = 2^-24 each estimate E = a w
+// (a in step units, w = d1 or d1^2) and the reference's value both lie within
+//     mse: (320 u sqrt(a) + 32 u a) w     mae: (640 u + 32 u a) w     abs_max: (40 u + 8 u a) w
+// of the exact real-number error, plus 8 u E for the rounding of d1 itself.  When the two estimates differ by
+// more than four times the sum of these bounds the reference's comparison has the same outcome; otherwise
+// (a few blocks in 10^4 of Gaussian data) the block is decided by exact_error.  `approx_ok` is false when the tensor amax is so
+// small or large that squares could leave the normal fp32 range; then every block is decided by exact_error.
+template <int RULE>
+__device__ __forceinline__ bool pick_four(const float (&X)[16], const ScaleEntry& e6, const ScaleEntry& e4, float a6,
+                                          float a4, uint32_t lo6, uint32_t hi6, uint32_t lo4, uint32_t hi4,
+                                          bool approx_ok) {
+  constexpr float u = 0x1p-24f;
+  const float w6 = (RULE == LL_RULE_MSE) ? e6.d1 * e6.d1 : e6.d1;
+  const float w4 = (RULE == LL_RULE_MSE) ? e4.d1 * e4.d1 : e4.d1;
+  const float E6 = a6 * w6, E4 = a4 * w4;
+  float b6, b4;
+  if (RULE == LL_RULE_MSE) {
+    b6 = 320.0f * u * __builtin_sqrtf(a6) + 32.0f * u * a6;
+    b4 = 320.0f * u * __builtin_sqrtf(a4) + 32.0f * u * a4;
+  } else if (RULE == LL_RULE_MAE) {
+    b6 = 640.0f * u + 32.0f * u * a6;
+    b4 = 640.0f * u + 32.0f * u * a4;
+  } else {
+    b6 = 40.0f * u + 8.0f * u * a6;
+    b4 = 40.0f * u + 8.0f * u * a4;
+  }
+  const float margin = 4.0f * (b6 * w6 + b4 * w4 + 8.0f * u * (E6 + E4)) + 0x1p-100f;
+  // abs_max compares two maxima over values that sit on a coarse grid (bf16 inputs): exact ties are common
+  // (a few percent of the blocks), so that rule always takes the reference's arithmetic.
+  if (RULE != LL_RULE_ABS_MAX && approx_ok && fabsf(E4 - E6) > margin) return E4 < E6;
+  return exact_error<RULE>(X, e4, lo4, hi4) < exact_error<RULE>(X, e6, lo6, hi6);
+}
+
 // Returns false when the block has to take the exact path (an element would round past the e2m1 range).
 template <int RULE>
 __device__ __forceinline__ bool quantize_block_fast(const float (&X)[16], float enc, const ScaleEntry* tab,
-                                                    uint32_t& lo, uint32_t& hi, uint32_t& scale_byte) {
+                                                    bool approx_ok, uint32_t& lo, uint32_t& hi,
+                                                    uint32_t& scale_byte) {
   constexpr bool kStatic = (RULE == LL_RULE_STATIC_6 || RULE == LL_RULE_STATIC_4);
   float bmax = fabsf(X[0]);
 #pragma unroll
@@ -258,16 +329,19 @@ __device__ __forceinline__ bool quantize_block_fast(const float (&X)[16], float 
   const ScaleEntry e6 = tab[s6];
   if (!(bmax * e6.r < 7.0f)) return false;
   if (kStatic) {
-    fast_candidate<RULE>(X, e6, lo, hi);
+    encode_candidate<RULE>(X, e6, lo, hi);
     scale_byte = s6;
     return true;
   }
   const ScaleEntry e4 = tab[s4];
   if (!(bmax * e4.r < 7.0f)) return false;
   uint32_t lo4, hi4;
-  const float err6 = fast_candidate<RULE>(X, e6, lo, hi);
-  const float err4 = fast_candidate<RULE>(X, e4, lo4, hi4);
-  const bool pick4 = err4 < err6;
+  const float a6 = encode_candidate<RULE>(X, e6, lo, hi);
+  const float a4 = encode_candidate<RULE>(X, e4, lo4, hi4);
+  // Equal scale bytes (blocks small enough for the subnormal end of e4m3) make the candidates identical: the
+  // reference's strict comparison then keeps "6".  A zero scale byte (block far below the tensor amax) has
+  // r = 0: its estimate says nothing about the error.
+  const bool pick4 = s4 != s6 && pick_four<RULE>(X, e6, e4, a6, a4, lo, hi, lo4, hi4, approx_ok && s6 != 0);
   lo = pick4 ? lo4 : lo;
   hi = pick4 ? hi4 : hi;
   scale_byte = pick4 ? s4 : s6;
@@ -322,6 +396,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
   constexpr float kE2 = (RULE == LL_RULE_STATIC_4) ? 4.0f : 6.0f;
   constexpr float kE4 = kStaticRule ? 448.0f : 256.0f;
   const bool fast = !amax_given && amax >= 0x1p-100f && amax <= 0x1p100f;
+  const bool approx_ok = amax >= 0x1p-30f && amax <= 0x1p30f;  // squares of errors stay normal fp32 numbers
   const float enc = (kE2 * kE4) / amax;
   if (fast && threadIdx.x < 128) {
     const float dec = 1.0f / enc;
@@ -341,8 +416,16 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
 
   // Tiles are dealt to the resident workgroups round-robin, so the prologue above (amax reduction,
   // scale table) is paid once per workgroup and not once per tile.
+  // A tile's rows receive 32 packed bytes each, a quarter of a 128-byte line; the four tiles that complete
+  // the lines are consecutive in tile order.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs,
+  // each with an L2 of its own, so the four tiles go to workgroups v, v + 8, v + 16, v + 24, which start on
+  // the same XCD at about the same time and let that L2 merge the partial lines before they are written back.
+  // (The grid is a multiple of 32 workgroups; v runs over all of them in every round.)
+  const uint32_t n_tiles = (uint32_t)total_tiles;  // 32-bit: cheap division
 #pragma unroll 1
-  for (uint32_t tile = blockIdx.x; tile < (uint32_t)total_tiles; tile += gridDim.x) {  // 32-bit: cheap division
+  for (uint32_t v = blockIdx.x; v < ((n_tiles + 31u) & ~31u); v += gridDim.x) {
+  const uint32_t tile = ((v >> 5) * 8u + (v & 7u)) * 4u + ((v >> 3) & 3u);
+  if (tile >= n_tiles) continue;  // uniform over the workgroup
   const uint32_t tile_y = tile / tiles_x;
   const int64_t row0 = (int64_t)tile_y * 128;
   const int64_t col0 = (int64_t)(tile - tile_y * tiles_x) * 64;
@@ -367,7 +450,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
         X[i] = (row < M && col + i < K) ? bf16_bits_to_f32(x[row * ldx + col + i]) : 0.0f;
     }
     uint32_t lo, hi, sb;
-    if (!fast || !quantize_block_fast<RULE>(X, enc, s_tab, lo, hi, sb)) quantize_block<RULE>(X, amax, lo, hi, sb);
+    if (!fast || !quantize_block_fast<RULE>(X, enc, s_tab, approx_ok, lo, hi, sb)) quantize_block<RULE>(X, amax, lo, hi, sb);
     *reinterpret_cast<uint2*>(values + row * (Kp >> 1) + (col >> 1)) = make_uint2(lo, hi);
     s_bytes[(r & 31) * 16 + (r >> 5) * 4 + cb] = (uint8_t)sb;
   }
@@ -419,7 +502,8 @@ static int quantize_impl(const void* x, int64_t M, int64_t K, int64_t ldx, int r
   // one workgroup per tile up to what the chip holds at once (256 CUs x 8 for the static rules,
   // x 4 for the rules that evaluate two candidates and need twice the registers)
   const int64_t resident = (rule == LL_RULE_STATIC_6 || rule == LL_RULE_STATIC_4) ? 2048 : 1024;
-  const dim3 grid((unsigned)(total_tiles < resident ? total_tiles : resident));
+  const int64_t padded_tiles = (total_tiles + 31) & ~(int64_t)31;  // whole groups of 32 for the XCD-aware tile order
+  const dim3 grid((unsigned)(padded_tiles < resident ? padded_tiles : resident));
 #define LL_LAUNCH_Q(R)                                                                                          \
   hipLaunchKernelGGL(quantize_kernel<R>, grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales, amax, \
                      workspace, amax_given, total_tiles, sink_parts, sink_epoch)

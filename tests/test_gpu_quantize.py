@@ -139,3 +139,21 @@ def test_round_trip_property_at_full_ffn_size(gpu):
     assert em <= e6 * 1.0001
     assert float(qm.amax.cpu()) == float(x.float().abs().max().cpu())
     assert q6.values.shape == (2688, 7168) and not q6.values[2640:].any()
+
+
+@pytest.mark.parametrize("rule", ["mse", "mae", "abs_max"])
+def test_four_over_six_choice_on_ties_and_near_ties(gpu, rule):
+    """The kernel decides most blocks from error estimates in units of the block's step and falls back to the
+    reference's own arithmetic when the two candidates are close.  Inputs built to make them close or equal:
+    values on a coarse lattice (many exact ties), lattice values nudged by one bf16 ulp, blocks repeated at
+    many magnitudes, a tensor amax far from the blocks' size, and blocks far below the tensor amax (scale byte 0)."""
+    rng = np.random.default_rng(7)
+    rows, cols = 1024, 256
+    lattice = rng.integers(-12, 13, size=(rows, cols)).astype(np.float32) * 0.25
+    nudged = lattice * (1.0 + rng.choice([-2.0 ** -8, 0.0, 2.0 ** -8], size=lattice.shape)).astype(np.float32)
+    magn = rng.standard_normal((rows, cols)).astype(np.float32) * np.exp2(rng.integers(-12, 6, size=(rows, 1))).astype(np.float32)
+    two_level = np.where(rng.random((rows, cols)) < 0.5, 1.0, 1.5).astype(np.float32) * rng.choice([-1.0, 1.0], size=(rows, cols)).astype(np.float32)
+    tiny = rng.standard_normal((rows, cols)).astype(np.float32) * 1e-7
+    tiny[0, 0] = 300.0  # tensor amax: the other blocks get scale byte 0 or subnormal scale bytes
+    for x in (lattice, nudged, magn, two_level, tiny):
+        _check(bits_of(torch.from_numpy(x).bfloat16()), rule, gpu)
