@@ -6,6 +6,10 @@ frames is denoised with a few flow-matching steps against the cached context and
 more at timestep 0 so that the cache holds the clean chunk's K / V (:639-647).  The cache keeps
 ``sink_size`` frames plus a sliding window, ``local_attn_size`` frames in total (:775-783).  VAE,
 text encoder and classifier-free guidance are outside this path.
+
+Two samplers: ``"euler"`` steps the flow prediction over the given timesteps (the fixed 1000/750/500/250
+schedule of the benchmark configuration); ``"unipc"`` is the reference pipeline's own choice (:566-612,
+892-900): a fresh FlowUniPCMultistepScheduler per chunk with ``len(timesteps)`` steps and ``sample_shift``.
 """
 from __future__ import annotations
 
@@ -14,14 +18,18 @@ import torch
 from ..fouroversix import ModelQuantizationConfig
 from ..utils import kv_cache as kvc
 from ..utils.quant import LongLiveQuantizationConfig, quantize_model_with_filter
+from ..utils.unipc import FlowUniPCMultistepScheduler
 from .model import CausalDiT, DiTConfig
 
 
 class StreamingGenerator:
     def __init__(self, cfg: DiTConfig, device, timesteps=(1000.0, 750.0, 500.0, 250.0), seed: int = 0,
                  model_quant: dict | None = None, kv_scale_rule: str = "mse", cache_text_kv: bool = True,
-                 skip_dead_cache_writes: bool = True) -> None:
+                 skip_dead_cache_writes: bool = True, sampler: str = "euler", sample_shift: float = 5.0) -> None:
+        if sampler not in ("euler", "unipc"):
+            raise ValueError(f"unknown sampler {sampler!r}")
         self.cfg, self.device = cfg, torch.device(device)
+        self.sampler, self.sample_shift = sampler, sample_shift
         self.timesteps = [float(t) for t in timesteps]
         torch.manual_seed(seed)
         with torch.device(self.device):
@@ -63,14 +71,23 @@ class StreamingGenerator:
         for ci, start in enumerate(range(0, F, nb)):
             x = noise[0, start:start + nb].transpose(0, 1).contiguous()  # [C, f, H, W]
             f = x.shape[1]
-            for si, t in enumerate(self.timesteps):
-                tt = torch.full((1, f), t, device=self.device, dtype=torch.float32)
+            if self.sampler == "unipc":
+                scheduler = FlowUniPCMultistepScheduler(num_train_timesteps=1000, shift=1)
+                scheduler.set_timesteps(len(self.timesteps), device=self.device, shift=self.sample_shift)
+                steps = scheduler.timesteps.tolist()
+            else:
+                scheduler, steps = None, self.timesteps
+            for si, t in enumerate(steps):
+                tt = torch.full((1, f), float(t), device=self.device, dtype=torch.float32)
                 # The K / V a denoising forward would write into the chunk's slot are overwritten by the next
                 # forward before anything reads them (the chunk attends its own K / V in bf16), so only the
                 # clean-context pass below writes; the cache after the chunk is the same either way.
                 flow = self.model(x, tt, context, self.kv_cache, start * fs, crossattn_cache=xcache,
                                   apply_cache_updates=not self.skip_dead_cache_writes)
-                x = (x.float() + (sigmas[si + 1] - sigmas[si]) * flow.float()).to(noise.dtype)
+                if scheduler is not None:
+                    x = scheduler.step(flow, t, x, return_dict=False)[0]
+                else:
+                    x = (x.float() + (sigmas[si + 1] - sigmas[si]) * flow.float()).to(noise.dtype)
             out[0, start:start + f] = x.transpose(0, 1)
             # clean-context pass: rewrites this chunk's K / V in the cache
             self.model(x, torch.zeros((1, f), device=self.device), context, self.kv_cache, start * fs,

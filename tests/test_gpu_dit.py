@@ -323,3 +323,47 @@ def test_text_kv_cache_gives_identical_latents(gpu):
         assert la["_global_end"] == lc["_global_end"] and la["_local_end"] == lc["_local_end"]
         for sa, sc in zip(la["k"] + la["v"], lc["k"] + lc["v"]):
             assert torch.equal(sa.values, sc.values) and torch.equal(sa.amax, sc.amax)
+
+
+def test_generator_with_the_unipc_sampler_follows_a_hand_stepped_scheduler(gpu):
+    """sampler="unipc": every chunk is stepped by a fresh FlowUniPCMultistepScheduler exactly as the reference
+    pipeline does (causal_diffusion_inference.py:566-612).  The first chunk is reproduced here by hand from the
+    model's flow predictions, stepping the numpy oracle next to it."""
+    import unipc_oracle as uo
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    g = torch.Generator().manual_seed(9)
+    noise = torch.randn(1, 4, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    gen = StreamingGenerator(cfg, gpu, seed=4, sampler="unipc", sample_shift=5.0)
+    out = gen.generate(noise, ctx)
+    assert out.shape == noise.shape and bool(torch.isfinite(out.float()).all())
+    euler = StreamingGenerator(cfg, gpu, seed=4).generate(noise, ctx)
+    assert not torch.equal(out, euler)
+
+    ref = StreamingGenerator(cfg, gpu, seed=4, sampler="unipc", sample_shift=5.0)
+    fs = (16 // cfg.patch_size[1]) * (16 // cfg.patch_size[2])
+    ref.reset_cache(fs)
+    sig, ts = uo.schedule(4, 5.0)
+    x = noise[0, :2].transpose(0, 1).contiguous()
+    ms, sig_hist, last, order, lower = [], [], None, 1, 0
+    xo = x.double().cpu().numpy()
+    with torch.no_grad():
+        for i in range(4):
+            tt = torch.full((1, 2), float(ts[i]), device=gpu)
+            flow = ref.model(x, tt, ctx, ref.kv_cache, 0, apply_cache_updates=False).double().cpu().numpy()
+            # the oracle in float64 on the model's own (bf16) trajectory
+            m = x.double().cpu().numpy() - sig[i] * flow
+            if i > 0:
+                xo = uo.uni_c(last, ms, sig_hist, sig[i], m, order)
+            else:
+                xo = x.double().cpu().numpy()
+            ms, sig_hist = (ms + [m])[-2:], (sig_hist + [sig[i]])[-2:]
+            order = min(min(2, 4 - i), lower + 1)
+            last = xo
+            xo = uo.uni_p(xo, ms, sig_hist, sig[i + 1], order)
+            lower = min(lower + 1, 2)
+            x = torch.from_numpy(xo).to(gpu).bfloat16()
+    # bf16 latents: the generator rounds after every step, the hand-stepped copy once per step as well
+    diff = (out[0, :2].transpose(0, 1).float() - x.float()).abs().max().item()
+    assert diff <= 2 * 2.0 ** -7 * out.float().abs().max().item(), diff  # two bf16 ulps of the largest latent
