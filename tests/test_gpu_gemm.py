@@ -218,3 +218,29 @@ def test_amax_sink_of_the_epilogue_feeds_the_next_quantization(gpu):
             assert torch.equal(via_sink.amax, direct.amax) and float(direct.amax) == float(y.abs().max())
             assert torch.equal(via_sink.values, direct.values)
             assert torch.equal(via_sink.scale_factors.view(torch.uint8), direct.scale_factors.view(torch.uint8))
+
+
+@pytest.mark.gpu
+def test_ffn_down_full_size_fused_epilogue_and_sink(gpu):
+    """The FFN pair at the benchmark size: GELU + amax sink in the up projection, gated residual in the down
+    projection, against the same GEMMs followed by the separate operations (bit-identical), and the sink-fed
+    quantization against the one that reduces the tensor itself (identical bytes)."""
+    from longlive_amd import _native
+    from longlive_amd.fouroversix import QuantizationConfig, fp4_matmul, quantize_to_fp4
+    cfg = QuantizationConfig(scale_rule="mse")
+    M, D, F, frame = 2640, 3072, 14336, 880
+    x = activations((M, D), 61).to(gpu)
+    w_up, w_down = quantize_to_fp4(weights((F, D), 62).to(gpu), cfg), quantize_to_fp4(weights((D, F), 63).to(gpu), cfg)
+    gen = torch.Generator().manual_seed(64)
+    residual = torch.randn(M, D, generator=gen).bfloat16().to(gpu)
+    gate = torch.randn(M // frame, 6, D, generator=gen).bfloat16().to(gpu)[:, 5]
+    xq = quantize_to_fp4(x, cfg)
+    ticket = _native.amax_ticket(gpu)
+    h = fp4_matmul(xq, w_up, activation="gelu_tanh", amax_out=ticket)
+    assert torch.equal(h, fp4_matmul(xq, w_up, activation="gelu_tanh"))
+    hq, hq_ref = quantize_to_fp4(h, cfg, amax=ticket), quantize_to_fp4(h, cfg)
+    assert torch.equal(hq.amax, hq_ref.amax) and torch.equal(hq.values, hq_ref.values)
+    assert torch.equal(hq.scale_factors.view(torch.uint8), hq_ref.scale_factors.view(torch.uint8))
+    y = fp4_matmul(hq, w_down)
+    fused = fp4_matmul(hq, w_down, residual=residual, gate=gate, gate_rows=frame)
+    assert torch.equal(fused, residual + (y.view(M // frame, frame, D) * gate[:, None]).view(M, D))
