@@ -63,6 +63,14 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
   return __builtin_bit_cast(uint32_t, p);
 }
 
+// max(v[lane], v[lane ^ 32]) in every lane: one v_permlane32_swap (register file only) instead of a
+// permute through LDS, whose result would also wait for every LDS read issued before it.
+__device__ __forceinline__ float max_over_wave_halves(float v) {
+  const uint32_t u = __float_as_uint(v);
+  const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // r[0] = lower half twice, r[1] = upper half twice
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 __device__ __forceinline__ float fp8_byte_to_f32(uint32_t word, int byte) {
   typedef float float2v_ __attribute__((ext_vector_type(2)));
   const float2v_ lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)word, false);
@@ -401,7 +409,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       float mx = s[qt][0];
 #pragma unroll
       for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[qt][r]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      mx = max_over_wave_halves(mx);
       const bool raise = (mx - m_run[qt]) * p.scale_log2 > kRescaleStep;  // also true for m_run = -inf
       const float m_new = raise ? mx : m_run[qt];
       alpha[qt] = raise ? __builtin_amdgcn_exp2f((m_run[qt] - m_new) * p.scale_log2) : 1.0f;
@@ -574,7 +582,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
         for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[kt][qt][r]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = max_over_wave_halves(mx);
         const bool raise = (mx - m_run[qt]) * p.scale_log2 > kRescaleStep;
         const float m_new = raise ? mx : m_run[qt];
         alpha[qt] = raise ? __builtin_amdgcn_exp2f((m_run[qt] - m_new) * p.scale_log2) : 1.0f;
