@@ -4,13 +4,15 @@
 // Replaces "dequantize the whole cache to bf16, copy the chunk in, call flash attention"
 // (wan_5b/modules/causal_model.py:557-567, 628-671, 781; utils/quant.py:731-768).
 //
-// Workgroup = one head x 128 queries, 4 waves.  Wave w owns 64 queries (w & 1) and every second
-// 64-key tile (w >> 1); the two halves of the key range are merged at the end.  Per iteration all
-// 256 threads decode 128 keys of K and V (e2m1 x e4m3 x amax/(6*256) -> bf16, the values the
-// reference's dequantized bf16 cache holds) into LDS: K row-major, V transposed.  The MFMAs compute
-// S^T = K Q^T and O^T = V^T P^T (v_mfma_f32_32x32x16_bf16), so every lane owns one query column:
-// row max / row sum need no cross-lane traffic beyond one swap between the wave halves, and the
-// online-softmax rescale is a per-lane scalar.
+// Workgroup = one head x 128 queries, 8 waves = two per SIMD.  Wave w owns 32 queries (w & 3) and every
+// second 64-key tile (w >> 2); the two halves of the key range are merged at the end.  A wave needs at most
+// 256 registers (64 for O^T, 32 for S^T, 32 for its Q fragments, the rest for tile fragments, raw FP4 data
+// and addressing), which is what lets two waves share a SIMD: while one wave converts FP4 data or evaluates
+// exponentials, the other one's MFMAs run.  Per iteration all 512 threads decode 128 keys of K and V
+// (e2m1 x e4m3 x amax/(6*256) -> bf16, the values the reference's dequantized bf16 cache holds) into LDS:
+// K row-major, V transposed.  The MFMAs compute S^T = K Q^T and O^T = V^T P^T (v_mfma_f32_32x32x16_bf16), so
+// every lane owns one query column: row max / row sum need no cross-lane traffic beyond one swap between the
+// wave halves, and the online-softmax rescale is a per-lane scalar.
 #include "ll_common.h"
 
 namespace ll {
@@ -23,13 +25,14 @@ constexpr int kHeadDim = 128;
 constexpr int kTileKeys = 64;                  // keys per wave tile
 constexpr int kIterKeys = 2 * kTileKeys;       // keys decoded per iteration (one tile per key-parity)
 constexpr int kWgQueries = 128;
+constexpr int kWaveQueries = 32;
 constexpr int kKPitch = 272;                   // bytes per key row of K in LDS (256 + 16 pad)
 constexpr int kVPitch = 136;                   // bytes per d row of V^T in LDS (128 + 8 pad)
 constexpr int kKTileBytes = kTileKeys * kKPitch;
 constexpr int kVTileBytes = kHeadDim * kVPitch;
 constexpr int kStageBytes = 2 * kKTileBytes + 2 * kVTileBytes;
 constexpr int kMaxSlots = 64;
-constexpr int kAttnThreads = 256;
+constexpr int kAttnThreads = 512;
 
 struct AttnParams {
   const uint16_t* q;
@@ -55,13 +58,7 @@ struct SlotTable {
   float vg[kMaxSlots];
 };
 
-__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
-  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-  bf16x2 p;
-  p[0] = (__bf16)a;
-  p[1] = (__bf16)b;
-  return __builtin_bit_cast(uint32_t, p);
-}
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) { return pack_bf16x2(a, b); }
 
 // max(v[lane], v[lane ^ 32]) in every lane: one v_permlane32_swap (register file only) instead of a
 // permute through LDS, whose result would also wait for every LDS read issued before it.
@@ -91,12 +88,12 @@ __device__ __forceinline__ void fp4x8_to_f32(uint32_t w, float sf, float (&o)[8]
 // Raw FP4 data prefetched one iteration ahead.  Only packed bytes and scale bytes are held in registers
 // across the MFMA phase; everything else (slot scale, kind of key, bf16 source rows of the current chunk)
 // is re-derived from the key index when the data is decoded.
-struct KRaw {         // K of one key, one half of the head dimension (64 elements)
-  uint4 v0, v1;       // 32 packed bytes
-  uint32_t scales;    // 4 e4m3 block scales
+struct KRaw {         // K of one key, one quarter of the head dimension (32 elements)
+  uint4 v;            // 16 packed bytes
+  uint32_t scales;    // 2 e4m3 block scales (low 16 bits)
 };
-struct VRaw {         // V of one key, one 16-element block
-  uint2 v;            // 8 packed bytes
+struct VRaw {         // V of one key, half a 16-element block
+  uint32_t v;         // 4 packed bytes
   uint32_t scale;     // e4m3 block scale byte
 };
 
@@ -108,117 +105,74 @@ __device__ __forceinline__ T load_global(const void* ptr) {
   return *(const __attribute__((address_space(1))) T*)ptr;
 }
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint4 load_global_b128(const void* ptr) {
   const u32x4 v = load_global<u32x4>(ptr);
   return make_uint4(v[0], v[1], v[2], v[3]);
-}
-__device__ __forceinline__ uint2 load_global_b64(const void* ptr) {
-  const u32x2 v = load_global<u32x2>(ptr);
-  return make_uint2(v[0], v[1]);
 }
 
 // Raw FP4 loads.  vo / so are byte offsets of the thread's data inside the slot's value / scale arrays;
 // the caller keeps them up to date incrementally (both advance by a constant per iteration inside a slot).
 __device__ __forceinline__ void fetch_k(const SlotTable& tab, int slot, uint32_t vo, uint32_t so, KRaw& f) {
-  const uint8_t* src = tab.kv[slot] + vo;
-  f.v0 = load_global_b128(src);
-  f.v1 = load_global_b128(src + 16);
-  f.scales = load_global<uint32_t>(tab.ks[slot] + so);
+  f.v = load_global_b128(tab.kv[slot] + vo);
+  f.scales = load_global<uint16_t>(tab.ks[slot] + so);
 }
-
 __device__ __forceinline__ void fetch_v(const SlotTable& tab, int slot, uint32_t vo, uint32_t so, VRaw& f) {
-  f.v = load_global_b64(tab.vv[slot] + vo);
+  f.v = load_global<uint32_t>(tab.vv[slot] + vo);
   f.scale = load_global<uint8_t>(tab.vs[slot] + so);
 }
 
-// Decode K (64 elements of one key) to bf16 and store the 128 bytes into the key's LDS row.
+// Decode K (32 elements of one key) to bf16 and store the 64 bytes into the key's LDS row.
 // kind: 0 = fp4 slot data in f (gs = slot amax / (e2m1_max * e4m3_max)), 1 = bf16 row at src, 2 = zeros.
 __device__ __forceinline__ void store_k(const KRaw& f, int kind, float gs, const uint4* src, uint8_t* dst) {
   uint4* d4 = reinterpret_cast<uint4*>(dst);
   if (kind == 0) {
-    const uint32_t w[8] = {f.v0.x, f.v0.y, f.v0.z, f.v0.w, f.v1.x, f.v1.y, f.v1.z, f.v1.w};
+    const uint32_t w[4] = {f.v.x, f.v.y, f.v.z, f.v.w};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {  // block j: dwords 2j, 2j+1
-      const float sf = fp8_byte_to_f32(f.scales, j) * gs;
-      float lo8[8], hi8[8];
-      fp4x8_to_f32(w[2 * j], sf, lo8);
-      fp4x8_to_f32(w[2 * j + 1], sf, hi8);
-      d4[2 * j] = make_uint4(pack_bf16(lo8[0], lo8[1]), pack_bf16(lo8[2], lo8[3]), pack_bf16(lo8[4], lo8[5]),
-                             pack_bf16(lo8[6], lo8[7]));
-      d4[2 * j + 1] = make_uint4(pack_bf16(hi8[0], hi8[1]), pack_bf16(hi8[2], hi8[3]), pack_bf16(hi8[4], hi8[5]),
-                                 pack_bf16(hi8[6], hi8[7]));
+    for (int j = 0; j < 4; ++j) {
+      const float sf = fp8_byte_to_f32(f.scales, j >> 1) * gs;
+      float v8[8];
+      fp4x8_to_f32(w[j], sf, v8);
+      d4[j] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]), pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
     }
   } else if (kind == 1) {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) d4[i] = src[i];
+    for (int i = 0; i < 4; ++i) d4[i] = src[i];
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) d4[i] = make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < 4; ++i) d4[i] = make_uint4(0, 0, 0, 0);
   }
 }
 
-// 16 head-dim elements of 4 consecutive keys -> for every element one 8-byte run of 4 bf16 along the key
+// 8 head-dim elements of 4 consecutive keys -> for every element one 8-byte run of 4 bf16 along the key
 // axis, written into the transposed V tile.  vt_tile points at the tile, row0 = first d row.
-// kind / gs / src per key as in store_k (src = the key's 16 bf16 elements).
+// kind / gs / src per key as in store_k (src = the key's 8 bf16 elements).
 __device__ __forceinline__ void store_v4(const VRaw (&f)[4], const int (&kind)[4], const float (&gs)[4],
                                          const uint4* const (&src)[4], uint8_t* vt_tile, int row0, int chunk) {
-  const bool all_fp4 = (kind[0] | kind[1] | kind[2] | kind[3]) == 0;
-  if (all_fp4) {
-    float v[4][16];
+  uint32_t w[4][4];
 #pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
+  for (int kk = 0; kk < 4; ++kk) {
+    if (kind[kk] == 0) {
       const float sf = fp8_byte_to_f32(f[kk].scale, 0) * gs[kk];
-      float lo8[8], hi8[8];
-      fp4x8_to_f32(f[kk].v.x, sf, lo8);
-      fp4x8_to_f32(f[kk].v.y, sf, hi8);
+      float v8[8];
+      fp4x8_to_f32(f[kk].v, sf, v8);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        v[kk][i] = lo8[i];
-        v[kk][8 + i] = hi8[i];
-      }
+      for (int i = 0; i < 4; ++i) w[kk][i] = pack_bf16(v8[2 * i], v8[2 * i + 1]);
+    } else if (kind[kk] == 1) {
+      const uint4 a = src[kk][0];
+      w[kk][0] = a.x; w[kk][1] = a.y; w[kk][2] = a.z; w[kk][3] = a.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[kk][i] = 0;
     }
+  }
 #pragma unroll
-    for (int dd = 0; dd < 16; ++dd) {
-      const int row = row0 + dd;
-      *reinterpret_cast<uint2*>(vt_tile + row * kVPitch + chunk * 8) =
-          make_uint2(pack_bf16(v[0][dd], v[1][dd]), pack_bf16(v[2][dd], v[3][dd]));
-    }
-  } else {
-    // generic: bring every key to 8 dwords of bf16, then interleave halves across keys
-    uint32_t w[4][8];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      if (kind[kk] == 0) {
-        const float sf = fp8_byte_to_f32(f[kk].scale, 0) * gs[kk];
-        float lo8[8], hi8[8];
-        fp4x8_to_f32(f[kk].v.x, sf, lo8);
-        fp4x8_to_f32(f[kk].v.y, sf, hi8);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          w[kk][i] = pack_bf16(lo8[2 * i], lo8[2 * i + 1]);
-          w[kk][4 + i] = pack_bf16(hi8[2 * i], hi8[2 * i + 1]);
-        }
-      } else if (kind[kk] == 1) {
-        const uint4 a = src[kk][0], b = src[kk][1];
-        w[kk][0] = a.x; w[kk][1] = a.y; w[kk][2] = a.z; w[kk][3] = a.w;
-        w[kk][4] = b.x; w[kk][5] = b.y; w[kk][6] = b.z; w[kk][7] = b.w;
-      } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) w[kk][i] = 0;
-      }
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      // v_perm_b32: bytes 0-3 come from the second operand, 4-7 from the first
-      const uint32_t e01 = __builtin_amdgcn_perm(w[1][i], w[0][i], 0x05040100u);
-      const uint32_t e23 = __builtin_amdgcn_perm(w[3][i], w[2][i], 0x05040100u);
-      const uint32_t o01 = __builtin_amdgcn_perm(w[1][i], w[0][i], 0x07060302u);
-      const uint32_t o23 = __builtin_amdgcn_perm(w[3][i], w[2][i], 0x07060302u);
-      const int r0 = row0 + 2 * i, r1 = r0 + 1;
-      *reinterpret_cast<uint2*>(vt_tile + r0 * kVPitch + chunk * 8) = make_uint2(e01, e23);
-      *reinterpret_cast<uint2*>(vt_tile + r1 * kVPitch + chunk * 8) = make_uint2(o01, o23);
-    }
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t e01 = __builtin_amdgcn_perm(w[1][i], w[0][i], 0x05040100u);
+    const uint32_t e23 = __builtin_amdgcn_perm(w[3][i], w[2][i], 0x05040100u);
+    const uint32_t o01 = __builtin_amdgcn_perm(w[1][i], w[0][i], 0x07060302u);
+    const uint32_t o23 = __builtin_amdgcn_perm(w[3][i], w[2][i], 0x07060302u);
+    *reinterpret_cast<uint2*>(vt_tile + (row0 + 2 * i) * kVPitch + chunk * 8) = make_uint2(e01, e23);
+    *reinterpret_cast<uint2*>(vt_tile + (row0 + 2 * i + 1) * kVPitch + chunk * 8) = make_uint2(o01, o23);
   }
 }
 
@@ -228,9 +182,8 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
-  const int qh = wave & 1, kp = wave >> 1;
+  const int qq = wave & 3, kp = wave >> 2;  // query quarter (32 queries), key parity
 
-  // workgroup -> (head, query tile); workgroups that share an XCD get the same heads
   int wg = blockIdx.x;
   {
     const int total = p.H * p.n_qtiles;
@@ -247,70 +200,66 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     tab.vg[tid] = load_global<float>(reinterpret_cast<const void*>(p.va_ptrs[tid])) * p.inv_denom;
   }
 
-  // Q fragments: B operand, lane = query column, 8 consecutive head-dim elements per k-step
-  bf16x8 qf[2][8];
-#pragma unroll
-  for (int qt = 0; qt < 2; ++qt) {
-    int64_t query = (int64_t)qtile * kWgQueries + qh * 64 + qt * 32 + l32;
+  bf16x8 qf[8];
+  {
+    int64_t query = (int64_t)qtile * kWgQueries + qq * kWaveQueries + l32;
     if (query >= p.Lq) query = p.Lq - 1;
     const uint16_t* src = p.q + (query * p.H + head) * kHeadDim + 8 * lh;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) qf[qt][ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(src + 16 * ks));
+    for (int ks = 0; ks < 8; ++ks) qf[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(src + 16 * ks));
   }
 
-  float16v o[4][2];
+  float16v o[4];
 #pragma unroll
   for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) o[dt][qt][i] = 0.0f;
-  float m_run[2] = {-INFINITY, -INFINITY}, l_run[2] = {0.0f, 0.0f};
+    for (int i = 0; i < 16; ++i) o[dt][i] = 0.0f;
+  float m_run = -INFINITY, l_run = 0.0f;
 
   const int n_iter = (int)((p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys);
-  __syncthreads();  // slot table visible
+  __syncthreads();
 
-  // ---- decode plan.  K: thread = (key_local = tid / 2, half of the head dim = tid % 2).
-  //                    V: wave = (64-key tile = wave / 2, four of the eight 16-element blocks = wave % 2),
-  //                       lane = (4 consecutive keys = lane % 16, block = lane / 16): for one head-dim row
-  //                       a wave writes four full 128-byte rows of V^T, which the 136-byte pitch spreads
-  //                       over all LDS banks.
+  // ---- decode plan.  K: thread = (key_local = tid / 4, quarter of the head dim = tid % 4).
+  //                    V: key tile = wave / 4; a thread owns 8 elements (half of a 16-element block:
+  //                       hb = lane / 16 + 4 (wave % 4), block hb / 2, half hb % 2) of 4 consecutive keys
+  //                       4 (lane % 16): for one head-dim row 16 lanes write one full 128-byte row of V^T,
+  //                       which the 136-byte pitch spreads over all LDS banks.
   // Schedule of iteration `it`: the MFMAs work on LDS stage it & 1 while the raw FP4 bytes of iteration
-  // it + 1 (already in registers) are decoded into the other stage: K during the S phase, V during the PV
-  // phase, so the conversion arithmetic runs under the MFMAs.  As soon as the K (V) registers are free
-  // the raw bytes of iteration it + 2 are requested, which gives each load most of an iteration to land.
+  // it + 1 (already in registers) are decoded into the other stage during the S phase.  As soon as the raw
+  // registers are free the bytes of iteration it + 2 are requested, which gives each load most of an
+  // iteration to land.  Position of the data the raw registers hold (or will hold next): iter_base = first
+  // key of that iteration; per thread the K key iter_base + k_local and the four V keys
+  // iter_base + v_local + 0..3, each as (slot, offset in slot) plus the byte offsets of its packed values and
+  // scale(s) in the slot.
   KRaw kf;
   VRaw vf[4];
   const int n_cached = (int)p.n_cached, Lk_i = (int)(p.n_cached + p.n_new);
-  const int v_blk = (lane >> 4) + 4 * (wave & 1), v_chunk = lane & 15, v_tile = wave >> 1;
-  // key, slot and offset in the slot of this thread's K key and of its first V key for the iteration whose
-  // raw data is in kf / vf
-  // Position of the data the raw registers hold (or will hold next): iter_base = first key of that
-  // iteration; per thread the K key iter_base + k_local and the four V keys iter_base + v_local + 0..3,
-  // each as (slot, offset in slot) plus the byte offsets of its packed values and scale(s) in the slot.
-  const int k_local = tid >> 1, v_local = v_tile * kTileKeys + 4 * v_chunk;
-  const uint32_t row_bytes = (uint32_t)p.H * 64u;          // packed bytes between consecutive tokens
-  const uint32_t step_vo = (uint32_t)kIterKeys * row_bytes;  // advance of a value offset per iteration
-  const uint32_t step_so = (uint32_t)p.H * 1024u;            // advance of a scale offset (rows += 128 H)
+  const int v_hb = (lane >> 4) + 4 * (wave & 3), v_blk = v_hb >> 1, v_half = v_hb & 1;
+  const int v_chunk = lane & 15, v_tile = wave >> 2;
+  const int k_local = tid >> 2, k_quarter = tid & 3, v_local = v_tile * kTileKeys + 4 * v_chunk;
+  const uint32_t row_bytes = (uint32_t)p.H * 64u;
+  const uint32_t step_vo = (uint32_t)kIterKeys * row_bytes;
+  const uint32_t step_so = (uint32_t)p.H * 1024u;
   const uint32_t slot_bytes = (uint32_t)p.bts * row_bytes;
-  const int k_dst_off = (k_local >> 6) * kKTileBytes + (k_local & 63) * kKPitch + (tid & 1) * 128;
-  const int v_dst_off = 2 * kKTileBytes + v_tile * kVTileBytes + (v_blk * 16) * kVPitch + v_chunk * 8;
+  const int k_dst_off = (k_local >> 6) * kKTileBytes + (k_local & 63) * kKPitch + k_quarter * 64;
+  const int v_row0 = v_blk * 16 + v_half * 8;
+  const int v_dst_off = 2 * kKTileBytes + v_tile * kVTileBytes + v_row0 * kVPitch + v_chunk * 8;
   int iter_base = 0;
   int k_slot = k_local / p.bts, k_off = k_local - k_slot * p.bts;
   int v_slot = v_local / p.bts, v_off = v_local - v_slot * p.bts;
   uint32_t k_vo, k_so, v_vo, v_so[4];
   auto locate_k = [&]() __attribute__((always_inline)) {
     const int64_t row = (int64_t)k_off * p.H + head;
-    k_vo = (uint32_t)row * 64u + (tid & 1) * 32u;
-    k_so = (uint32_t)blocked_scale_offset(row, (tid & 1) * 4, 8);
+    k_vo = (uint32_t)row * 64u + k_quarter * 16u;
+    k_so = (uint32_t)blocked_scale_offset(row, k_quarter * 2, 8);
   };
   auto locate_v = [&]() __attribute__((always_inline)) {
-    v_vo = ((uint32_t)v_off * p.H + head) * 64u + v_blk * 8u;
+    v_vo = ((uint32_t)v_off * p.H + head) * 64u + v_blk * 8u + v_half * 4u;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
-      int o = v_off + kk;
-      if (o >= p.bts) o -= p.bts;  // the key sits in the next slot
-      v_so[kk] = (uint32_t)blocked_scale_offset((int64_t)o * p.H + head, v_blk, 8);
+      int oo = v_off + kk;
+      if (oo >= p.bts) oo -= p.bts;
+      v_so[kk] = (uint32_t)blocked_scale_offset((int64_t)oo * p.H + head, v_blk, 8);
     }
   };
   locate_k();
@@ -342,7 +291,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     v_vo += step_vo;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) v_so[kk] += step_so;
-    if (v_off + 3 >= p.bts) {  // a slot boundary at or inside the thread's four keys
+    if (v_off + 3 >= p.bts) {
       while (v_off >= p.bts) {
         v_off -= p.bts;
         ++v_slot;
@@ -355,7 +304,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     const int kind = k_key < n_cached ? 0 : (k_key < Lk_i ? 1 : 2);
     const float gs = kind == 0 ? tab.kg[k_slot] : 0.0f;
     const uint4* src = reinterpret_cast<const uint4*>(
-        p.k_new + ((int64_t)(k_key - n_cached) * p.H + head) * kHeadDim + (tid & 1) * 64);  // read only if kind == 1
+        p.k_new + ((int64_t)(k_key - n_cached) * p.H + head) * kHeadDim + k_quarter * 32);
     store_k(kf, kind, gs, src, smem + stage * kStageBytes + k_dst_off);
   };
   auto decode_v_any = [&](int stage) __attribute__((always_inline)) {
@@ -367,106 +316,92 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       const int key = iter_base + v_local + kk;
       kind[kk] = key < n_cached ? 0 : (key < Lk_i ? 1 : 2);
       gs[kk] = kind[kk] == 0 ? tab.vg[v_slot + (v_off + kk >= p.bts ? 1 : 0)] : 0.0f;
-      src[kk] = reinterpret_cast<const uint4*>(p.v_new + ((int64_t)(key - n_cached) * p.H + head) * kHeadDim + v_blk * 16);
+      src[kk] = reinterpret_cast<const uint4*>(p.v_new + ((int64_t)(key - n_cached) * p.H + head) * kHeadDim + v_row0);
     }
-    store_v4(vf, kind, gs, src, smem + stage * kStageBytes + 2 * kKTileBytes + v_tile * kVTileBytes, v_blk * 16, v_chunk);
-  };
-
-  // Plain loop: the wave's 64-key tile is handled as two 32-key halves: S half -> running max -> P, PV half.
-  // S^T of one half (32 keys x 64 queries).
-  float16v s[2];
-  auto s_half = [&](const uint8_t* kt_base, int kt) __attribute__((always_inline)) {
-#pragma unroll
-    for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-      for (int i = 0; i < 16; ++i) s[qt][i] = 0.0f;
-    // K fragments are read two steps ahead of their MFMAs
-    const uint8_t* krow = kt_base + (kt * 32 + l32) * kKPitch + lh * 16;
-    uint4 afrag[8];
-    afrag[0] = *reinterpret_cast<const uint4*>(krow);
-    afrag[1] = *reinterpret_cast<const uint4*>(krow + 32);
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      if (ks + 2 < 8) afrag[ks + 2] = *reinterpret_cast<const uint4*>(krow + (ks + 2) * 32);
-      __builtin_amdgcn_sched_barrier(0);  // keep the read up here instead of next to its MFMA
-      const bf16x8 a = __builtin_bit_cast(bf16x8, afrag[ks]);
-#pragma unroll
-      for (int qt = 0; qt < 2; ++qt) s[qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, qf[qt][ks], s[qt], 0, 0, 0);
-    }
+    store_v4(vf, kind, gs, src, smem + stage * kStageBytes + 2 * kKTileBytes + v_tile * kVTileBytes, v_row0, v_chunk);
   };
 
   // Reference point of the exponentials.  m_run is not the exact running maximum: it is raised only when
   // the maximum has grown by more than kRescaleStep (in the exp2 domain) since it was last raised, so P can
-  // reach 2^kRescaleStep instead of 1 (harmless in fp32 / bf16) and the 128 accumulator registers per lane
+  // reach 2^kRescaleStep instead of 1 (harmless in fp32 / bf16) and the 64 accumulator registers per lane
   // are rescaled a handful of times per kernel instead of at almost every tile.  The final division by
   // the row sum, which is accumulated against the same reference, makes the result independent of it.
   constexpr float kRescaleStep = 8.0f;
-  float neg[2];
-  auto softmax_max = [&]() __attribute__((always_inline)) {
-    float alpha[2];
+
+  // Second half of an iteration: reference point of the exponentials over the wave's 64 keys (S^T in sc:
+  // register r of tile kt <-> key 32 kt + 8 (r / 4) + 4 lh + r % 4), then the PV phase in four steps of 16
+  // keys, the exponentials of step j + 1 computed under the four MFMAs of step j.
+  auto softmax_pv = [&](float16v (&sc)[2], const uint8_t* vt_base) __attribute__((always_inline)) {
+    float neg;
+    {
+      float mx = sc[0][0];
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-      float mx = s[qt][0];
+      for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[qt][r]);
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[kt][r]);
       mx = max_over_wave_halves(mx);
-      const bool raise = (mx - m_run[qt]) * p.scale_log2 > kRescaleStep;  // also true for m_run = -inf
-      const float m_new = raise ? mx : m_run[qt];
-      alpha[qt] = raise ? __builtin_amdgcn_exp2f((m_run[qt] - m_new) * p.scale_log2) : 1.0f;
-      neg[qt] = -m_new * p.scale_log2;
-      m_run[qt] = m_new;
-    }
-    if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f) != 0) {
-#pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
-        l_run[qt] *= alpha[qt];
+      const bool raise = (mx - m_run) * p.scale_log2 > kRescaleStep;
+      const float m_new = raise ? mx : m_run;
+      const float alpha = raise ? __builtin_amdgcn_exp2f((m_run - m_new) * p.scale_log2) : 1.0f;
+      neg = -m_new * p.scale_log2;
+      m_run = m_new;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+        l_run *= alpha;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) o[dt][qt][i] *= alpha[qt];
+          for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
       }
     }
-  };
-
-  // P = exp2(...) sixteen keys at a time, then O^T += V^T P^T for those keys.  k-slot e of wave half lh
-  // <-> key 16 hf + 8 (e / 4) + 4 lh + e % 4 of the 32-key half tile.
-  auto pv_half = [&](const uint8_t* vt_base, int kt) __attribute__((always_inline)) {
-    float sum[2] = {0.0f, 0.0f};
+    float sum = 0.0f;
+    auto make_p = [&](int step, bf16x8& dst) __attribute__((always_inline)) {
+      const int kt = step >> 1, hf = step & 1;
+      uint32_t w[4];
 #pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      // V^T fragments of this step first, so that their LDS latency runs under the exponentials
-      const int chunk0 = kt * 8 + hf * 4 + lh;  // 8-byte chunk holding keys 4*chunk0 .. +3 of the tile
-      uint2 vfrag[4][2];
+      for (int i = 0; i < 4; ++i) {
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[kt][8 * hf + 2 * i], p.scale_log2, neg));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[kt][8 * hf + 2 * i + 1], p.scale_log2, neg));
+        sum += p0 + p1;
+        w[i] = pack_bf16(p0, p1);
+      }
+      dst = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+    };
+    auto read_v = [&](int step, uint2 (&dst)[4][2]) __attribute__((always_inline)) {
+      const int chunk0 = (step >> 1) * 8 + (step & 1) * 4 + lh;
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) {
         const uint8_t* src = vt_base + (dt * 32 + l32) * kVPitch;
-        vfrag[dt][0] = *reinterpret_cast<const uint2*>(src + chunk0 * 8);
-        vfrag[dt][1] = *reinterpret_cast<const uint2*>(src + (chunk0 + 2) * 8);
+        dst[dt][0] = *reinterpret_cast<const uint2*>(src + chunk0 * 8);
+        dst[dt][1] = *reinterpret_cast<const uint2*>(src + (chunk0 + 2) * 8);
       }
-      __builtin_amdgcn_sched_barrier(0);  // keep the reads up here instead of next to their MFMAs
-      bf16x8 pb[2];
+    };
+    bf16x8 pb[2];
+    uint2 vfr[2][4][2];
+    read_v(0, vfr[0]);
+    make_p(0, pb[0]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
-        uint32_t w[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float p0 = __builtin_amdgcn_exp2f(fmaf(s[qt][8 * hf + 2 * i], p.scale_log2, neg[qt]));
-          const float p1 = __builtin_amdgcn_exp2f(fmaf(s[qt][8 * hf + 2 * i + 1], p.scale_log2, neg[qt]));
-          sum[qt] += p0 + p1;
-          w[i] = pack_bf16(p0, p1);
-        }
-        pb[qt] = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
-      }
+    for (int step = 0; step < 4; ++step) {
+      if (step < 3) read_v(step + 1, vfr[(step + 1) & 1]);
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) {
-        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(vfrag[dt][0].x, vfrag[dt][0].y, vfrag[dt][1].x, vfrag[dt][1].y));
+        const uint2(&v)[2] = vfr[step & 1][dt];
+        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(v[0].x, v[0].y, v[1].x, v[1].y));
+        o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[step & 1], o[dt], 0, 0, 0);
+      }
+      if (step < 3) {
+        make_p(step + 1, pb[(step + 1) & 1]);
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt) o[dt][qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[qt], o[dt][qt], 0, 0, 0);
+        for (int g = 0; g < 4; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+          __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);  // two exponentials
+          __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);  // their multiply-adds, sums and packing
+        }
       }
     }
-#pragma unroll
-    for (int qt = 0; qt < 2; ++qt) l_run[qt] += sum[qt];
+    l_run += sum;
   };
+
   // prologue: stage 0 <- iteration 0, raw registers <- iteration 1
   fetch_k_next();
   fetch_v_next();
@@ -484,8 +419,10 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   __builtin_amdgcn_s_waitcnt(0x0F70);
 
   // Iterations whose own 128 keys all exist and whose successor is all FP4 form a prefix of the key range;
-  // they run the interleaved body.  The rest (the bf16 chunk, the tail) runs the plain body in a loop of
-  // its own, so that its large temporaries do not add to the register pressure of the first loop.
+  // they run the interleaved body: S^T (64 keys x 32 queries) = 16 MFMAs in eight steps of two, each step
+  // also converting one dword of the prefetched K row (even steps) or two elements of the prefetched V data
+  // for four keys (odd steps) into the other LDS stage.  The rest (the bf16 chunk, the tail) runs the plain
+  // body in a loop of its own.
   int n_fast = n_cached / kIterKeys - 1;
   n_fast = n_fast < 0 ? 0 : (n_fast > n_iter ? n_iter : n_fast);
   int it = 0;
@@ -494,18 +431,14 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     uint8_t* nxt = smem + ((it + 1) & 1) * kStageBytes;
     const uint8_t* vt_base = cur + 2 * kKTileBytes + kp * kVTileBytes;
     const bool has_next2 = it + 2 < n_iter;
-
-    // ---- S phase: S^T (64 keys x 64 queries) = 32 MFMAs, eight steps of four.  Each step also converts
-    //      one dword of the prefetched K row and half a "piece" (2 of the 16 elements x 4 keys) of the
-    //      prefetched V data into the other LDS stage: 32 conversion instructions per four MFMAs.
-    float16v sc[2][2];
+    float16v sc[2];
     {
       const float gsk = tab.kg[k_slot];
       float sfv[4];
 #pragma unroll
       for (int kk = 0; kk < 4; ++kk)
         sfv[kk] = fp8_byte_to_f32(vf[kk].scale, 0) * tab.vg[v_slot + (v_off + kk >= p.bts ? 1 : 0)];
-      const uint32_t w[8] = {kf.v0.x, kf.v0.y, kf.v0.z, kf.v0.w, kf.v1.x, kf.v1.y, kf.v1.z, kf.v1.w};
+      const uint32_t w[4] = {kf.v.x, kf.v.y, kf.v.z, kf.v.w};
       uint8_t* kdst = nxt + k_dst_off;
       uint8_t* vdst = nxt + v_dst_off;
       const uint8_t* krow0 = cur + kp * kKTileBytes + l32 * kKPitch + lh * 16;
@@ -513,9 +446,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) sc[kt][qt][i] = 0.0f;
+        for (int i = 0; i < 16; ++i) sc[kt][i] = 0.0f;
       uint4 a0 = *reinterpret_cast<const uint4*>(krow0), a1 = *reinterpret_cast<const uint4*>(krow1);
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
@@ -525,44 +456,37 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
           n1 = *reinterpret_cast<const uint4*>(krow1 + (ks + 1) * 32);
         }
         const bf16x8 fa0 = __builtin_bit_cast(bf16x8, a0), fa1 = __builtin_bit_cast(bf16x8, a1);
-        sc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, qf[0][ks], sc[0][0], 0, 0, 0);
-        sc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, qf[1][ks], sc[0][1], 0, 0, 0);
-        sc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, qf[0][ks], sc[1][0], 0, 0, 0);
-        sc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, qf[1][ks], sc[1][1], 0, 0, 0);
-        {  // K: dword ks of the row
-          const float sf = fp8_byte_to_f32(kf.scales, ks >> 1) * gsk;
+        sc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, qf[ks], sc[0], 0, 0, 0);
+        sc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, qf[ks], sc[1], 0, 0, 0);
+        if ((ks & 1) == 0) {  // K: dword ks / 2 of the quarter row
+          const int j = ks >> 1;
+          const float sf = fp8_byte_to_f32(kf.scales, j >> 1) * gsk;
           float v8[8];
-          fp4x8_to_f32(w[ks], sf, v8);
-          reinterpret_cast<uint4*>(kdst)[ks] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
-                                                           pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
-        }
-        {  // V: elements 2 ks, 2 ks + 1 of the thread's 16, for its 4 keys -> two rows of V^T
+          fp4x8_to_f32(w[j], sf, v8);
+          reinterpret_cast<uint4*>(kdst)[j] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
+                                                          pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
+        } else {  // V: elements 2 j, 2 j + 1 of the thread's 8, for its 4 keys -> two rows of V^T
+          const int j = ks >> 1;
           float e[4][2];
 #pragma unroll
           for (int kk = 0; kk < 4; ++kk) {
-            const uint32_t word = (ks & 4) ? vf[kk].v.y : vf[kk].v.x;
             float2v q;
-            switch (ks & 3) {
-              case 0: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 0); break;
-              case 1: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 1); break;
-              case 2: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 2); break;
-              default: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(word, 1.0f, 3); break;
+            switch (j) {
+              case 0: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(vf[kk].v, 1.0f, 0); break;
+              case 1: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(vf[kk].v, 1.0f, 1); break;
+              case 2: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(vf[kk].v, 1.0f, 2); break;
+              default: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(vf[kk].v, 1.0f, 3); break;
             }
             e[kk][0] = q[0] * sfv[kk];
             e[kk][1] = q[1] * sfv[kk];
           }
 #pragma unroll
-          for (int j = 0; j < 2; ++j)
-            *reinterpret_cast<uint2*>(vdst + (2 * ks + j) * kVPitch) =
-                make_uint2(pack_bf16(e[0][j], e[1][j]), pack_bf16(e[2][j], e[3][j]));
+          for (int jj = 0; jj < 2; ++jj)
+            *reinterpret_cast<uint2*>(vdst + (2 * j + jj) * kVPitch) =
+                make_uint2(pack_bf16(e[0][jj], e[1][jj]), pack_bf16(e[2][jj], e[3][jj]));
         }
         a0 = n0;
         a1 = n1;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-          __builtin_amdgcn_sched_group_barrier(0x002, 8, 0);  // eight conversion instructions under it
-        }
       }
     }
     advance();
@@ -570,155 +494,71 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       fetch_k_next();
       fetch_v_next();
     }
-
-    // ---- reference point of the exponentials over the 64 keys (see softmax_max)
-    float neg2[2];
-    {
-      float alpha[2];
-#pragma unroll
-      for (int qt = 0; qt < 2; ++qt) {
-        float mx = sc[0][qt][0];
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, sc[kt][qt][r]);
-        mx = max_over_wave_halves(mx);
-        const bool raise = (mx - m_run[qt]) * p.scale_log2 > kRescaleStep;
-        const float m_new = raise ? mx : m_run[qt];
-        alpha[qt] = raise ? __builtin_amdgcn_exp2f((m_run[qt] - m_new) * p.scale_log2) : 1.0f;
-        neg2[qt] = -m_new * p.scale_log2;
-        m_run[qt] = m_new;
-      }
-      if (__builtin_amdgcn_ballot_w64(alpha[0] != 1.0f || alpha[1] != 1.0f) != 0) {
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
-          l_run[qt] *= alpha[qt];
-#pragma unroll
-          for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o[dt][qt][i] *= alpha[qt];
-        }
-      }
-    }
-
-    // ---- PV phase: four steps of 16 keys.  The exponentials of step j + 1 are computed under the eight
-    //      MFMAs of step j.
-    {
-      float sum[2] = {0.0f, 0.0f};
-      auto make_p = [&](int step, bf16x8 (&dst)[2]) __attribute__((always_inline)) {
-        const int kt = step >> 1, hf = step & 1;
-#pragma unroll
-        for (int qt = 0; qt < 2; ++qt) {
-          uint32_t w[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float p0 = __builtin_amdgcn_exp2f(fmaf(sc[kt][qt][8 * hf + 2 * i], p.scale_log2, neg2[qt]));
-            const float p1 = __builtin_amdgcn_exp2f(fmaf(sc[kt][qt][8 * hf + 2 * i + 1], p.scale_log2, neg2[qt]));
-            sum[qt] += p0 + p1;
-            w[i] = pack_bf16(p0, p1);
-          }
-          dst[qt] = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
-        }
-      };
-      auto read_v = [&](int step, uint2 (&dst)[4][2]) __attribute__((always_inline)) {
-        const int chunk0 = (step >> 1) * 8 + (step & 1) * 4 + lh;  // 8-byte chunk holding keys 4*chunk0 .. +3
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-          const uint8_t* src = vt_base + (dt * 32 + l32) * kVPitch;
-          dst[dt][0] = *reinterpret_cast<const uint2*>(src + chunk0 * 8);
-          dst[dt][1] = *reinterpret_cast<const uint2*>(src + (chunk0 + 2) * 8);
-        }
-      };
-      bf16x8 pb[2][2];
-      uint2 vfr[2][4][2];
-      read_v(0, vfr[0]);
-      make_p(0, pb[0]);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int step = 0; step < 4; ++step) {
-        if (step < 3) read_v(step + 1, vfr[(step + 1) & 1]);
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt) {
-          const uint2(&v)[2] = vfr[step & 1][dt];
-          const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(v[0].x, v[0].y, v[1].x, v[1].y));
-#pragma unroll
-          for (int qt = 0; qt < 2; ++qt) o[dt][qt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[step & 1][qt], o[dt][qt], 0, 0, 0);
-        }
-        if (step < 3) {
-          make_p(step + 1, pb[(step + 1) & 1]);
-#pragma unroll
-          for (int g = 0; g < 8; ++g) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-            __builtin_amdgcn_sched_group_barrier(0x400, 2, 0);  // two exponentials
-            __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);  // their multiply-adds, sums and packing
-          }
-        }
-      }
-#pragma unroll
-      for (int qt = 0; qt < 2; ++qt) l_run[qt] += sum[qt];
-    }
+    softmax_pv(sc, vt_base);
     __syncthreads();
   }
+
+  // Plain body: the S phase without interleaved conversion, masking in the last tile, and the successor tile
+  // decoded after the MFMAs (or, for the chunk's own bf16 tiles, brought in ahead of them).
   typedef __attribute__((address_space(1))) const void* gptr_t;
   typedef __attribute__((address_space(3))) void* lptr_t;
   for (; it < n_iter; ++it) {
     const uint8_t* cur = smem + (it & 1) * kStageBytes;
-    const uint8_t* kt_base = cur + kp * kKTileBytes;
     const uint8_t* vt_base = cur + 2 * kKTileBytes + kp * kVTileBytes;
     const int tile_base = it * kIterKeys + kp * kTileKeys;
     // A successor that lies wholly in the bf16 chunk is brought in ahead of the MFMAs: its K rows go
-    // straight from global memory into the other stage (one 256-byte row per wave instruction, 32 rows per
+    // straight from global memory into the other stage (one 256-byte row per wave instruction, 16 rows per
     // wave), its V pieces are requested now and transposed into LDS after the PV phase.
     const bool next_is_chunk = iter_base >= n_cached && iter_base + kIterKeys <= Lk_i;  // iter_base = first key of tile it + 1
-    uint4 vraw[4][2];
+    uint4 vraw[4];
     if (next_is_chunk) {
       uint8_t* nxt = smem + ((it + 1) & 1) * kStageBytes;
-      const uint16_t* ksrc = p.k_new + ((int64_t)(iter_base + wave * 32 - n_cached) * p.H + head) * kHeadDim + lane * 2;
-      uint8_t* kdst = nxt + (wave >> 1) * kKTileBytes + ((wave & 1) * 32) * kKPitch;
+      const uint16_t* ksrc = p.k_new + ((int64_t)(iter_base + wave * 16 - n_cached) * p.H + head) * kHeadDim + lane * 2;
+      uint8_t* kdst = nxt + (wave >> 2) * kKTileBytes + ((wave & 3) * 16) * kKPitch;
 #pragma unroll
-      for (int r = 0; r < 32; ++r)
+      for (int r = 0; r < 16; ++r)
         __builtin_amdgcn_global_load_lds((gptr_t)(ksrc + (int64_t)r * p.H * kHeadDim), (lptr_t)(kdst + r * kKPitch), 4, 0, 0);
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk) {
-        const uint16_t* vsrc = p.v_new + ((int64_t)(iter_base + v_local + kk - n_cached) * p.H + head) * kHeadDim + v_blk * 16;
-        vraw[kk][0] = load_global_b128(vsrc);
-        vraw[kk][1] = load_global_b128(vsrc + 8);
-      }
+      for (int kk = 0; kk < 4; ++kk)
+        vraw[kk] = load_global_b128(p.v_new + ((int64_t)(iter_base + v_local + kk - n_cached) * p.H + head) * kHeadDim + v_row0);
     }
+    if (tile_base < Lk_i) {
+      float16v sc[2];
+      const uint8_t* krow0 = cur + kp * kKTileBytes + l32 * kKPitch + lh * 16;
+      const uint8_t* krow1 = krow0 + 32 * kKPitch;
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt) {
-      const int half_base = tile_base + kt * 32;
-      if (half_base < Lk_i) {
-        s_half(kt_base, kt);
-        if (half_base + 32 > Lk_i) {  // mask keys beyond the end (only in the last tile)
+      for (int kt = 0; kt < 2; ++kt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) sc[kt][i] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const bf16x8 fa0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow0 + ks * 32));
+        const bf16x8 fa1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow1 + ks * 32));
+        sc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, qf[ks], sc[0], 0, 0, 0);
+        sc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, qf[ks], sc[1], 0, 0, 0);
+      }
+      if (tile_base + kTileKeys > Lk_i) {
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const int key = half_base + 8 * (r >> 2) + 4 * lh + (r & 3);
-            if (key >= Lk_i) {
-              s[0][r] = -INFINITY;
-              s[1][r] = -INFINITY;
-            }
+            const int key = tile_base + kt * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+            if (key >= Lk_i) sc[kt][r] = -INFINITY;
           }
-        }
-        softmax_max();
-        pv_half(vt_base, kt);
       }
+      softmax_pv(sc, vt_base);
     }
     if (next_is_chunk) {
       uint8_t* vdst = smem + ((it + 1) & 1) * kStageBytes + v_dst_off;
+      const uint32_t w[4][4] = {{vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w}, {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w},
+                                {vraw[2].x, vraw[2].y, vraw[2].z, vraw[2].w}, {vraw[3].x, vraw[3].y, vraw[3].z, vraw[3].w}};
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {  // elements 2 i, 2 i + 1 of the thread's 16, for its 4 keys -> two rows of V^T
-        uint32_t w[4];
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-          const uint4 q = vraw[kk][i >> 2];
-          w[kk] = (i & 3) == 0 ? q.x : (i & 3) == 1 ? q.y : (i & 3) == 2 ? q.z : q.w;
-        }
+      for (int i = 0; i < 4; ++i) {  // elements 2 i, 2 i + 1 of the thread's 8, for its 4 keys -> two rows of V^T
         // v_perm_b32: bytes 0-3 come from the second operand, 4-7 from the first
         *reinterpret_cast<uint2*>(vdst + (2 * i) * kVPitch) =
-            make_uint2(__builtin_amdgcn_perm(w[1], w[0], 0x05040100u), __builtin_amdgcn_perm(w[3], w[2], 0x05040100u));
+            make_uint2(__builtin_amdgcn_perm(w[1][i], w[0][i], 0x05040100u), __builtin_amdgcn_perm(w[3][i], w[2][i], 0x05040100u));
         *reinterpret_cast<uint2*>(vdst + (2 * i + 1) * kVPitch) =
-            make_uint2(__builtin_amdgcn_perm(w[1], w[0], 0x07060302u), __builtin_amdgcn_perm(w[3], w[2], 0x07060302u));
+            make_uint2(__builtin_amdgcn_perm(w[1][i], w[0][i], 0x07060302u), __builtin_amdgcn_perm(w[3][i], w[2][i], 0x07060302u));
       }
       iter_base += kIterKeys;  // the slot bookkeeping of advance() has no use beyond the cache
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K rows have landed in LDS
@@ -735,57 +575,48 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   }
 
   // ---- merge the two key-parity halves and write out.  Row sums are per wave half so far.
-#pragma unroll
-  for (int qt = 0; qt < 2; ++qt) l_run[qt] += __shfl_xor(l_run[qt], 32, 64);
-  float* xo = reinterpret_cast<float*>(smem);                 // [qh][128 regs][64 lanes]
-  float* xm = xo + 2 * 128 * 64;                               // [qh][2][64]
-  float* xl = xm + 2 * 2 * 64;
+  l_run += __shfl_xor(l_run, 32, 64);
+  float* xo = reinterpret_cast<float*>(smem);   // [qq][64 regs][64 lanes]
+  float* xm = xo + 4 * 64 * 64;                  // [qq][64]
+  float* xl = xm + 4 * 64;
   if (kp == 1) {
 #pragma unroll
     for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-      for (int qt = 0; qt < 2; ++qt)
-#pragma unroll
-        for (int i = 0; i < 16; ++i) xo[(qh * 128 + (dt * 2 + qt) * 16 + i) * 64 + lane] = o[dt][qt][i];
-#pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-      xm[(qh * 2 + qt) * 64 + lane] = m_run[qt];
-      xl[(qh * 2 + qt) * 64 + lane] = l_run[qt];
-    }
+      for (int i = 0; i < 16; ++i) xo[(qq * 64 + dt * 16 + i) * 64 + lane] = o[dt][i];
+    xm[qq * 64 + lane] = m_run;
+    xl[qq * 64 + lane] = l_run;
   }
   __syncthreads();
   if (kp == 0) {
     float out_max = 0.0f;
+    const float m1 = xm[qq * 64 + lane], l1 = xl[qq * 64 + lane];
+    const float m = fmaxf(m_run, m1);
+    const float a0 = __builtin_amdgcn_exp2f((m_run - m) * p.scale_log2);
+    const float a1 = (m1 == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m1 - m) * p.scale_log2);
+    const float inv_l = 1.0f / (l_run * a0 + l1 * a1);
+    const int64_t query = (int64_t)qtile * kWgQueries + qq * kWaveQueries + l32;
+    if (query < p.Lq) {
+      uint16_t* dst = p.out + (query * p.H + head) * kHeadDim;
 #pragma unroll
-    for (int qt = 0; qt < 2; ++qt) {
-      const float m1 = xm[(qh * 2 + qt) * 64 + lane], l1 = xl[(qh * 2 + qt) * 64 + lane];
-      const float m = fmaxf(m_run[qt], m1);
-      const float a0 = __builtin_amdgcn_exp2f((m_run[qt] - m) * p.scale_log2);
-      const float a1 = (m1 == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m1 - m) * p.scale_log2);
-      const float inv_l = 1.0f / (l_run[qt] * a0 + l1 * a1);
-      const int64_t query = (int64_t)qtile * kWgQueries + qh * 64 + qt * 32 + l32;
-      if (query < p.Lq) {
-        uint16_t* dst = p.out + (query * p.H + head) * kHeadDim;
+      for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int rg = 0; rg < 4; ++rg) {
+          float v[4];
 #pragma unroll
-          for (int rg = 0; rg < 4; ++rg) {
-            float v[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-              const float o1 = xo[(qh * 128 + (dt * 2 + qt) * 16 + 4 * rg + i) * 64 + lane];
-              v[i] = (o[dt][qt][4 * rg + i] * a0 + o1 * a1) * inv_l;
-            }
-            const int d = dt * 32 + 8 * rg + 4 * lh;
-            const uint2 packed = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
-            *reinterpret_cast<uint2*>(dst + d) = packed;
-            out_max = abs_max_bf16x8(make_uint4(packed.x, packed.y, 0u, 0u), out_max);
+          for (int i = 0; i < 4; ++i) {
+            const float o1 = xo[(qq * 64 + dt * 16 + 4 * rg + i) * 64 + lane];
+            v[i] = (o[dt][4 * rg + i] * a0 + o1 * a1) * inv_l;
           }
-      }
+          const int d = dt * 32 + 8 * rg + 4 * lh;
+          const uint2 packed = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+          *reinterpret_cast<uint2*>(dst + d) = packed;
+          out_max = abs_max_bf16x8(make_uint4(packed.x, packed.y, 0u, 0u), out_max);
+        }
     }
     if (p.sink.parts) {
       out_max = wave_max(out_max);
-      if (lane == 0) amax_sink_update(p.sink, blockIdx.x * 2 + qh, out_max);
+      if (lane == 0) amax_sink_update(p.sink, blockIdx.x * 4 + qq, out_max);
     }
   }
 }
@@ -859,7 +690,6 @@ extern "C" int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads, co
   p.vv_ptrs = v_values_ptrs; p.vs_ptrs = v_scales_ptrs; p.va_ptrs = v_amax_ptrs;
   p.n_cached = n_cached;
   p.n_new = n_new;
-  // without cached tokens the slot size only feeds the (unused) position bookkeeping: make it never wrap
   p.bts = n_cached > 0 ? block_token_size : (1 << 30);
   p.n_slots = n_slots;
   p.inv_denom = n_cached > 0 ? 1.0f / (e2m1_max * e4m3_max) : 0.f;
@@ -868,8 +698,6 @@ extern "C" int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads, co
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.out = static_cast<uint16_t*>(out);
   if (amax_sink && amax_sink->parts) {
-    LL_REQUIRE((reinterpret_cast<uintptr_t>(amax_sink->parts) & 7) == 0 && amax_sink->epoch != 0,
-               "ll_kv_attention_amax: amax sink needs 8-byte alignment and a non-zero epoch");
     p.sink.parts = reinterpret_cast<unsigned long long*>(amax_sink->parts);
     p.sink.epoch = amax_sink->epoch;
   }
