@@ -220,10 +220,10 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   __syncthreads();
 
   // ---- decode plan.  K: thread = (key_local = tid / 4, quarter of the head dim = tid % 4).
-  //                    V: key tile = wave / 4; a thread owns 8 elements (half of a 16-element block:
-  //                       hb = lane / 16 + 4 (wave % 4), block hb / 2, half hb % 2) of 4 consecutive keys
-  //                       4 (lane % 16): for one head-dim row 16 lanes write one full 128-byte row of V^T,
-  //                       which the 136-byte pitch spreads over all LDS banks.
+  //                    V: key tile = wave / 4; a thread owns 8 elements (half lane / 32 of the 16-element
+  //                       block 2 (wave % 4) + lane / 16 % 2) of 4 consecutive keys 4 (lane % 16): for one
+  //                       head-dim row 16 lanes write one full 128-byte row of V^T, which the 136-byte pitch
+  //                       spreads over all LDS banks.
   // Schedule of iteration `it`: the MFMAs work on LDS stage it & 1 while the raw FP4 bytes of iteration
   // it + 1 (already in registers) are decoded into the other stage during the S phase.  As soon as the raw
   // registers are free the bytes of iteration it + 2 are requested, which gives each load most of an
@@ -234,7 +234,8 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   KRaw kf;
   VRaw vf[4];
   const int n_cached = (int)p.n_cached, Lk_i = (int)(p.n_cached + p.n_new);
-  const int v_hb = (lane >> 4) + 4 * (wave & 3), v_blk = v_hb >> 1, v_half = v_hb & 1;
+  // lanes 0-31 of a wave (one pass of an 8-byte LDS write) get rows 16 apart = 32 banks apart
+  const int v_blk = 2 * (wave & 3) + ((lane >> 4) & 1), v_half = lane >> 5;
   const int v_chunk = lane & 15, v_tile = wave >> 2;
   const int k_local = tid >> 2, k_quarter = tid & 3, v_local = v_tile * kTileKeys + 4 * v_chunk;
   const uint32_t row_bytes = (uint32_t)p.H * 64u;
