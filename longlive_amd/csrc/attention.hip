@@ -249,10 +249,12 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   int k_slot = k_local / p.bts, k_off = k_local - k_slot * p.bts;
   int v_slot = v_local / p.bts, v_off = v_local - v_slot * p.bts;
   uint32_t k_vo, k_so, v_vo, v_so[4];
+  float k_gs, v_gs[4];  // slot scale amax / (e2m1_max * e4m3_max) of the thread's K key and of its four V keys
   auto locate_k = [&]() __attribute__((always_inline)) {
     const int64_t row = (int64_t)k_off * p.H + head;
     k_vo = (uint32_t)row * 64u + k_quarter * 16u;
     k_so = (uint32_t)blocked_scale_offset(row, k_quarter * 2, 8);
+    k_gs = tab.kg[min(k_slot, kMaxSlots - 1)];
   };
   auto locate_v = [&]() __attribute__((always_inline)) {
     v_vo = ((uint32_t)v_off * p.H + head) * 64u + v_blk * 8u + v_half * 4u;
@@ -261,6 +263,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       int oo = v_off + kk;
       if (oo >= p.bts) oo -= p.bts;
       v_so[kk] = (uint32_t)blocked_scale_offset((int64_t)oo * p.H + head, v_blk, 8);
+      v_gs[kk] = tab.vg[min(v_slot + (v_off + kk >= p.bts ? 1 : 0), kMaxSlots - 1)];
     }
   };
   locate_k();
@@ -303,7 +306,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   auto decode_k_any = [&](int stage) __attribute__((always_inline)) {
     const int k_key = iter_base + k_local;
     const int kind = k_key < n_cached ? 0 : (k_key < Lk_i ? 1 : 2);
-    const float gs = kind == 0 ? tab.kg[k_slot] : 0.0f;
+    const float gs = kind == 0 ? k_gs : 0.0f;
     const uint4* src = reinterpret_cast<const uint4*>(
         p.k_new + ((int64_t)(k_key - n_cached) * p.H + head) * kHeadDim + k_quarter * 32);
     store_k(kf, kind, gs, src, smem + stage * kStageBytes + k_dst_off);
@@ -316,7 +319,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     for (int kk = 0; kk < 4; ++kk) {
       const int key = iter_base + v_local + kk;
       kind[kk] = key < n_cached ? 0 : (key < Lk_i ? 1 : 2);
-      gs[kk] = kind[kk] == 0 ? tab.vg[v_slot + (v_off + kk >= p.bts ? 1 : 0)] : 0.0f;
+      gs[kk] = kind[kk] == 0 ? v_gs[kk] : 0.0f;
       src[kk] = reinterpret_cast<const uint4*>(p.v_new + ((int64_t)(key - n_cached) * p.H + head) * kHeadDim + v_row0);
     }
     store_v4(vf, kind, gs, src, smem + stage * kStageBytes + 2 * kKTileBytes + v_tile * kVTileBytes, v_row0, v_chunk);
@@ -434,11 +437,10 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     const bool has_next2 = it + 2 < n_iter;
     float16v sc[2];
     {
-      const float gsk = tab.kg[k_slot];
+      const float gsk = k_gs;
       float sfv[4];
 #pragma unroll
-      for (int kk = 0; kk < 4; ++kk)
-        sfv[kk] = fp8_byte_to_f32(vf[kk].scale, 0) * tab.vg[v_slot + (v_off + kk >= p.bts ? 1 : 0)];
+      for (int kk = 0; kk < 4; ++kk) sfv[kk] = fp8_byte_to_f32(vf[kk].scale, 0) * v_gs[kk];
       const uint32_t w[4] = {kf.v.x, kf.v.y, kf.v.z, kf.v.w};
       uint8_t* kdst = nxt + k_dst_off;
       uint8_t* vdst = nxt + v_dst_off;
