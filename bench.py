@@ -36,7 +36,7 @@ LINEAR_SET = [
 PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak (the GEMM runs v_mfma_f32_32x32x16_f16)
 # HBM-side bytes of one FFN-up GEMM launch from the rocprofv3 counter runs kept under profiles/:
 # FETCH_SIZE 82078 KiB x 2.0 (the factor a 256 MiB copy calibrates) + WRITE_SIZE 73920 KiB x 1.0
-FFN_UP_TRAFFIC_BYTES = (93378.6 * 2.0 + 73927.3) * 1024  # FETCH_SIZE x 2.00 (copy yardstick) + WRITE_SIZE, KiB per launch
+FFN_UP_TRAFFIC_BYTES = (93206.0 * 2.0 + 73927.3) * 1024  # FETCH_SIZE x 2.00 (copy yardstick) + WRITE_SIZE, KiB per launch
 
 
 def step_flops() -> float:
@@ -173,6 +173,31 @@ def run_e2e(torch, dev):
                         "sink 3 + window 12 frames, text K/V projected once per prompt, cache written by the recache forward only (the denoising forwards' writes are dead stores); one untimed 3-frame run first; the chunks get slower until the window of 12 frames is full"}
 
 
+def run_gemm_shapes(torch, dev, work, cfg, steps):
+    """The W4A4 GEMM kernel alone on each distinct shape of the linear set (operands already quantized), with the
+    vendor library's dense f16 GEMM (torch.matmul) on operands of the same shape beside it: the library kernel
+    does the same MFMA work without any FP4 decoding, which makes it the yardstick for the fused kernel."""
+    from longlive_amd.fouroversix import fp4_matmul, quantize_to_fp4
+
+    rows, seen = [], set()
+    for name, x, wq in work:
+        m, k = x.shape
+        n = wq.original_shape[0]
+        if (m, n, k) in seen:
+            continue
+        seen.add((m, n, k))
+        xq = quantize_to_fp4(x, cfg)
+        ms = _time_events(torch, lambda: fp4_matmul(xq, wq), steps)
+        a16 = x.to(torch.float16)
+        w16 = torch.randn(n, k, device=dev, dtype=torch.float16)
+        lib = _time_events(torch, lambda: torch.matmul(a16, w16.t()), steps)
+        flops = 2.0 * m * n * k
+        rows.append({"linear": name, "M": m, "N": n, "K": k, "w4a4_us": 1e3 * ms, "w4a4_TFLOPs": flops / ms / 1e9,
+                     "library_f16_us": 1e3 * lib, "library_f16_TFLOPs": flops / lib / 1e9})
+        del a16, w16
+    return rows
+
+
 def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -299,7 +324,8 @@ def main() -> None:
     }
     if not args.no_extras:
         extras = {}
-        for key, fn in (("attention", lambda: run_attention(torch, dev, 10)), ("block", lambda: run_block(torch, dev, 10)),
+        for key, fn in (("gemm_shapes", lambda: run_gemm_shapes(torch, dev, work, cfg, 10)),
+                        ("attention", lambda: run_attention(torch, dev, 10)), ("block", lambda: run_block(torch, dev, 10)),
                         ("e2e", lambda: run_e2e(torch, dev))):
             try:
                 extras[key] = fn()
