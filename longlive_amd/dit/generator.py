@@ -7,6 +7,11 @@ more at timestep 0 so that the cache holds the clean chunk's K / V (:639-647).  
 ``sink_size`` frames plus a sliding window, ``local_attn_size`` frames in total (:775-783).  VAE,
 text encoder and classifier-free guidance are outside this path.
 
+Multi-shot generation (:104-107, 630-665, 974-1043): with ``multi_shot_sink`` the first ``sink_size`` frames of
+the stream become a global sink that is never evicted, and the first chunk of every later scene (``scene_cuts``)
+is pinned after its clean-context pass, so that the new scene attends its own opening frames instead of the
+previous scene's; ``shot_clean_recache`` additionally forgets everything but the global sink before that pass.
+
 Two samplers: ``"euler"`` steps the flow prediction over the given timesteps (the fixed 1000/750/500/250
 schedule of the benchmark configuration); ``"unipc"`` is the reference pipeline's own choice (:566-612,
 892-900): a fresh FlowUniPCMultistepScheduler per chunk with ``len(timesteps)`` steps and ``sample_shift``.
@@ -25,7 +30,8 @@ from .model import CausalDiT, DiTConfig
 class StreamingGenerator:
     def __init__(self, cfg: DiTConfig, device, timesteps=(1000.0, 750.0, 500.0, 250.0), seed: int = 0,
                  model_quant: dict | None = None, kv_scale_rule: str = "mse", cache_text_kv: bool = True,
-                 skip_dead_cache_writes: bool = True, sampler: str = "euler", sample_shift: float = 5.0) -> None:
+                 skip_dead_cache_writes: bool = True, sampler: str = "euler", sample_shift: float = 5.0,
+                 multi_shot_sink: bool = False, shot_clean_recache: bool = False) -> None:
         if sampler not in ("euler", "unipc"):
             raise ValueError(f"unknown sampler {sampler!r}")
         self.cfg, self.device = cfg, torch.device(device)
@@ -44,6 +50,9 @@ class StreamingGenerator:
         self.kv_quant_config = LongLiveQuantizationConfig(scale_rule=kv_scale_rule, backend="cuda", type="kv")
         self.model.kv_quant_config = self.kv_quant_config
         self.kv_cache = None
+        self.multi_shot_sink, self.shot_clean_recache = multi_shot_sink, shot_clean_recache
+        self.global_sink_size = cfg.sink_size if multi_shot_sink else 0   # :107
+        self.model.global_sink_size = self.global_sink_size
         self.cache_text_kv = cache_text_kv
         self.skip_dead_cache_writes = skip_dead_cache_writes
 
@@ -55,9 +64,11 @@ class StreamingGenerator:
                                                 cfg.dim // cfg.num_heads, self.kv_quant_config, self.device)
 
     @torch.no_grad()
-    def generate(self, noise: torch.Tensor, context: torch.Tensor, on_chunk=None) -> torch.Tensor:
-        """noise [1, F, C, H, W] bf16 latents, context [L, text_dim] bf16 -> denoised latents of the
-        same shape.  ``on_chunk(index)`` is called after each chunk (timing hooks)."""
+    def generate(self, noise: torch.Tensor, context, on_chunk=None, scene_cuts=()) -> torch.Tensor:
+        """noise [1, F, C, H, W] bf16 latents, context [L, text_dim] bf16 (or one such tensor per chunk) ->
+        denoised latents of the same shape.  ``on_chunk(index)`` is called after each chunk (timing hooks).
+        ``scene_cuts``: indices of the chunks that open a new scene (the reference recognises them by a prefix
+        of the chunk's prompt, :974-996); they matter in multi-shot mode only."""
         cfg = self.cfg
         _, F, C, H, W = noise.shape
         fs = (H // cfg.patch_size[1]) * (W // cfg.patch_size[2])
@@ -67,10 +78,17 @@ class StreamingGenerator:
         nb = cfg.num_frame_per_block
         # projected text K / V per layer: one prompt per call, so they are computed by the first forward only
         xcache = [{"is_init": False} for _ in range(cfg.num_layers)] if self.cache_text_kv else None
+        contexts = list(context) if isinstance(context, (list, tuple)) else None
+        scene_cuts = {int(c) for c in scene_cuts}
         sigmas = [t / 1000.0 for t in self.timesteps] + [0.0]
         for ci, start in enumerate(range(0, F, nb)):
             x = noise[0, start:start + nb].transpose(0, 1).contiguous()  # [C, f, H, W]
             f = x.shape[1]
+            if contexts is not None:
+                if ci > 0 and contexts[ci] is not contexts[ci - 1] and xcache is not None:
+                    xcache = [{"is_init": False} for _ in range(cfg.num_layers)]  # new prompt: re-project its K / V
+                context = contexts[ci]
+            is_scene_cut = self.multi_shot_sink and cfg.sink_size > 0 and ci > 0 and ci in scene_cuts
             if self.sampler == "unipc":
                 scheduler = FlowUniPCMultistepScheduler(num_train_timesteps=1000, shift=1)
                 scheduler.set_timesteps(len(self.timesteps), device=self.device, shift=self.sample_shift)
@@ -90,8 +108,12 @@ class StreamingGenerator:
                     x = (x.float() + (sigmas[si + 1] - sigmas[si]) * flow.float()).to(noise.dtype)
             out[0, start:start + f] = x.transpose(0, 1)
             # clean-context pass: rewrites this chunk's K / V in the cache
+            if is_scene_cut and self.shot_clean_recache:
+                kvc.zero_kv_data(self.kv_cache, start * fs, self.global_sink_size * fs)
             self.model(x, torch.zeros((1, f), device=self.device), context, self.kv_cache, start * fs,
                        crossattn_cache=xcache)
+            if is_scene_cut:
+                kvc.pin_current_chunk(self.kv_cache, f * fs, cfg.sink_size * fs)
             if on_chunk is not None:
                 on_chunk(ci)
         return out

@@ -41,6 +41,7 @@ class DiTConfig:
     num_frame_per_block: int = 3
     local_attn_size: int = 15   # frames kept in the KV cache (sink + window)
     sink_size: int = 3          # frames
+    global_sink_size: int = 0   # frames anchored for good (the pipeline sets it to sink_size in multi-shot mode)
 
 
 class WanRMSNorm(nn.Module):
@@ -119,8 +120,9 @@ class CausalSelfAttention(nn.Module):
         self.norm_q, self.norm_k = WanRMSNorm(dim, eps), WanRMSNorm(dim, eps)
 
     def forward(self, x, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size, *, input_amax=None,
-                residual=None, gate=None, gate_rows=0):
+                residual=None, gate=None, gate_rows=0, global_sink_tokens=0):
         """``input_amax``: the amax ticket the producer of ``x`` was given, if any.
+        ``global_sink_tokens``: leading tokens of the stream that stay in the cache for good (multi-shot mode).
         ``residual`` [B, L, C] (with ``gate`` [B*F, C], ``gate_rows`` tokens per gate row) turns the result into
         ``residual + out * gate``, folded into the output projection."""
         b, s = x.shape[:2]
@@ -146,7 +148,7 @@ class CausalSelfAttention(nn.Module):
         out_amax = _native.amax_ticket(x.device) if isinstance(self.o, FourOverSixLinear) else None
         out, update = kvc.kv_cache_attention(roped_q, roped_k, v, kv_cache, current_start, sink_tokens,
                                              max_attention_size=max_attention_size, smoothed_key=smooth_k,
-                                             amax_out=out_amax)
+                                             amax_out=out_amax, global_sink_tokens=global_sink_tokens)
         return _project_out(self.o, out.flatten(2), out_amax, residual, gate, gate_rows), update
 
 
@@ -205,7 +207,7 @@ class DiTBlock(nn.Module):
         return _project_out(down, h, h_amax, residual, gate, gate_rows)
 
     def forward(self, x, e, cos, sin, context, kv_cache, current_start, sink_tokens, max_attention_size=None,
-                crossattn_cache=None):
+                crossattn_cache=None, global_sink_tokens=0):
         """x [1, L, C]; e [1, F, 6, C]; returns (x, (current_end, local_end_index, cache_update_info)).
         The tensor amax that each activation quantization needs is produced by the kernel that writes the
         activation wherever that kernel is one of this package's."""
@@ -215,7 +217,8 @@ class DiTBlock(nn.Module):
         y_amax = _native.amax_ticket(x.device) if isinstance(self.self_attn.q, FourOverSixLinear) else None
         y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.eps, amax_out=y_amax)
         x, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size,
-                                   input_amax=y_amax, residual=x, gate=gates[0], gate_rows=frame_seqlen)
+                                   input_amax=y_amax, residual=x, gate=gates[0], gate_rows=frame_seqlen,
+                                   global_sink_tokens=global_sink_tokens)
         x = self.cross_attn(self.norm3(x), context, crossattn_cache, residual=x)
         y_amax = _native.amax_ticket(x.device) if isinstance(self.ffn[0], FourOverSixLinear) else None
         y = adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps, amax_out=y_amax)
@@ -255,6 +258,7 @@ class CausalDiT(nn.Module):
         self.blocks = nn.ModuleList([DiTBlock(cfg.dim, cfg.ffn_dim, cfg.num_heads, cfg.eps) for _ in range(cfg.num_layers)])
         self.head = CausalHead(cfg.dim, cfg.out_dim, cfg.patch_size, cfg.eps)
         self.rope_angles = build_rope_angles(cfg.dim // cfg.num_heads)
+        self.global_sink_size = cfg.global_sink_size  # frames; the generator overrides it like the reference pipeline
         self.kv_quant_config = None
         self._rope_cache: dict = {}
         self.init_weights()
@@ -314,7 +318,8 @@ class CausalDiT(nn.Module):
         updates = []
         for i, block in enumerate(self.blocks):
             x, upd = block(x, e0, cos, sin, ctx, kv_cache[i], current_start, sink_tokens, max_attn,
-                           None if crossattn_cache is None else crossattn_cache[i])
+                           None if crossattn_cache is None else crossattn_cache[i],
+                           global_sink_tokens=self.global_sink_size * frame_seqlen)
             updates.append(upd)
         if apply_cache_updates:
             for i, (cur_end, loc_end, info) in enumerate(updates):

@@ -3,7 +3,8 @@
 Same cache dictionary as the reference pipeline allocates
 (pipeline/causal_diffusion_inference.py:767-813) and the same cache policy as
 ``CausalWanSelfAttention.forward`` / ``CausalWanModel._apply_cache_updates``
-(wan_5b/modules/causal_model.py:491-724, 1371-1483), for whole-block sinks and windows.  Where the
+(wan_5b/modules/causal_model.py:491-724, 1371-1483) including the global sink, the multi-shot pinned region
+and the scene-cut handling of the pipeline, for whole-block sinks and windows.  Where the
 reference dequantizes all slots to bf16, copies the chunk in and calls flash attention, this
 module hands the slot list and the chunk's bf16 K/V to one kernel that decodes FP4 tiles on load.
 """
@@ -38,10 +39,12 @@ def initialize_kv_cache(num_layers: int, block_token_size: int, max_blocks: int,
             "local_end_index": torch.tensor([0], dtype=torch.long, device=device),
             "pinned_start": torch.tensor([-1], dtype=torch.long, device=device),
             "pinned_len": torch.tensor([0], dtype=torch.long, device=device),
-            # host copies of the two indices: the reference publishes them once per forward to avoid
+            # host copies of the four scalars: the reference publishes them once per forward to avoid
             # device syncs (utils/wan_5b_wrapper.py:355-366); here they are kept in step on the host
             "_global_end": 0,
             "_local_end": 0,
+            "_pinned_start": -1,
+            "_pinned_len": 0,
             "_tables": {},
         })
     return cache
@@ -58,54 +61,84 @@ def _tables_for(cache: dict, slot_ids: tuple[int, ...]):
 
 
 def plan_cache_step(cache: dict, current_start: int, num_new_tokens: int, sink_tokens: int,
-                    max_attention_size: int | None = None):
-    """Host-side cache policy for one forward of one layer: which slots are attended (in order) and
-    what ``_apply_cache_updates`` must do afterwards.  Returns (slot_ids, update_info, local_end)."""
+                    max_attention_size: int | None = None, global_sink_tokens: int = 0):
+    """Host-side cache policy for one forward of one layer (wan_5b/modules/causal_model.py:491-674): which
+    slots are attended, in order, and what ``_apply_cache_updates`` must do afterwards.
+    Returns (slot_ids, update_info, local_end).
+
+    The protected prefix of the buffer is the global sink (``global_sink_tokens``, never moves) plus the
+    multi-shot pinned region when it sits right behind it; a pinned region elsewhere floats: rolling shifts it
+    with the data until it reaches the prefix.  Without a pinned region the prefix is
+    ``max(global_sink_tokens, sink_tokens)``.  The attended keys are [prefix] + [floating pinned region, when it
+    lies before the window] + [the most recent tokens that fit ``max_attention_size``], the chunk itself last.
+    Everything has to fall on block boundaries, since a slot is quantized as a whole."""
     blk = cache["block_token_size"]
     size = cache["max_blocks"] * blk
     g_end, l_end = cache["_global_end"], cache["_local_end"]
+    ps, pl = cache["_pinned_start"], cache["_pinned_len"]
     current_end = current_start + num_new_tokens
-    if num_new_tokens % blk or sink_tokens % blk:
+    if num_new_tokens % blk or sink_tokens % blk or global_sink_tokens % blk:
         raise NotImplementedError("the FP4 KV cache works on whole blocks: chunk and sink sizes must be "
                                   f"multiples of block_token_size={blk}")
+    has_pinned = ps >= 0 and pl > 0
+    if has_pinned and ps == global_sink_tokens:
+        effective_sink = global_sink_tokens + pl
+    elif has_pinned:
+        effective_sink = global_sink_tokens
+    else:
+        effective_sink = max(global_sink_tokens, sink_tokens)
     if current_end > g_end and num_new_tokens + l_end > size:
         evicted = num_new_tokens + l_end - size
-        rolled = l_end - evicted - sink_tokens
+        rolled = l_end - evicted - effective_sink
         local_end = l_end + current_end - g_end - evicted
         local_start = local_end - num_new_tokens
-        if evicted % blk or rolled % blk or rolled < 0:
+        if evicted % blk or rolled % blk or rolled < 0 or effective_sink % blk:
             raise NotImplementedError("cache roll must move whole blocks")
-        sink_b, ev_b, roll_b = sink_tokens // blk, evicted // blk, rolled // blk
-        slot_ids = tuple(range(sink_b)) + tuple(range(sink_b + ev_b, sink_b + ev_b + roll_b))
-        info = {"action": "roll_and_insert", "sink_tokens": sink_tokens, "num_rolled_tokens": rolled,
+        info = {"action": "roll_and_insert", "sink_tokens": effective_sink, "num_rolled_tokens": rolled,
                 "num_evicted_tokens": evicted, "local_start_index": local_start, "local_end_index": local_end,
-                "current_end": current_end, "pinned_shift": 0}
+                "current_end": current_end,
+                "pinned_shift": evicted if (has_pinned and ps >= effective_sink) else 0}
     else:
+        evicted = rolled = 0
         local_end = l_end + current_end - g_end
         local_start = local_end - num_new_tokens
-        if local_start % blk or local_start < 0:
-            raise NotImplementedError("chunks must start on a block boundary of the cache")
-        slot_ids = tuple(range(local_start // blk))
         info = {"action": "direct_insert", "local_start_index": local_start, "local_end_index": local_end,
                 "current_end": current_end, "pinned_shift": 0}
-    if max_attention_size is not None and local_end - max_attention_size > 0:
-        # sliding window shorter than the cache: keep the sink blocks, then the most recent blocks
-        window_start = local_end - max_attention_size
-        if window_start % blk or max_attention_size % blk:
-            raise NotImplementedError("attention window must cover whole blocks")
-        n_cached_blocks = (max_attention_size - num_new_tokens) // blk
-        sink_b = sink_tokens // blk
-        keep_tail = max(n_cached_blocks - sink_b, 0)
-        head = slot_ids[:min(sink_b, n_cached_blocks)]
-        tail = slot_ids[len(slot_ids) - keep_tail:] if keep_tail else ()
-        slot_ids = tuple(dict.fromkeys(head + tuple(t for t in tail if t not in head)))
+    if local_start % blk or local_start < 0 or local_end > size:
+        raise NotImplementedError("chunks must start on a block boundary of the cache and fit into it")
+
+    def slots(a: int, b: int) -> tuple[int, ...]:
+        """Slots that hold rows a..b of the buffer as it will look after the roll."""
+        if a % blk or b % blk or b > local_start:
+            raise NotImplementedError("attended ranges must cover whole cached blocks")
+        ids = []
+        for p in range(a, b, blk):
+            ids.append((p + evicted if effective_sink <= p < effective_sink + rolled else p) // blk)
+        return tuple(ids)
+
+    window = size if max_attention_size is None else max_attention_size
+    window_start = max(0, local_end - window)
+    prepend_sink = effective_sink > 0 and window_start > 0
+    # the reference slices the rolled buffer with the not yet shifted pinned_start (:651-671)
+    prepend_pinned = has_pinned and effective_sink <= ps < window_start
+    if prepend_sink and prepend_pinned:
+        lws = max(effective_sink, local_end - (window - effective_sink - pl))
+        slot_ids = slots(0, effective_sink) + slots(ps, ps + pl) + slots(lws, local_start)
+    elif prepend_sink:
+        lws = max(effective_sink, local_end - (window - effective_sink))
+        slot_ids = slots(0, effective_sink) + slots(lws, local_start)
+    elif prepend_pinned:
+        lws = max(0, local_end - (window - pl))
+        slot_ids = slots(ps, ps + pl) + slots(lws, local_start)
+    else:
+        slot_ids = slots(window_start, local_start)
     return slot_ids, info, local_end
 
 
 def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Tensor, cache: dict,
                        current_start: int, sink_tokens: int, softmax_scale: float | None = None,
                        max_attention_size: int | None = None, smoothed_key: torch.Tensor | None = None,
-                       amax_out=None):
+                       amax_out=None, global_sink_tokens: int = 0):
     """Self-attention of one chunk against the FP4 cache.
 
     q, key_to_cache (RoPE'd, un-smoothed), v: bf16 [1, S, H, 128].  Attends
@@ -119,7 +152,8 @@ def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Ten
     if q.shape[0] != 1:
         raise ValueError("the quantized KV cache holds one sequence (batch size 1)")
     S, H, D = q.shape[1:]
-    slot_ids, info, local_end = plan_cache_step(cache, current_start, S, sink_tokens, max_attention_size)
+    slot_ids, info, local_end = plan_cache_step(cache, current_start, S, sink_tokens, max_attention_size,
+                                                global_sink_tokens)
     info["new_k"], info["new_v"] = key_to_cache, v
     k_new = (k_smooth(key_to_cache) if smoothed_key is None else smoothed_key)[0]
     scale = D ** -0.5 if softmax_scale is None else softmax_scale
@@ -146,6 +180,9 @@ def apply_cache_update(cache: dict, current_end: int, local_end_index: int, info
             for i in range(info["num_rolled_tokens"] // blk):
                 copy_quantized_into(cache["k"][sink_b + i], cache["k"][sink_b + ev_b + i])
                 copy_quantized_into(cache["v"][sink_b + i], cache["v"][sink_b + ev_b + i])
+            if info.get("pinned_shift", 0) > 0:  # a floating pinned region moves with the data (:1437-1443)
+                cache["pinned_start"].sub_(info["pinned_shift"])
+                cache["_pinned_start"] -= info["pinned_shift"]
         start_blk = info["local_start_index"] // blk
         n_insert = (info["local_end_index"] - info["local_start_index"]) // blk
         rule = kv_quant_config.scale_rule.value
@@ -158,3 +195,26 @@ def apply_cache_update(cache: dict, current_end: int, local_end_index: int, info
     cache["local_end_index"].fill_(local_end_index)
     cache["_global_end"] = current_end
     cache["_local_end"] = local_end_index
+
+
+def pin_current_chunk(kv_cache: list[dict], chunk_tokens: int, sink_tokens: int) -> None:
+    """Scene cut with a multi-shot sink: the chunk written last becomes the pinned region of every layer
+    (pipeline/causal_diffusion_inference.py:1017-1033).  Nothing is copied; from the next roll on the region
+    is protected like the sink once it has floated to the front."""
+    for cache in kv_cache:
+        start, length = cache["_local_end"] - chunk_tokens, min(sink_tokens, chunk_tokens)
+        cache["pinned_start"].fill_(start)
+        cache["pinned_len"].fill_(length)
+        cache["_pinned_start"], cache["_pinned_len"] = start, length
+
+
+def zero_kv_data(kv_cache: list[dict], current_start_tokens: int, global_sink_tokens: int) -> None:
+    """Scene cut with clean recache: forget everything but the global sink, so that the chunk's clean-context
+    forward re-enters it right behind the sink (pipeline/causal_diffusion_inference.py:1035-1043)."""
+    for cache in kv_cache:
+        cache["local_end_index"].fill_(global_sink_tokens)
+        cache["global_end_index"].fill_(current_start_tokens)
+        cache["pinned_start"].fill_(-1)
+        cache["pinned_len"].zero_()
+        cache["_local_end"], cache["_global_end"] = global_sink_tokens, current_start_tokens
+        cache["_pinned_start"], cache["_pinned_len"] = -1, 0

@@ -126,6 +126,50 @@ def test_cache_streaming_against_oracle(gpu, H, T, n_chunks, sink_blocks, max_bl
             assert np.array_equal(got_k[i * T:(i + 1) * T], ref_slots_k[i]), (c, i)
 
 
+@pytest.mark.parametrize("window_blocks,clean", [(5, False), (5, True), (4, False), (4, True)])
+def test_multi_shot_cache_streaming_against_the_policy_oracle(gpu, window_blocks, clean):
+    """Global sink + scene cuts (pinned chunk, optional clean recache) on the FP4 cache: in every forward the
+    kernel has to attend exactly the tokens the token-level policy oracle names, with the values the oracle's
+    quantize-on-write left for them."""
+    import cache_policy_oracle as cpo
+
+    H, T, max_blocks, n_chunks, cuts = 2, 64, 5, 13, (3, 8)
+    sink = gsink = T
+    cache = kvc.initialize_kv_cache(1, T, max_blocks, H, 128, CFG, gpu)[0]
+    st = cpo.new_state(max_blocks * T)
+    content = {}   # chunk index -> (dequantized K, dequantized V) as last written
+    for c in range(n_chunks):
+        for fwd in range(2):
+            if fwd == 1 and c in cuts and clean:
+                cpo.zero_kv_data(st, c * T, gsink)
+                kvc.zero_kv_data([cache], c * T, gsink)
+            q, k, v = (_randn((1, T, H, 128), 1000 + 100 * c + 10 * fwd + s) for s in (1, 2, 3))
+            ids, upd = cpo.attend(st, c * T, T, sink, gsink, window_blocks * T)
+            out, (ce, le, info) = kvc.kv_cache_attention(q.to(gpu), k.to(gpu), v.to(gpu), cache, c * T, sink_tokens=sink,
+                                                         max_attention_size=window_blocks * T, global_sink_tokens=gsink)
+            chunks = [int(i) // T for i in ids[::T]]
+            assert chunks[-1] == c and all(list(ids[j * T:(j + 1) * T]) == list(range(ch * T, (ch + 1) * T))
+                                           for j, ch in enumerate(chunks))
+            ks = [content[ch][0] for ch in chunks[:-1]] + [o.k_smooth(k[0].float().numpy())]
+            vs = [content[ch][1] for ch in chunks[:-1]] + [v[0].float().numpy()]
+            ref = o.attention(q[0].float().numpy(), np.concatenate(ks), np.concatenate(vs))
+            err = np.abs(out[0].float().cpu().numpy() - ref).max()
+            assert err <= 2e-2, (c, fwd, chunks, err)
+            assert (le, info["action"], info["pinned_shift"]) == (upd[1], upd[2]["action"], upd[2]["pinned_shift"])
+            cpo.apply(st, upd)
+            kvc.apply_cache_update(cache, ce, le, info, CFG)
+            content[c] = (_oracle_slot(k[0])[0], _oracle_slot(v[0])[0])
+        if c in cuts:
+            cpo.pin_current_chunk(st, T, sink)
+            kvc.pin_current_chunk([cache], T, sink)
+        assert int(cache["pinned_start"]) == st["pinned_start"] and int(cache["local_end_index"]) == st["local_end"]
+    assert 0 in chunks and 8 in chunks   # the global sink and the last scene's first chunk are still attended
+    # the buffer itself: every row up to local_end holds the chunk the oracle says it holds
+    got_k = dequantize_kv_cache(cache["k"], max_blocks, H, T, torch.bfloat16, gpu)[0].float().cpu().numpy()
+    for b in range(st["local_end"] // T):
+        assert np.array_equal(got_k[b * T:(b + 1) * T], content[int(st["buf"][b * T]) // T][0]), b
+
+
 def test_rope_matches_oracle_bit_exact_and_complex_reference(gpu):
     f, h, w, N = 3, 4, 6, 5
     angles = build_rope_angles()

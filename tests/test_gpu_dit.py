@@ -252,6 +252,45 @@ def test_streaming_generator_small_end_to_end(gpu):
     assert torch.equal(gen3.generate(noise[:, :2], ctx), out[:, :2])
 
 
+@pytest.mark.parametrize("clean", [False, True])
+def test_streaming_generator_multi_shot_sink(gpu, clean):
+    """Multi-shot mode at reduced size: global sink = first block, scene cuts at chunks 2 and 5 (with and without
+    the clean recache).  The cache bookkeeping after the run has to equal the token-level policy oracle's, the
+    frames before the first cut must not depend on the mode, and a second prompt takes effect from its chunk on."""
+    import cache_policy_oracle as cpo
+
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=8, sink_size=2)
+    g = torch.Generator().manual_seed(6)
+    noise = torch.randn(1, 16, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx_a, ctx_b = (torch.randn(10, 64, generator=g).bfloat16().to(gpu) for _ in range(2))
+    contexts = [ctx_a] * 2 + [ctx_b] * 6
+    cuts = (2, 5)
+    gen = StreamingGenerator(cfg, gpu, seed=4, multi_shot_sink=True, shot_clean_recache=clean)
+    out = gen.generate(noise, contexts, scene_cuts=cuts)
+    assert torch.isfinite(out.float()).all()
+    plain = StreamingGenerator(cfg, gpu, seed=4).generate(noise, contexts)
+    assert torch.equal(out[:, :4], plain[:, :4])                  # nothing differs before the first roll / cut
+    assert not torch.equal(out[:, 12:], plain[:, 12:])            # the protected prefix changes what later chunks see
+    single = StreamingGenerator(cfg, gpu, seed=4).generate(noise, ctx_a)
+    assert torch.equal(plain[:, :4], single[:, :4]) and not torch.equal(plain[:, 4:6], single[:, 4:6])
+
+    blk, size = 2 * 64, 4 * 2 * 64
+    st = cpo.new_state(size)
+    for c in range(8):
+        if c in cuts and clean:
+            cpo.zero_kv_data(st, c * blk, blk)
+        ids, upd = cpo.attend(st, c * blk, blk, blk, blk, size)
+        cpo.apply(st, upd)
+        if c in cuts:
+            cpo.pin_current_chunk(st, blk, blk)
+    for cache in gen.kv_cache:
+        assert (cache["_global_end"], cache["_local_end"], cache["_pinned_start"], cache["_pinned_len"]) == \
+            (st["global_end"], st["local_end"], st["pinned_start"], st["pinned_len"])
+        assert int(cache["pinned_start"]) == st["pinned_start"] and int(cache["local_end_index"]) == st["local_end"]
+    assert st["pinned_start"] == blk or clean                     # the pinned chunk ends up right behind the sink
+
+
 def test_packed_nvfp4_checkpoint_round_trip(gpu, tmp_path):
     """Export a quantized generator as a packed NVFP4 checkpoint, load it into a fresh bf16 model
     (utils/inference_utils.py:186-218 order: swap linears, drop master weights, strict load) and check
