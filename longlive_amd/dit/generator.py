@@ -11,6 +11,7 @@ Multi-shot generation (:104-107, 630-665, 974-1043): with ``multi_shot_sink`` th
 the stream become a global sink that is never evicted, and the first chunk of every later scene (``scene_cuts``)
 is pinned after its clean-context pass, so that the new scene attends its own opening frames instead of the
 previous scene's; ``shot_clean_recache`` additionally forgets everything but the global sink before that pass.
+``use_relative_rope`` (:149, 316) caches K without RoPE and rotates the attended window by its own frame positions.
 
 Two samplers: ``"euler"`` steps the flow prediction over the given timesteps (the fixed 1000/750/500/250
 schedule of the benchmark configuration); ``"unipc"`` is the reference pipeline's own choice (:566-612,
@@ -31,7 +32,8 @@ class StreamingGenerator:
     def __init__(self, cfg: DiTConfig, device, timesteps=(1000.0, 750.0, 500.0, 250.0), seed: int = 0,
                  model_quant: dict | None = None, kv_scale_rule: str = "mse", cache_text_kv: bool = True,
                  skip_dead_cache_writes: bool = True, sampler: str = "euler", sample_shift: float = 5.0,
-                 multi_shot_sink: bool = False, shot_clean_recache: bool = False) -> None:
+                 multi_shot_sink: bool = False, shot_clean_recache: bool = False,
+                 use_relative_rope: bool = False) -> None:
         if sampler not in ("euler", "unipc"):
             raise ValueError(f"unknown sampler {sampler!r}")
         self.cfg, self.device = cfg, torch.device(device)
@@ -53,6 +55,8 @@ class StreamingGenerator:
         self.multi_shot_sink, self.shot_clean_recache = multi_shot_sink, shot_clean_recache
         self.global_sink_size = cfg.sink_size if multi_shot_sink else 0   # :107
         self.model.global_sink_size = self.global_sink_size
+        for block in self.model.blocks:                                   # :316
+            block.self_attn.use_relative_rope = use_relative_rope
         self.cache_text_kv = cache_text_kv
         self.skip_dead_cache_writes = skip_dead_cache_writes
 

@@ -118,17 +118,30 @@ class CausalSelfAttention(nn.Module):
         self.dim, self.num_heads, self.head_dim = dim, num_heads, dim // num_heads
         self.q, self.k, self.v, self.o = (nn.Linear(dim, dim) for _ in range(4))
         self.norm_q, self.norm_k = WanRMSNorm(dim, eps), WanRMSNorm(dim, eps)
+        self.use_relative_rope = False  # set on the module by the pipeline (pipeline/causal_diffusion_inference.py:316)
 
     def forward(self, x, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size, *, input_amax=None,
-                residual=None, gate=None, gate_rows=0, global_sink_tokens=0):
+                residual=None, gate=None, gate_rows=0, global_sink_tokens=0, rope_fn=None):
         """``input_amax``: the amax ticket the producer of ``x`` was given, if any.
         ``global_sink_tokens``: leading tokens of the stream that stay in the cache for good (multi-shot mode).
+        ``rope_fn(frames, start_frame) -> (cos, sin)``: needed when ``use_relative_rope`` is set; the positions
+        then count frames of the attended window instead of frames of the stream.
         ``residual`` [B, L, C] (with ``gate`` [B*F, C], ``gate_rows`` tokens per gate row) turns the result into
         ``residual + out * gate``, folded into the output projection."""
         b, s = x.shape[:2]
         n, d = self.num_heads, self.head_dim
         q, k, v = _project_shared(x, [self.q, self.k, self.v], amax=input_amax)
         v = v.view(b, s, n, d)
+        if self.use_relative_rope:
+            if rope_fn is None:
+                raise ValueError("use_relative_rope needs rope_fn")
+            q = self.norm_q(q).view(b, s, n, d)
+            k = self.norm_k(k).view(b, s, n, d)
+            out_amax = None
+            out, update = kvc.kv_cache_attention_relative(q, k, v, kv_cache, current_start, sink_tokens, rope_fn,
+                                                          max_attention_size=max_attention_size,
+                                                          global_sink_tokens=global_sink_tokens)
+            return _project_out(self.o, out.flatten(2), out_amax, residual, gate, gate_rows), update
         if b == 1 and d == 128:
             # RMSNorm -> RoPE (-> K smoothing) of the reference in one pass over q and k
             if self.norm_q.eps == self.norm_k.eps:
@@ -207,7 +220,7 @@ class DiTBlock(nn.Module):
         return _project_out(down, h, h_amax, residual, gate, gate_rows)
 
     def forward(self, x, e, cos, sin, context, kv_cache, current_start, sink_tokens, max_attention_size=None,
-                crossattn_cache=None, global_sink_tokens=0):
+                crossattn_cache=None, global_sink_tokens=0, rope_fn=None):
         """x [1, L, C]; e [1, F, 6, C]; returns (x, (current_end, local_end_index, cache_update_info)).
         The tensor amax that each activation quantization needs is produced by the kernel that writes the
         activation wherever that kernel is one of this package's."""
@@ -218,7 +231,7 @@ class DiTBlock(nn.Module):
         y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.eps, amax_out=y_amax)
         x, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size,
                                    input_amax=y_amax, residual=x, gate=gates[0], gate_rows=frame_seqlen,
-                                   global_sink_tokens=global_sink_tokens)
+                                   global_sink_tokens=global_sink_tokens, rope_fn=rope_fn)
         x = self.cross_attn(self.norm3(x), context, crossattn_cache, residual=x)
         y_amax = _native.amax_ticket(x.device) if isinstance(self.ffn[0], FourOverSixLinear) else None
         y = adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps, amax_out=y_amax)
@@ -319,7 +332,8 @@ class CausalDiT(nn.Module):
         for i, block in enumerate(self.blocks):
             x, upd = block(x, e0, cos, sin, ctx, kv_cache[i], current_start, sink_tokens, max_attn,
                            None if crossattn_cache is None else crossattn_cache[i],
-                           global_sink_tokens=self.global_sink_size * frame_seqlen)
+                           global_sink_tokens=self.global_sink_size * frame_seqlen,
+                           rope_fn=lambda frames, first: self._rope(frames, h, w, first, x.device))
             updates.append(upd)
         if apply_cache_updates:
             for i, (cur_end, loc_end, info) in enumerate(updates):

@@ -169,6 +169,44 @@ def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Ten
     return out.unsqueeze(0), (current_start + S, local_end, info)
 
 
+def kv_cache_attention_relative(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache: dict, current_start: int,
+                                sink_tokens: int, rope_fn, softmax_scale: float | None = None,
+                                max_attention_size: int | None = None, global_sink_tokens: int = 0):
+    """Self-attention of one chunk with *relative* RoPE (wan_5b/modules/causal_model.py:486-487, 716-771): the
+    cache holds K without RoPE, and the rotation is applied to the attended window at attention time with the
+    frame positions 0, 1, ... of the window itself (sink first), the chunk's queries sitting on its last frames.
+
+    q, k (RMS-normed, no RoPE), v: bf16 [1, S, H, 128]; ``rope_fn(frames, start_frame) -> (cos, sin)`` gives the
+    float32 tables of a (frames, h, w) grid.  As in the reference this path materialises the window: the attended
+    slots are dequantized to bf16 in one launch, concatenated with the smoothed chunk keys, rotated, and handed
+    to the plain bf16 attention kernel.  Returns the same tuple as ``kv_cache_attention``; ``new_k`` is the
+    un-rotated ``k``."""
+    if q.shape[0] != 1:
+        raise ValueError("the quantized KV cache holds one sequence (batch size 1)")
+    S, H, D = q.shape[1:]
+    frame_seqlen = rope_fn(1, 0)[0].shape[0]
+    if S % frame_seqlen or cache["block_token_size"] % frame_seqlen:
+        raise ValueError("chunks and cache blocks must hold whole frames")
+    slot_ids, info, local_end = plan_cache_step(cache, current_start, S, sink_tokens, max_attention_size,
+                                                global_sink_tokens)
+    info["new_k"], info["new_v"] = k, v
+    blk = cache["block_token_size"]
+    keys, values = [k_smooth(k)[0]], [v[0]]
+    if slot_ids:
+        from .quant import dequantize_kv_cache
+        n = len(slot_ids)
+        keys.insert(0, dequantize_kv_cache([cache["k"][i] for i in slot_ids], n, H, blk, q.dtype, q.device)[0])
+        values.insert(0, dequantize_kv_cache([cache["v"][i] for i in slot_ids], n, H, blk, q.dtype, q.device)[0])
+    window_k, window_v = torch.cat(keys), torch.cat(values)
+    window_frames, new_frames = window_k.shape[0] // frame_seqlen, S // frame_seqlen
+    from .rope import rope_apply
+    roped_k = rope_apply(window_k, *rope_fn(window_frames, 0))
+    roped_q = rope_apply(q[0].contiguous(), *rope_fn(new_frames, window_frames - new_frames))
+    scale = D ** -0.5 if softmax_scale is None else softmax_scale
+    out = _native.attention_bf16(roped_q, roped_k, window_v.contiguous(), scale)
+    return out.unsqueeze(0), (current_start + S, local_end, info)
+
+
 def apply_cache_update(cache: dict, current_end: int, local_end_index: int, info: dict | None,
                        kv_quant_config: QuantizationConfig) -> None:
     """Roll whole slots and quantize the chunk's K / V into their slots, in place."""

@@ -170,6 +170,47 @@ def test_multi_shot_cache_streaming_against_the_policy_oracle(gpu, window_blocks
         assert np.array_equal(got_k[b * T:(b + 1) * T], content[int(st["buf"][b * T]) // T][0]), b
 
 
+@pytest.mark.parametrize("window_blocks", [4, 3])
+def test_relative_rope_cache_streaming_against_oracle(gpu, window_blocks):
+    """Relative RoPE: the cache holds un-rotated K, and every forward rotates the attended window with the frame
+    positions of the window itself (queries on its last frames).  Oracle: policy oracle for the token list,
+    oracle quantize-on-write for the cached values, oracle RoPE over the window, textbook attention."""
+    import cache_policy_oracle as cpo
+
+    H, fh, fw, frames_per_block, max_blocks, n_chunks = 2, 4, 4, 4, 4, 7
+    fs = fh * fw
+    T = frames_per_block * fs
+    sink = T
+    angles = build_rope_angles(128)
+
+    def rope_fn(frames, first):
+        return rope_cos_sin(angles, frames, fh, fw, first, gpu)
+
+    cache = kvc.initialize_kv_cache(1, T, max_blocks, H, 128, CFG, gpu)[0]
+    st = cpo.new_state(max_blocks * T)
+    content = {}
+    for c in range(n_chunks):
+        for fwd in range(2):
+            q, k, v = (_randn((1, T, H, 128), 2000 + 100 * c + 10 * fwd + s) for s in (1, 2, 3))
+            ids, upd = cpo.attend(st, c * T, T, sink, 0, window_blocks * T)
+            out, (ce, le, info) = kvc.kv_cache_attention_relative(q.to(gpu), k.to(gpu), v.to(gpu), cache, c * T, sink, rope_fn,
+                                                                  max_attention_size=window_blocks * T)
+            chunks = [int(i) // T for i in ids[::T]]
+            wk = np.concatenate([content[ch][0] for ch in chunks[:-1]] + [o.k_smooth(k[0].float().numpy())])
+            wv = np.concatenate([content[ch][1] for ch in chunks[:-1]] + [v[0].float().numpy()])
+            wf = len(chunks) * frames_per_block
+            rk = o.rope_apply(wk, *o.rope_cos_sin(wf, fh, fw, 0))
+            rq = o.rope_apply(q[0].float().numpy(), *o.rope_cos_sin(frames_per_block, fh, fw, wf - frames_per_block))
+            ref = o.attention(rq, rk, wv)
+            err = np.abs(out[0].float().cpu().numpy() - ref).max()
+            assert err <= 2e-2, (c, fwd, chunks, err)
+            assert torch.equal(info["new_k"].cpu(), k)      # what goes into the cache is the un-rotated key
+            cpo.apply(st, upd)
+            kvc.apply_cache_update(cache, ce, le, info, CFG)
+            content[c] = (_oracle_slot(k[0])[0], _oracle_slot(v[0])[0])
+    assert chunks == ([0, 4, 5, 6] if window_blocks == 4 else [0, 5, 6])
+
+
 def test_rope_matches_oracle_bit_exact_and_complex_reference(gpu):
     f, h, w, N = 3, 4, 6, 5
     angles = build_rope_angles()

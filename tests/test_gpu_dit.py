@@ -291,6 +291,23 @@ def test_streaming_generator_multi_shot_sink(gpu, clean):
     assert st["pinned_start"] == blk or clean                     # the pinned chunk ends up right behind the sink
 
 
+def test_streaming_generator_relative_rope(gpu):
+    """While the window still starts at frame 0 of the stream, relative and absolute positions coincide, so the
+    two modes may only differ by the bf16 rounding of cached-then-rotated keys."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    g = torch.Generator().manual_seed(8)
+    noise = torch.randn(1, 12, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    gen_rel, gen_abs = StreamingGenerator(cfg, gpu, seed=4, use_relative_rope=True), StreamingGenerator(cfg, gpu, seed=4)
+    rel, ab = gen_rel.generate(noise, ctx), gen_abs.generate(noise, ctx)
+    assert torch.isfinite(rel.float()).all()
+    early = (rel[:, :6].float() - ab[:, :6].float()).abs().max().item()
+    scale = ab.float().abs().max().item()
+    assert early <= 0.06 * scale, (early, scale)
+    assert gen_rel.kv_cache[0]["_local_end"] == gen_abs.kv_cache[0]["_local_end"] == 3 * 128
+
+
 def test_packed_nvfp4_checkpoint_round_trip(gpu, tmp_path):
     """Export a quantized generator as a packed NVFP4 checkpoint, load it into a fresh bf16 model
     (utils/inference_utils.py:186-218 order: swap linears, drop master weights, strict load) and check
