@@ -75,7 +75,7 @@ def plan_cache_step(cache: dict, current_start: int, num_new_tokens: int, sink_t
     blk = cache["block_token_size"]
     size = cache["max_blocks"] * blk
     g_end, l_end = cache["_global_end"], cache["_local_end"]
-    ps, pl = cache["_pinned_start"], cache["_pinned_len"]
+    ps, pl = cache.get("_pinned_start", -1), cache.get("_pinned_len", 0)
     current_end = current_start + num_new_tokens
     if num_new_tokens % blk or sink_tokens % blk or global_sink_tokens % blk:
         raise NotImplementedError("the FP4 KV cache works on whole blocks: chunk and sink sizes must be "
