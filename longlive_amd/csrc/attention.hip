@@ -9,10 +9,12 @@
 // 256 registers (64 for O^T, 32 for S^T, 32 for its Q fragments, the rest for tile fragments, raw FP4 data
 // and addressing), which is what lets two waves share a SIMD: while one wave converts FP4 data or evaluates
 // exponentials, the other one's MFMAs run.  Per iteration all 512 threads decode 128 keys of K and V
-// (e2m1 x e4m3 x amax/(6*256) -> bf16, the values the reference's dequantized bf16 cache holds) into LDS:
-// K row-major, V transposed.  The MFMAs compute S^T = K Q^T and O^T = V^T P^T (v_mfma_f32_32x32x16_bf16), so
-// every lane owns one query column: row max / row sum need no cross-lane traffic beyond one swap between the
-// wave halves, and the online-softmax rescale is a per-lane scalar.
+// (e2m1 x e4m3 x amax/(6*256) -> bf16, the values the reference's dequantized bf16 cache holds) into LDS, both
+// row-major (one row per key), with the same thread layout and the same byte offsets for K and V.  The MFMAs
+// compute S^T = K Q^T and O^T = V^T P^T (v_mfma_f32_32x32x16_bf16), so every lane owns one query column: row max /
+// row sum need no cross-lane traffic beyond one swap between the wave halves, and the online-softmax rescale is
+// a per-lane scalar.  The V^T operand (a lane needs eight consecutive keys of one head-dim column) comes out of
+// the row-major tile through ds_read_b64_tr_b16, the LDS read that transposes 16-bit elements across 16 lanes.
 #include "ll_common.h"
 
 namespace ll {
@@ -27,9 +29,9 @@ constexpr int kIterKeys = 2 * kTileKeys;       // keys decoded per iteration (on
 constexpr int kWgQueries = 128;
 constexpr int kWaveQueries = 32;
 constexpr int kKPitch = 272;                   // bytes per key row of K in LDS (256 + 16 pad)
-constexpr int kVPitch = 136;                   // bytes per d row of V^T in LDS (128 + 8 pad)
+constexpr int kVPitch = 288;                   // bytes per key row of V in LDS (256 + 32 pad: four rows of a transposing read hit 32 different banks)
 constexpr int kKTileBytes = kTileKeys * kKPitch;
-constexpr int kVTileBytes = kHeadDim * kVPitch;
+constexpr int kVTileBytes = kTileKeys * kVPitch;
 constexpr int kStageBytes = 2 * kKTileBytes + 2 * kVTileBytes;
 constexpr int kMaxSlots = 64;
 constexpr int kAttnThreads = 512;
@@ -88,13 +90,9 @@ __device__ __forceinline__ void fp4x8_to_f32(uint32_t w, float sf, float (&o)[8]
 // Raw FP4 data prefetched one iteration ahead.  Only packed bytes and scale bytes are held in registers
 // across the MFMA phase; everything else (slot scale, kind of key, bf16 source rows of the current chunk)
 // is re-derived from the key index when the data is decoded.
-struct KRaw {         // K of one key, one quarter of the head dimension (32 elements)
+struct KRaw {         // K or V of one key, one quarter of the head dimension (32 elements)
   uint4 v;            // 16 packed bytes
   uint32_t scales;    // 2 e4m3 block scales (low 16 bits)
-};
-struct VRaw {         // V of one key, half a 16-element block
-  uint32_t v;         // 4 packed bytes
-  uint32_t scale;     // e4m3 block scale byte
 };
 
 // Load through a pointer that is known to address global memory.  Slot pointers come out of a table, so
@@ -112,18 +110,14 @@ __device__ __forceinline__ uint4 load_global_b128(const void* ptr) {
 
 // Raw FP4 loads.  vo / so are byte offsets of the thread's data inside the slot's value / scale arrays;
 // the caller keeps them up to date incrementally (both advance by a constant per iteration inside a slot).
-__device__ __forceinline__ void fetch_k(const SlotTable& tab, int slot, uint32_t vo, uint32_t so, KRaw& f) {
-  f.v = load_global_b128(tab.kv[slot] + vo);
-  f.scales = load_global<uint16_t>(tab.ks[slot] + so);
-}
-__device__ __forceinline__ void fetch_v(const SlotTable& tab, int slot, uint32_t vo, uint32_t so, VRaw& f) {
-  f.v = load_global<uint32_t>(tab.vv[slot] + vo);
-  f.scale = load_global<uint8_t>(tab.vs[slot] + so);
+__device__ __forceinline__ void fetch_row(const uint8_t* values, const uint8_t* scales, uint32_t vo, uint32_t so, KRaw& f) {
+  f.v = load_global_b128(values + vo);
+  f.scales = load_global<uint16_t>(scales + so);
 }
 
-// Decode K (32 elements of one key) to bf16 and store the 64 bytes into the key's LDS row.
+// Decode 32 elements of one key (K or V) to bf16 and store the 64 bytes into the key's LDS row.
 // kind: 0 = fp4 slot data in f (gs = slot amax / (e2m1_max * e4m3_max)), 1 = bf16 row at src, 2 = zeros.
-__device__ __forceinline__ void store_k(const KRaw& f, int kind, float gs, const uint4* src, uint8_t* dst) {
+__device__ __forceinline__ void store_row(const KRaw& f, int kind, float gs, const uint4* src, uint8_t* dst) {
   uint4* d4 = reinterpret_cast<uint4*>(dst);
   if (kind == 0) {
     const uint32_t w[4] = {f.v.x, f.v.y, f.v.z, f.v.w};
@@ -140,39 +134,6 @@ __device__ __forceinline__ void store_k(const KRaw& f, int kind, float gs, const
   } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i) d4[i] = make_uint4(0, 0, 0, 0);
-  }
-}
-
-// 8 head-dim elements of 4 consecutive keys -> for every element one 8-byte run of 4 bf16 along the key
-// axis, written into the transposed V tile.  vt_tile points at the tile, row0 = first d row.
-// kind / gs / src per key as in store_k (src = the key's 8 bf16 elements).
-__device__ __forceinline__ void store_v4(const VRaw (&f)[4], const int (&kind)[4], const float (&gs)[4],
-                                         const uint4* const (&src)[4], uint8_t* vt_tile, int row0, int chunk) {
-  uint32_t w[4][4];
-#pragma unroll
-  for (int kk = 0; kk < 4; ++kk) {
-    if (kind[kk] == 0) {
-      const float sf = fp8_byte_to_f32(f[kk].scale, 0) * gs[kk];
-      float v8[8];
-      fp4x8_to_f32(f[kk].v, sf, v8);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) w[kk][i] = pack_bf16(v8[2 * i], v8[2 * i + 1]);
-    } else if (kind[kk] == 1) {
-      const uint4 a = src[kk][0];
-      w[kk][0] = a.x; w[kk][1] = a.y; w[kk][2] = a.z; w[kk][3] = a.w;
-    } else {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) w[kk][i] = 0;
-    }
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const uint32_t e01 = __builtin_amdgcn_perm(w[1][i], w[0][i], 0x05040100u);
-    const uint32_t e23 = __builtin_amdgcn_perm(w[3][i], w[2][i], 0x05040100u);
-    const uint32_t o01 = __builtin_amdgcn_perm(w[1][i], w[0][i], 0x07060302u);
-    const uint32_t o23 = __builtin_amdgcn_perm(w[3][i], w[2][i], 0x07060302u);
-    *reinterpret_cast<uint2*>(vt_tile + (row0 + 2 * i) * kVPitch + chunk * 8) = make_uint2(e01, e23);
-    *reinterpret_cast<uint2*>(vt_tile + (row0 + 2 * i + 1) * kVPitch + chunk * 8) = make_uint2(o01, o23);
   }
 }
 
@@ -219,64 +180,37 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   const int n_iter = (int)((p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys);
   __syncthreads();
 
-  // ---- decode plan.  K: thread = (key_local = tid / 4, quarter of the head dim = tid % 4).
-  //                    V: key tile = wave / 4; a thread owns 8 elements (half lane / 32 of the 16-element
-  //                       block 2 (wave % 4) + lane / 16 % 2) of 4 consecutive keys 4 (lane % 16): for one
-  //                       head-dim row 16 lanes write one full 128-byte row of V^T, which the 136-byte pitch
-  //                       spreads over all LDS banks.
+  // ---- decode plan.  Thread = (key_local = tid / 4, quarter of the head dim = tid % 4), the same for K and V.
   // Schedule of iteration `it`: the MFMAs work on LDS stage it & 1 while the raw FP4 bytes of iteration
   // it + 1 (already in registers) are decoded into the other stage during the S phase.  As soon as the raw
   // registers are free the bytes of iteration it + 2 are requested, which gives each load most of an
   // iteration to land.  Position of the data the raw registers hold (or will hold next): iter_base = first
-  // key of that iteration; per thread the K key iter_base + k_local and the four V keys
-  // iter_base + v_local + 0..3, each as (slot, offset in slot) plus the byte offsets of its packed values and
-  // scale(s) in the slot.
-  KRaw kf;
-  VRaw vf[4];
+  // key of that iteration; per thread the key iter_base + k_local as (slot, offset in slot) plus the byte
+  // offsets of its packed values and scales in the slot, which K and V share.
+  KRaw kf, vf;
   const int n_cached = (int)p.n_cached, Lk_i = (int)(p.n_cached + p.n_new);
-  // lanes 0-31 of a wave (one pass of an 8-byte LDS write) get rows 16 apart = 32 banks apart
-  const int v_blk = 2 * (wave & 3) + ((lane >> 4) & 1), v_half = lane >> 5;
-  const int v_chunk = lane & 15, v_tile = wave >> 2;
-  const int k_local = tid >> 2, k_quarter = tid & 3, v_local = v_tile * kTileKeys + 4 * v_chunk;
+  const int k_local = tid >> 2, k_quarter = tid & 3;
   const uint32_t row_bytes = (uint32_t)p.H * 64u;
   const uint32_t step_vo = (uint32_t)kIterKeys * row_bytes;
   const uint32_t step_so = (uint32_t)p.H * 1024u;
-  const uint32_t slot_bytes = (uint32_t)p.bts * row_bytes;
   const int k_dst_off = (k_local >> 6) * kKTileBytes + (k_local & 63) * kKPitch + k_quarter * 64;
-  const int v_row0 = v_blk * 16 + v_half * 8;
-  const int v_dst_off = 2 * kKTileBytes + v_tile * kVTileBytes + v_row0 * kVPitch + v_chunk * 8;
+  const int v_dst_off = 2 * kKTileBytes + (k_local >> 6) * kVTileBytes + (k_local & 63) * kVPitch + k_quarter * 64;
   int iter_base = 0;
   int k_slot = k_local / p.bts, k_off = k_local - k_slot * p.bts;
-  int v_slot = v_local / p.bts, v_off = v_local - v_slot * p.bts;
-  uint32_t k_vo, k_so, v_vo, v_so[4];
-  float k_gs, v_gs[4];  // slot scale amax / (e2m1_max * e4m3_max) of the thread's K key and of its four V keys
-  auto locate_k = [&]() __attribute__((always_inline)) {
+  uint32_t k_vo, k_so;
+  float k_gs, v_gs;  // slot scale amax / (e2m1_max * e4m3_max) of the thread's key, for K and for V
+  auto locate = [&]() __attribute__((always_inline)) {
     const int64_t row = (int64_t)k_off * p.H + head;
     k_vo = (uint32_t)row * 64u + k_quarter * 16u;
     k_so = (uint32_t)blocked_scale_offset(row, k_quarter * 2, 8);
     k_gs = tab.kg[min(k_slot, kMaxSlots - 1)];
+    v_gs = tab.vg[min(k_slot, kMaxSlots - 1)];
   };
-  auto locate_v = [&]() __attribute__((always_inline)) {
-    v_vo = ((uint32_t)v_off * p.H + head) * 64u + v_blk * 8u + v_half * 4u;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      int oo = v_off + kk;
-      if (oo >= p.bts) oo -= p.bts;
-      v_so[kk] = (uint32_t)blocked_scale_offset((int64_t)oo * p.H + head, v_blk, 8);
-      v_gs[kk] = tab.vg[min(v_slot + (v_off + kk >= p.bts ? 1 : 0), kMaxSlots - 1)];
-    }
-  };
-  locate_k();
-  locate_v();
-  auto fetch_k_next = [&]() __attribute__((always_inline)) {
-    if (iter_base + k_local < n_cached) fetch_k(tab, k_slot, k_vo, k_so, kf);
-  };
-  auto fetch_v_next = [&]() __attribute__((always_inline)) {
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const bool wrap = v_off + kk >= p.bts;
-      if (iter_base + v_local + kk < n_cached)
-        fetch_v(tab, v_slot + (wrap ? 1 : 0), v_vo + kk * row_bytes - (wrap ? slot_bytes : 0u), v_so[kk], vf[kk]);
+  locate();
+  auto fetch_next = [&]() __attribute__((always_inline)) {
+    if (iter_base + k_local < n_cached) {
+      fetch_row(tab.kv[k_slot], tab.ks[k_slot], k_vo, k_so, kf);
+      fetch_row(tab.vv[k_slot], tab.vs[k_slot], k_vo, k_so, vf);
     }
   };
   auto advance = [&]() __attribute__((always_inline)) {
@@ -289,40 +223,15 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
         k_off -= p.bts;
         ++k_slot;
       } while (k_off >= p.bts);
-      locate_k();
-    }
-    v_off += kIterKeys;
-    v_vo += step_vo;
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) v_so[kk] += step_so;
-    if (v_off + 3 >= p.bts) {
-      while (v_off >= p.bts) {
-        v_off -= p.bts;
-        ++v_slot;
-      }
-      locate_v();
+      locate();
     }
   };
-  auto decode_k_any = [&](int stage) __attribute__((always_inline)) {
-    const int k_key = iter_base + k_local;
-    const int kind = k_key < n_cached ? 0 : (k_key < Lk_i ? 1 : 2);
-    const float gs = kind == 0 ? k_gs : 0.0f;
-    const uint4* src = reinterpret_cast<const uint4*>(
-        p.k_new + ((int64_t)(k_key - n_cached) * p.H + head) * kHeadDim + k_quarter * 32);
-    store_k(kf, kind, gs, src, smem + stage * kStageBytes + k_dst_off);
-  };
-  auto decode_v_any = [&](int stage) __attribute__((always_inline)) {
-    int kind[4];
-    float gs[4];
-    const uint4* src[4];
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      const int key = iter_base + v_local + kk;
-      kind[kk] = key < n_cached ? 0 : (key < Lk_i ? 1 : 2);
-      gs[kk] = kind[kk] == 0 ? v_gs[kk] : 0.0f;
-      src[kk] = reinterpret_cast<const uint4*>(p.v_new + ((int64_t)(key - n_cached) * p.H + head) * kHeadDim + v_row0);
-    }
-    store_v4(vf, kind, gs, src, smem + stage * kStageBytes + 2 * kKTileBytes + v_tile * kVTileBytes, v_row0, v_chunk);
+  auto decode_any = [&](int stage) __attribute__((always_inline)) {
+    const int key = iter_base + k_local;
+    const int kind = key < n_cached ? 0 : (key < Lk_i ? 1 : 2);
+    const int64_t src_off = ((int64_t)(key - n_cached) * p.H + head) * kHeadDim + k_quarter * 32;
+    store_row(kf, kind, k_gs, reinterpret_cast<const uint4*>(p.k_new + src_off), smem + stage * kStageBytes + k_dst_off);
+    store_row(vf, kind, v_gs, reinterpret_cast<const uint4*>(p.v_new + src_off), smem + stage * kStageBytes + v_dst_off);
   };
 
   // Reference point of the exponentials.  m_run is not the exact running maximum: it is raised only when
@@ -370,17 +279,23 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       }
       dst = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
     };
-    auto read_v = [&](int step, uint2 (&dst)[4][2]) __attribute__((always_inline)) {
-      const int chunk0 = (step >> 1) * 8 + (step & 1) * 4 + lh;
+    // V^T fragment of step `step` (16 keys), head-dim tile dt: lane l needs column d = 32 dt + l % 32 for the keys
+    // 16 step + 8 j + 4 (l / 32) + 0..3 (j = 0, 1: the order of P's registers).  One transposing read serves a
+    // 16-lane group: source lane i points at row key0 + i / 4, columns d0 + 4 (i % 4) .. + 3, and every lane of
+    // the group receives column d0 + i of the four rows.
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) bf16x4* lds_bf16x4_t;
+    const uint8_t* vt_lane = vt_base + (4 * lh + ((lane & 15) >> 2)) * kVPitch + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+    auto read_v = [&](int step, bf16x4 (&dst)[4][2]) __attribute__((always_inline)) {
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt) {
-        const uint8_t* src = vt_base + (dt * 32 + l32) * kVPitch;
-        dst[dt][0] = *reinterpret_cast<const uint2*>(src + chunk0 * 8);
-        dst[dt][1] = *reinterpret_cast<const uint2*>(src + (chunk0 + 2) * 8);
-      }
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          dst[dt][j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+              (lds_bf16x4_t)(vt_lane + (16 * step + 8 * j) * kVPitch + dt * 64));
     };
     bf16x8 pb[2];
-    uint2 vfr[2][4][2];
+    bf16x4 vfr[2][4][2];
     read_v(0, vfr[0]);
     make_p(0, pb[0]);
     __builtin_amdgcn_sched_barrier(0);
@@ -389,8 +304,8 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       if (step < 3) read_v(step + 1, vfr[(step + 1) & 1]);
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) {
-        const uint2(&v)[2] = vfr[step & 1][dt];
-        const bf16x8 a = __builtin_bit_cast(bf16x8, make_uint4(v[0].x, v[0].y, v[1].x, v[1].y));
+        const bf16x4(&v)[2] = vfr[step & 1][dt];
+        const bf16x8 a = __builtin_shufflevector(v[0], v[1], 0, 1, 2, 3, 4, 5, 6, 7);
         o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, pb[step & 1], o[dt], 0, 0, 0);
       }
       if (step < 3) {
@@ -407,15 +322,10 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   };
 
   // prologue: stage 0 <- iteration 0, raw registers <- iteration 1
-  fetch_k_next();
-  fetch_v_next();
-  decode_k_any(0);
-  decode_v_any(0);
+  fetch_next();
+  decode_any(0);
   advance();
-  if (n_iter > 1) {
-    fetch_k_next();
-    fetch_v_next();
-  }
+  if (n_iter > 1) fetch_next();
   __syncthreads();
   // Every load issued so far (Q fragments, first tiles) has to have landed before the loop: otherwise the
   // compiler's wait-count bookkeeping carries them into the loop and makes the MFMA phase wait for the
@@ -424,8 +334,8 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
 
   // Iterations whose own 128 keys all exist and whose successor is all FP4 form a prefix of the key range;
   // they run the interleaved body: S^T (64 keys x 32 queries) = 16 MFMAs in eight steps of two, each step
-  // also converting one dword of the prefetched K row (even steps) or two elements of the prefetched V data
-  // for four keys (odd steps) into the other LDS stage.  The rest (the bf16 chunk, the tail) runs the plain
+  // also converting one dword of the prefetched K row (even steps) or V row (odd steps) into the other LDS
+  // stage.  The rest (the bf16 chunk, the tail) runs the plain
   // body in a loop of its own.
   int n_fast = n_cached / kIterKeys - 1;
   n_fast = n_fast < 0 ? 0 : (n_fast > n_iter ? n_iter : n_fast);
@@ -437,11 +347,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     const bool has_next2 = it + 2 < n_iter;
     float16v sc[2];
     {
-      const float gsk = k_gs;
-      float sfv[4];
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk) sfv[kk] = fp8_byte_to_f32(vf[kk].scale, 0) * v_gs[kk];
-      const uint32_t w[4] = {kf.v.x, kf.v.y, kf.v.z, kf.v.w};
+      const uint32_t wk[4] = {kf.v.x, kf.v.y, kf.v.z, kf.v.w}, wv[4] = {vf.v.x, vf.v.y, vf.v.z, vf.v.w};
       uint8_t* kdst = nxt + k_dst_off;
       uint8_t* vdst = nxt + v_dst_off;
       const uint8_t* krow0 = cur + kp * kKTileBytes + l32 * kKPitch + lh * 16;
@@ -461,42 +367,21 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
         const bf16x8 fa0 = __builtin_bit_cast(bf16x8, a0), fa1 = __builtin_bit_cast(bf16x8, a1);
         sc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, qf[ks], sc[0], 0, 0, 0);
         sc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, qf[ks], sc[1], 0, 0, 0);
-        if ((ks & 1) == 0) {  // K: dword ks / 2 of the quarter row
+        {  // one dword (8 elements) of the prefetched row per step: K in the even steps, V in the odd ones
           const int j = ks >> 1;
-          const float sf = fp8_byte_to_f32(kf.scales, j >> 1) * gsk;
+          const bool is_k = (ks & 1) == 0;
+          const float sf = fp8_byte_to_f32(is_k ? kf.scales : vf.scales, j >> 1) * (is_k ? k_gs : v_gs);
           float v8[8];
-          fp4x8_to_f32(w[j], sf, v8);
-          reinterpret_cast<uint4*>(kdst)[j] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
-                                                          pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
-        } else {  // V: elements 2 j, 2 j + 1 of the thread's 8, for its 4 keys -> two rows of V^T
-          const int j = ks >> 1;
-          float e[4][2];
-#pragma unroll
-          for (int kk = 0; kk < 4; ++kk) {
-            float2v q;
-            switch (j) {
-              case 0: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(vf[kk].v, 1.0f, 0); break;
-              case 1: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(vf[kk].v, 1.0f, 1); break;
-              case 2: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(vf[kk].v, 1.0f, 2); break;
-              default: q = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(vf[kk].v, 1.0f, 3); break;
-            }
-            e[kk][0] = q[0] * sfv[kk];
-            e[kk][1] = q[1] * sfv[kk];
-          }
-#pragma unroll
-          for (int jj = 0; jj < 2; ++jj)
-            *reinterpret_cast<uint2*>(vdst + (2 * j + jj) * kVPitch) =
-                make_uint2(pack_bf16(e[0][jj], e[1][jj]), pack_bf16(e[2][jj], e[3][jj]));
+          fp4x8_to_f32(is_k ? wk[j] : wv[j], sf, v8);
+          reinterpret_cast<uint4*>(is_k ? kdst : vdst)[j] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
+                                                                       pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
         }
         a0 = n0;
         a1 = n1;
       }
     }
     advance();
-    if (has_next2) {
-      fetch_k_next();
-      fetch_v_next();
-    }
+    if (has_next2) fetch_next();
     softmax_pv(sc, vt_base);
     __syncthreads();
   }
@@ -510,20 +395,20 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     const uint8_t* vt_base = cur + 2 * kKTileBytes + kp * kVTileBytes;
     const int tile_base = it * kIterKeys + kp * kTileKeys;
     // A successor that lies wholly in the bf16 chunk is brought in ahead of the MFMAs: its K rows go
-    // straight from global memory into the other stage (one 256-byte row per wave instruction, 16 rows per
-    // wave), its V pieces are requested now and transposed into LDS after the PV phase.
+    // and V rows go straight from global memory into the other stage (one 256-byte row per wave instruction,
+    // 16 rows of each per wave).
     const bool next_is_chunk = iter_base >= n_cached && iter_base + kIterKeys <= Lk_i;  // iter_base = first key of tile it + 1
-    uint4 vraw[4];
     if (next_is_chunk) {
       uint8_t* nxt = smem + ((it + 1) & 1) * kStageBytes;
-      const uint16_t* ksrc = p.k_new + ((int64_t)(iter_base + wave * 16 - n_cached) * p.H + head) * kHeadDim + lane * 2;
+      const int64_t src_off = ((int64_t)(iter_base + wave * 16 - n_cached) * p.H + head) * kHeadDim + lane * 2;
+      const int64_t src_step = (int64_t)p.H * kHeadDim;
       uint8_t* kdst = nxt + (wave >> 2) * kKTileBytes + ((wave & 3) * 16) * kKPitch;
+      uint8_t* vdst = nxt + 2 * kKTileBytes + (wave >> 2) * kVTileBytes + ((wave & 3) * 16) * kVPitch;
 #pragma unroll
-      for (int r = 0; r < 16; ++r)
-        __builtin_amdgcn_global_load_lds((gptr_t)(ksrc + (int64_t)r * p.H * kHeadDim), (lptr_t)(kdst + r * kKPitch), 4, 0, 0);
-#pragma unroll
-      for (int kk = 0; kk < 4; ++kk)
-        vraw[kk] = load_global_b128(p.v_new + ((int64_t)(iter_base + v_local + kk - n_cached) * p.H + head) * kHeadDim + v_row0);
+      for (int r = 0; r < 16; ++r) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(p.k_new + src_off + r * src_step), (lptr_t)(kdst + r * kKPitch), 4, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(p.v_new + src_off + r * src_step), (lptr_t)(vdst + r * kVPitch), 4, 0, 0);
+      }
     }
     if (tile_base < Lk_i) {
       float16v sc[2];
@@ -552,27 +437,12 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       softmax_pv(sc, vt_base);
     }
     if (next_is_chunk) {
-      uint8_t* vdst = smem + ((it + 1) & 1) * kStageBytes + v_dst_off;
-      const uint32_t w[4][4] = {{vraw[0].x, vraw[0].y, vraw[0].z, vraw[0].w}, {vraw[1].x, vraw[1].y, vraw[1].z, vraw[1].w},
-                                {vraw[2].x, vraw[2].y, vraw[2].z, vraw[2].w}, {vraw[3].x, vraw[3].y, vraw[3].z, vraw[3].w}};
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {  // elements 2 i, 2 i + 1 of the thread's 8, for its 4 keys -> two rows of V^T
-        // v_perm_b32: bytes 0-3 come from the second operand, 4-7 from the first
-        *reinterpret_cast<uint2*>(vdst + (2 * i) * kVPitch) =
-            make_uint2(__builtin_amdgcn_perm(w[1][i], w[0][i], 0x05040100u), __builtin_amdgcn_perm(w[3][i], w[2][i], 0x05040100u));
-        *reinterpret_cast<uint2*>(vdst + (2 * i + 1) * kVPitch) =
-            make_uint2(__builtin_amdgcn_perm(w[1][i], w[0][i], 0x07060302u), __builtin_amdgcn_perm(w[3][i], w[2][i], 0x07060302u));
-      }
       iter_base += kIterKeys;  // the slot bookkeeping of advance() has no use beyond the cache
-      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the K rows have landed in LDS
+      __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the rows have landed in LDS
     } else if (it + 1 < n_iter) {
-      decode_k_any((it + 1) & 1);
-      decode_v_any((it + 1) & 1);
+      decode_any((it + 1) & 1);
       advance();
-      if (it + 2 < n_iter) {
-        fetch_k_next();
-        fetch_v_next();
-      }
+      if (it + 2 < n_iter) fetch_next();
     }
     __syncthreads();
   }
