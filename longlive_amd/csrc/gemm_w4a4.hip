@@ -12,8 +12,11 @@
 //
 // Tiling: 256 threads = 4 waves in a 2x2 grid, each wave owns FA x FB MFMA tiles of 32x32
 // (workgroup tile = 64*FA rows of A by 64*FB rows of B), K step 128 (64 packed bytes per row),
-// two LDS stages filled through registers.  The kernel keeps to 256 registers per wave so that two
-// workgroups share a CU: while one wave decodes, another wave's MFMAs run.  K is consumed in a
+// two LDS stages filled straight from global memory (global_load_lds_dwordx4: no staging registers, no LDS
+// store instructions).  Such a load writes the 64 lanes' 16-byte pieces to consecutive LDS addresses, so rows are
+// unpadded (64 bytes) and the four pieces of a row are stored in the order piece ^ (row / 4 % 4), which spreads
+// the fragment reads of 16 consecutive rows over all banks.  The kernel keeps to 256 registers per wave so that
+// two workgroups share a CU: while one wave decodes, another wave's MFMAs run.  K is consumed in a
 // permuted order (lanes 0-31 and 32-63 take alternate 32-element runs), identical for A and B, so
 // the sum is unchanged.
 #include <stdlib.h>
@@ -22,13 +25,28 @@
 
 namespace ll {
 
+// sixteen zero bytes in global memory: what lanes load in place of K elements beyond the end of a row
+__device__ uint4 g_gemm_zero16;
+
+// 16 bytes per lane from global memory straight into LDS at lds_base + 16 * lane (lds_base wave-uniform).
+// Written as an asm statement on purpose: for the builtin the compiler's wait-count pass, which cannot tell the
+// two LDS stages apart, makes every later LDS read wait for the load, which would expose the whole memory latency
+// in every K step.  The kernel waits for these loads itself (vmcnt(0) ahead of the barrier that hands the stage
+// over) and issues no other vector-memory loads while they are in flight.
+__device__ __forceinline__ void load_to_lds_b128(const void* src, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(lds_base) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p);
+}
+
 typedef _Float16 half2v __attribute__((ext_vector_type(2)));
 typedef _Float16 half8v __attribute__((ext_vector_type(8)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 
 constexpr int kBK = 128;          // K elements per main-loop step
 constexpr int kRowBytes = 64;     // packed bytes per row per step
-constexpr int kLdsRow = 80;       // padded LDS row pitch (bank-conflict free for 16-byte reads)
+constexpr int kLdsRow = 64;       // LDS row pitch: unpadded, pieces swizzled (see above)
 constexpr int kGemmThreads = 256;
 
 // Decode 8 e2m1 codes (one dword) and scale them by the f16 pair (s, s).
@@ -104,94 +122,86 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
   const int wm = wave & 1, wn = wave >> 1;
   const int l32 = lane & 31, lh = lane >> 5;
 
-  // ---- global -> register staging plan
-  constexpr int kAChunks = BM * 4 / kGemmThreads;  // 16-byte chunks of A values per thread
+  // ---- global -> LDS plan.  Load instruction i of a wave covers the 1024 bytes (16 rows) at piece index
+  // i * 256 + wave * 64 of the A (or B) region; lane -> (row, stored position), and the piece of the row that
+  // belongs there is position ^ (row / 4 % 4).
+  constexpr int kAChunks = BM * 4 / kGemmThreads;  // 16-byte pieces of A values per thread
   constexpr int kBChunks = BN * 4 / kGemmThreads;
   const int64_t row_bytes = Kp >> 1;
   const uint8_t* a_src[kAChunks];
   const uint8_t* b_src[kBChunks];
-  int a_dst[kAChunks], b_dst[kBChunks];
+  bool tail_piece;  // the thread's pieces lie in the second 64 K elements of a step (the same for all its pieces)
+  {
+    const int q = tid, r = q >> 2;
+    tail_piece = (((q & 3) ^ ((r >> 2) & 3)) & 2) != 0;
+  }
 #pragma unroll
   for (int i = 0; i < kAChunks; ++i) {
-    const int q = tid + i * kGemmThreads, r = q >> 2, ck = q & 3;
+    const int q = tid + i * kGemmThreads, r = q >> 2, ck = (q & 3) ^ ((r >> 2) & 3);
     const int gr = min(row0 + r, Mp - 1);
     a_src[i] = Av + (int64_t)gr * row_bytes + ck * 16;
-    a_dst[i] = r * kLdsRow + ck * 16;
   }
 #pragma unroll
   for (int i = 0; i < kBChunks; ++i) {
-    const int q = tid + i * kGemmThreads, r = q >> 2, ck = q & 3;
+    const int q = tid + i * kGemmThreads, r = q >> 2, ck = (q & 3) ^ ((r >> 2) & 3);
     const int gr = min(col0 + r, Np - 1);
     b_src[i] = Bv + (int64_t)gr * row_bytes + ck * 16;
-    b_dst[i] = S::kAVals + r * kLdsRow + ck * 16;
   }
-  // scales: 1024 contiguous bytes per 128-row block per step (two 128x4 tiles) = 64 threads x 16 bytes
+  // scales: 1024 contiguous bytes per 128-row block per step (two 128x4 tiles) = one load instruction of one wave
   constexpr int kARb = (BM + 127) / 128, kBRb = (BN + 127) / 128;
-  // Waves beyond the number of runs repeat run 0 (same bytes to the same place), which keeps the
-  // copy free of branches.
-  const int sgrp = (tid >> 6) < kARb + kBRb ? (tid >> 6) : 0;
-  const bool s_is_a = sgrp < kARb;
+  const bool s_wave = wave < kARb + kBRb;
+  const bool s_is_a = wave < kARb;
   const uint8_t* s_src;
-  int s_dst;
+  int s_dst;  // wave-uniform
   {
-    const int rbi = s_is_a ? sgrp : sgrp - kARb;
+    const int rbi = s_is_a ? wave : wave - kARb;
     const int rb = s_is_a ? min(row0 / 128 + rbi, Mp / 128 - 1) : min(col0 / 128 + rbi, Np / 128 - 1);
-    s_src = (s_is_a ? As : Bs) + (int64_t)rb * (Kp >> 6) * 512 + (tid & 63) * 16;
-    s_dst = S::kAVals + S::kBVals + (s_is_a ? 0 : S::kAScales) + rbi * 1024 + (tid & 63) * 16;
+    s_src = (s_is_a ? As : Bs) + (int64_t)rb * (Kp >> 6) * 512 + lane * 16;
+    s_dst = S::kAVals + S::kBVals + (s_is_a ? 0 : S::kAScales) + rbi * 1024;
   }
+  static_assert(kARb + kBRb <= 4, "one wave per 128-row block of scales");
 
-  uint4 a_reg[kAChunks], b_reg[kBChunks], s_reg;
   const int nk = (Kp + kBK - 1) / kBK;
-  // Kp is a multiple of 64 but maybe not of 128: in the last step the second 64 elements may not
-  // exist.  Those lanes re-read the first half (in bounds) and are masked to zero, so the loads stay
-  // unconditional.
-  auto load_step = [&](int t) {
+  const uint8_t* zero16 = reinterpret_cast<const uint8_t*>(&g_gemm_zero16);
+  // Kp is a multiple of 64 but maybe not of 128: in the last step the second 64 elements may not exist; the
+  // lanes that would fetch them fetch zeros instead.
+  auto load_step = [&](int t, int stage) {
+    const uint32_t base = lds_address(smem + stage * S::kStage + wave * 1024);
+    const uint32_t sbase = lds_address(smem + stage * S::kStage + s_dst);
     const bool second_half_valid = (t * kBK + 64) < Kp;
+    if (second_half_valid) {
 #pragma unroll
-    for (int i = 0; i < kAChunks; ++i) {
-      const bool bad = ((tid + i * kGemmThreads) & 2) && !second_half_valid;
-      const uint32_t keep = bad ? 0u : 0xFFFFFFFFu;
-      uint4 v = *reinterpret_cast<const uint4*>(a_src[i] + (int64_t)t * kRowBytes - (bad ? 32 : 0));
-      a_reg[i] = make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
+      for (int i = 0; i < kAChunks; ++i) load_to_lds_b128(a_src[i] + (int64_t)t * kRowBytes, base + i * 4096);
+#pragma unroll
+      for (int i = 0; i < kBChunks; ++i) load_to_lds_b128(b_src[i] + (int64_t)t * kRowBytes, base + S::kAVals + i * 4096);
+      if (s_wave) load_to_lds_b128(s_src + (int64_t)t * 1024, sbase);
+    } else {
+#pragma unroll
+      for (int i = 0; i < kAChunks; ++i)
+        load_to_lds_b128(tail_piece ? zero16 : a_src[i] + (int64_t)t * kRowBytes, base + i * 4096);
+#pragma unroll
+      for (int i = 0; i < kBChunks; ++i)
+        load_to_lds_b128(tail_piece ? zero16 : b_src[i] + (int64_t)t * kRowBytes, base + S::kAVals + i * 4096);
+      if (s_wave) load_to_lds_b128(lane >= 32 ? zero16 : s_src + (int64_t)t * 1024, sbase);
     }
-#pragma unroll
-    for (int i = 0; i < kBChunks; ++i) {
-      const bool bad = ((tid + i * kGemmThreads) & 2) && !second_half_valid;
-      const uint32_t keep = bad ? 0u : 0xFFFFFFFFu;
-      uint4 v = *reinterpret_cast<const uint4*>(b_src[i] + (int64_t)t * kRowBytes - (bad ? 32 : 0));
-      b_reg[i] = make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
-    }
-    {
-      const bool bad = ((tid & 63) >= 32) && !second_half_valid;
-      const uint32_t keep = bad ? 0u : 0xFFFFFFFFu;
-      uint4 v = *reinterpret_cast<const uint4*>(s_src + (int64_t)t * 1024 - (bad ? 512 : 0));
-      s_reg = make_uint4(v.x & keep, v.y & keep, v.z & keep, v.w & keep);
-    }
-  };
-  auto store_step = [&](int stage) {
-    uint8_t* base = smem + stage * S::kStage;
-#pragma unroll
-    for (int i = 0; i < kAChunks; ++i) *reinterpret_cast<uint4*>(base + a_dst[i]) = a_reg[i];
-#pragma unroll
-    for (int i = 0; i < kBChunks; ++i) *reinterpret_cast<uint4*>(base + b_dst[i]) = b_reg[i];
-    *reinterpret_cast<uint4*>(base + s_dst) = s_reg;
   };
 
   // ---- per-lane LDS read offsets
-  // fragment f of A: rows wm*32*FA + 32 f + l32 ; chunk (cc, lh) = bytes [32 cc + 16 lh, +16)
+  // fragment f of A: rows wm*32*FA + 32 f + l32 ; piece 2 cc + lh of the row, stored at position piece ^ (row / 4 % 4):
+  // the offsets below are those of cc = 0, cc = 1 flips the 32-byte bit
   int a_voff[FA], a_soff[FA], b_voff[FB], b_soff[FB];
 #pragma unroll
   for (int f = 0; f < FA; ++f) {
     const int r = wm * 32 * FA + 32 * f + l32;
     const int rs = r + (row0 & 127);  // row inside the staged 128-row scale blocks (64-row tiles start mid-block)
-    a_voff[f] = r * kLdsRow + 16 * lh;
+    a_voff[f] = r * kLdsRow + 16 * (lh ^ ((r >> 2) & 3));
     a_soff[f] = S::kAVals + S::kBVals + (rs >> 7) * 1024 + (rs & 31) * 16 + ((rs & 127) >> 5) * 4 + 2 * lh;
   }
 #pragma unroll
   for (int f = 0; f < FB; ++f) {
     const int r = wn * 32 * FB + 32 * f + l32;
     const int rs = r + (col0 & 127);
-    b_voff[f] = S::kAVals + r * kLdsRow + 16 * lh;
+    b_voff[f] = S::kAVals + r * kLdsRow + 16 * (lh ^ ((r >> 2) & 3));
     b_soff[f] = S::kAVals + S::kBVals + S::kAScales + (rs >> 7) * 1024 + (rs & 31) * 16 + ((rs & 127) >> 5) * 4 + 2 * lh;
   }
 
@@ -212,7 +222,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
     const uint8_t* base = smem + stage * S::kStage;
 #pragma unroll
     for (int f = 0; f < FA; ++f) {
-      h.a[f] = *reinterpret_cast<const uint4*>(base + a_voff[f] + 32 * cc);
+      h.a[f] = *reinterpret_cast<const uint4*>(base + (a_voff[f] ^ (32 * cc)));
       const uint32_t sb = *reinterpret_cast<const uint16_t*>(base + a_soff[f] + 512 * cc);
       const half2v sc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(sb, 1.0f, false);
       h.as[f][0] = half2v{sc[0], sc[0]};
@@ -220,7 +230,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
     }
 #pragma unroll
     for (int g = 0; g < FB; ++g) {
-      h.b[g] = *reinterpret_cast<const uint4*>(base + b_voff[g] + 32 * cc);
+      h.b[g] = *reinterpret_cast<const uint4*>(base + (b_voff[g] ^ (32 * cc)));
       const uint32_t sb = *reinterpret_cast<const uint16_t*>(base + b_soff[g] + 512 * cc);
       const half2v sc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(sb, 1.0f, false);
       h.bs[g][0] = half2v{sc[0], sc[0]};
@@ -248,19 +258,18 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
 #pragma unroll
       for (int f = 0; f < FA; ++f) acc[g][f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(o.b[g], o.a[f], acc[g][f], 0, 0, 0);
   };
-  // ---- main loop: two LDS stages, global loads for step t+1 in flight while step t is computed.
-  // No software pipelining inside the wave: two workgroups share a CU and the hardware overlaps one
-  // wave's decode (VALU) with another wave's MFMAs.  The last iteration re-loads its own step
-  // (clamped index) so the loop body has no branch.
+  // ---- main loop: two LDS stages, the loads of step t+1 in flight into the other stage while step t is
+  // computed.  No software pipelining inside the wave: two workgroups share a CU and the hardware overlaps one
+  // wave's decode (VALU) with another wave's MFMAs.
   {
-    load_step(0);
-    store_step(0);
+    load_step(0, 0);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces are in LDS
     __syncthreads();
     // A wave whose rows (or columns) all lie beyond M (N) only helps with the staging: in the last row of
     // tiles of M = 2640 with 256-row tiles that is half of the waves.
     const bool wave_has_output = row0 + wm * 32 * FA < M && col0 + wn * 32 * FB < N;
     for (int t = 0; t < nk; ++t) {
-      load_step(min(t + 1, nk - 1));
+      if (t + 1 < nk) load_step(t + 1, (t + 1) & 1);
       if (wave_has_output) {
 #pragma unroll
         for (int cc = 0; cc < 2; ++cc) {
@@ -274,7 +283,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
           }
         }
       }
-      store_step((t + 1) & 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70);
       __syncthreads();
     }
   }
