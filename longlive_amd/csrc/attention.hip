@@ -115,6 +115,17 @@ __device__ __forceinline__ void fetch_row(const uint8_t* values, const uint8_t* 
   f.scales = load_global<uint16_t>(scales + so);
 }
 
+// 4 bytes per lane from global memory straight into LDS at lds_base + 4 * lane (lds_base wave-uniform).  An asm
+// statement on purpose: for the builtin the compiler's wait-count pass, which cannot tell the two LDS stages apart,
+// makes later LDS reads of the *other* stage wait for the load.  The kernel waits for these loads itself
+// (vmcnt(0) ahead of the barrier that hands the stage over).
+__device__ __forceinline__ void load_to_lds_b32(const void* src, uint32_t lds_base) {
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" ::"v"(src), "s"(lds_base) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+  return __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p);
+}
+
 // Decode 32 elements of one key (K or V) to bf16 and store the 64 bytes into the key's LDS row.
 // kind: 0 = fp4 slot data in f (gs = slot amax / (e2m1_max * e4m3_max)), 1 = bf16 row at src, 2 = zeros.
 __device__ __forceinline__ void store_row(const KRaw& f, int kind, float gs, const uint4* src, uint8_t* dst) {
@@ -388,8 +399,6 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
 
   // Plain body: the S phase without interleaved conversion, masking in the last tile, and the successor tile
   // decoded after the MFMAs (or, for the chunk's own bf16 tiles, brought in ahead of them).
-  typedef __attribute__((address_space(1))) const void* gptr_t;
-  typedef __attribute__((address_space(3))) void* lptr_t;
   for (; it < n_iter; ++it) {
     const uint8_t* cur = smem + (it & 1) * kStageBytes;
     const uint8_t* vt_base = cur + 2 * kKTileBytes + kp * kVTileBytes;
@@ -404,10 +413,11 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       const int64_t src_step = (int64_t)p.H * kHeadDim;
       uint8_t* kdst = nxt + (wave >> 2) * kKTileBytes + ((wave & 3) * 16) * kKPitch;
       uint8_t* vdst = nxt + 2 * kKTileBytes + (wave >> 2) * kVTileBytes + ((wave & 3) * 16) * kVPitch;
+      const uint32_t kdst_lds = lds_address(kdst), vdst_lds = lds_address(vdst);
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
-        __builtin_amdgcn_global_load_lds((gptr_t)(p.k_new + src_off + r * src_step), (lptr_t)(kdst + r * kKPitch), 4, 0, 0);
-        __builtin_amdgcn_global_load_lds((gptr_t)(p.v_new + src_off + r * src_step), (lptr_t)(vdst + r * kVPitch), 4, 0, 0);
+        load_to_lds_b32(p.k_new + src_off + r * src_step, kdst_lds + r * kKPitch);
+        load_to_lds_b32(p.v_new + src_off + r * src_step, vdst_lds + r * kVPitch);
       }
     }
     if (tile_base < Lk_i) {
