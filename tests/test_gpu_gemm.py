@@ -55,7 +55,7 @@ def test_golden_matmul(golden, gpu):
 
 
 @pytest.mark.parametrize("M,N,K,seed", [(128, 128, 64, 0), (200, 192, 256, 1), (130, 70, 200, 2), (1, 3072, 128, 3),
-                                        (640, 384, 1152, 4), (300, 1000, 3072, 5)])
+                                        (640, 384, 1152, 4), (300, 1000, 3072, 5), (96, 160, 320, 6), (257, 129, 192, 7)])
 def test_against_oracle(gpu, M, N, K, seed):
     x, w = activations((M, K), seed), weights((N, K), seed + 100)
     xq, wq = quantize_to_fp4(x.to(gpu)), quantize_to_fp4(w.to(gpu))
