@@ -259,8 +259,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
       for (int f = 0; f < FA; ++f) acc[g][f] = __builtin_amdgcn_mfma_f32_32x32x16_f16(o.b[g], o.a[f], acc[g][f], 0, 0, 0);
   };
   // ---- main loop: two LDS stages, the loads of step t+1 in flight into the other stage while step t is
-  // computed.  No software pipelining inside the wave: two workgroups share a CU and the hardware overlaps one
-  // wave's decode (VALU) with another wave's MFMAs.
+  // computed.
   {
     load_step(0, 0);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this wave's pieces are in LDS
@@ -268,23 +267,57 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
     // A wave whose rows (or columns) all lie beyond M (N) only helps with the staging: in the last row of
     // tiles of M = 2640 with 256-row tiles that is half of the waves.
     const bool wave_has_output = row0 + wm * 32 * FA < M && col0 + wn * 32 * FB < N;
-    for (int t = 0; t < nk; ++t) {
-      if (t + 1 < nk) load_step(t + 1, (t + 1) & 1);
-      if (wave_has_output) {
+    if constexpr (FA * FB <= 4) {
+      // Software pipeline inside the wave (the tiles with up to 2x2 fragments have the registers for it): the
+      // operands of sub-step j + 1 are decoded between the MFMAs of sub-step j, one MFMA per group of VALU
+      // instructions, so that the wave never issues MFMAs back to back (the second one would block the wave's
+      // issue until the matrix pipe is free again).  The MFMAs of the last sub-step of a K step are issued after
+      // the barrier, behind the LDS reads of the next step, whose latency they cover.
+      Operands o[2];
+      for (int t = 0; t < nk; ++t) {
+        if (t + 1 < nk) load_step(t + 1, (t + 1) & 1);
+        if (wave_has_output) {
+          Half h[2];
+          read_half(h[0], t & 1, 0);
+          read_half(h[1], t & 1, 1);
+          if (t > 0) mma(o[1]);
+          decode(o[0], h[0], 0);
 #pragma unroll
-        for (int cc = 0; cc < 2; ++cc) {
-          Half h;
-          read_half(h, t & 1, cc);
+          for (int j = 0; j < 7; ++j) {
+            decode(o[(j + 1) & 1], h[(j + 1) >> 2], (j + 1) & 3);
+            mma(o[j & 1]);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            Operands o;
-            decode(o, h, j);
-            mma(o);
+            for (int g = 0; g < FA * FB; ++g) {
+              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);                                          // one MFMA
+              __builtin_amdgcn_sched_group_barrier(0x002, (9 * (FA + FB) + FA * FB - 1) / (FA * FB), 0);  // its share of the decode
+            }
           }
         }
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
       }
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-      __syncthreads();
+      if (wave_has_output) mma(o[1]);
+    } else {
+      // The large tiles need all registers for accumulators and fragments; there two workgroups share a CU and
+      // the hardware overlaps one wave's decode (VALU) with another wave's MFMAs.
+      for (int t = 0; t < nk; ++t) {
+        if (t + 1 < nk) load_step(t + 1, (t + 1) & 1);
+        if (wave_has_output) {
+#pragma unroll
+          for (int cc = 0; cc < 2; ++cc) {
+            Half h;
+            read_half(h, t & 1, cc);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              Operands o;
+              decode(o, h, j);
+              mma(o);
+            }
+          }
+        }
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+      }
     }
   }
 
