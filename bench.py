@@ -1,7 +1,7 @@
 #!/usr/bin/env python
 """Benchmark of the NVFP4 W4A4 hot path on one MI355X.
 
-Workload (BASELINE.json configs[1]): the Wan2.2-TI2V-5B transformer-block linear set in NVFP4 W4A4 for
+Workload (benchmark configuration 2, `configs[1]`): the Wan2.2-TI2V-5B transformer-block linear set in NVFP4 W4A4 for
 one 3-latent-frame chunk (M = 2640 tokens): q/k/v/o and cross q/o (6x K=N=3072), cross k/v on the 512
 text tokens (2x), FFN up (N=14336) and FFN down (K=14336).  One step = quantize each activation to
 NVFP4 (four-over-six, mse) and run its W4A4 GEMM against the pre-quantized weight: 783.4 GFLOP.
@@ -9,7 +9,7 @@ Inputs are synthetic (seed 1) and resident in HBM before the timed region.
 
 Prints one JSON line: whole-step TFLOP/s, plus `roofline` for the dominant kernel (the FFN-up W4A4
 GEMM, timed with HIP events on the launch stream) and `cpu_baseline` (the numpy oracle of the same
-step timed once on the host cores).  `--workload attention|block|e2e` run BASELINE.json configs[2..4]
+step timed once on the host cores).  `--workload attention|block|e2e` run benchmark configurations 3 to 5 (`configs[2..4]`)
 alone (one kernel or model under a profiler); the default run reports them under `extras`.
 """
 from __future__ import annotations
@@ -92,7 +92,7 @@ def _time_events(torch, fn, n, warm=10, repeats=3):
 
 
 def _filled_cache(torch, dev, g):
-    """BASELINE.json configs[2]: a 5-slot FP4 cache of 2640-token blocks with slots 0..3 written
+    """Benchmark configuration 3 (`configs[2]`): a 5-slot FP4 cache of 2640-token blocks with slots 0..3 written
     (sink + three window blocks) by four streaming steps, so the next chunk attends 13200 keys."""
     from longlive_amd.fouroversix import QuantizationConfig
     from longlive_amd.utils import kv_cache as kvc

@@ -159,7 +159,7 @@ def test_block_stage_by_stage_against_oracle(gpu):
 
 
 def test_config4_full_size_block_runs_and_matches_a_dequantized_torch_graph(gpu):
-    """BASELINE config 4 shape: dim 3072, 24 heads, FFN 14336, 2640 tokens, 512 text tokens, KV cache of
+    """Benchmark configuration 4 shape: dim 3072, 24 heads, FFN 14336, 2640 tokens, 512 text tokens, KV cache of
     4 full slots.  The CPU oracle is too slow at this size, so the check is against the same graph
     evaluated with torch on the GPU from the dequantized NVFP4 weights and fake-quantized activations
     (each of those conversions is verified bit-exactly elsewhere); tolerance 6e-2 relative Frobenius (see the first test)."""

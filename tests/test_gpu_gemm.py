@@ -84,7 +84,7 @@ def test_high_precision_operands_are_quantized_on_the_fly(gpu):
 
 
 def test_config1_single_linear_full_size(gpu):
-    """BASELINE config 1: X [2640, 3072] seed 0 with outliers, W [3072, 3072] ~ N(0, 0.02), rule mse."""
+    """Benchmark configuration 1: X [2640, 3072] seed 0 with outliers, W [3072, 3072] ~ N(0, 0.02), rule mse."""
     x, w = activations((2640, 3072), 0), weights((3072, 3072), 0)
     xq, wq = quantize_to_fp4(x.to(gpu)), quantize_to_fp4(w.to(gpu))
     y = fp4_matmul(xq, wq)
@@ -94,7 +94,7 @@ def test_config1_single_linear_full_size(gpu):
 
 
 def test_ffn_shapes_linearity_property(gpu):
-    """BASELINE config 2 FFN shapes (too large for a CPU matmul in a unit test): the GEMM is linear in
+    """Benchmark configuration 2, FFN shapes (too large for a CPU matmul in a unit test): the GEMM is linear in
     the tensor scale of A, so doubling amax_a doubles every output exactly (power of two), and rows of
     A that are zero give zero rows."""
     for M, N, K in ((2640, 14336, 3072), (2640, 3072, 14336)):
