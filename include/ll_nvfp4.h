@@ -213,6 +213,13 @@ int ll_adaln_modulate_amax(const void* x, int64_t B, int64_t L, int C, const voi
 int ll_gate_residual(const void* x, const void* y, int64_t B, int64_t L, int C, const void* gate,
                      int64_t gate_stride_b, int64_t gate_stride_f, int64_t frame_seqlen, void* out, void* stream);
 
+/* WanLayerNorm with elementwise affine (wan_5b/modules/model.py:101-111, used as norm3 ahead of cross-attention,
+ * wan_5b/modules/causal_model.py:892-906): y = bf16(((x - mean) * rsqrt(var + eps)) * w + b) over the last dim C of
+ * x bf16 [rows, C], statistics and affine map in fp32; weight / bias bf16 [C], either may be NULL (1 / 0).
+ * amax_sink (may be NULL) receives the absolute maximum of y, see ll_amax_sink. */
+int ll_layer_norm(const void* x, int64_t rows, int C, const void* weight, const void* bias, float eps, void* out,
+                  const ll_amax_sink* amax_sink, void* stream);
+
 /* WanRMSNorm (wan_5b/modules/model.py:82-98): y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) over the
  * last dim C of x bf16 [rows, C]; w bf16 [C]. */
 int ll_rms_norm(const void* x, int64_t rows, int C, const void* weight, float eps, void* out, void* stream);

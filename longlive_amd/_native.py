@@ -64,6 +64,7 @@ _SIGNATURES = {
     "ll_gate_residual": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_int64, c_int64,
                                  c_void_p, c_void_p]),
     "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
+    "ll_layer_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p]),
     "ll_debug_convert": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
 }
 
@@ -448,6 +449,27 @@ def rms_norm(x, weight, eps=1e-6):
         code = load().ll_rms_norm(x2.data_ptr(), x2.shape[0], C, weight.contiguous().data_ptr(), float(eps),
                                   out.data_ptr(), _stream())
     _check(code, "ll_rms_norm")
+    return out.view(x.shape)
+
+
+def layer_norm(x, weight, bias, eps=1e-6, amax_out=None):
+    """LayerNorm over the last dimension with optional bf16 weight / bias (fp32 statistics, one rounding);
+    ``amax_out`` (an :class:`AmaxTicket`) receives the absolute maximum of the result."""
+    _require_cuda(x, weight, bias)
+    if x.dtype != torch.bfloat16 or any(t is not None and t.dtype != torch.bfloat16 for t in (weight, bias)):
+        raise ValueError("layer_norm takes bfloat16 input, weight and bias")
+    C = x.shape[-1]
+    x2 = x.reshape(-1, C)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    out = torch.empty_like(x2)
+    sink = _sink_struct(amax_out)
+    w = None if weight is None else weight.contiguous()
+    b = None if bias is None else bias.contiguous()
+    with torch.cuda.device(x.device):
+        code = load().ll_layer_norm(x2.data_ptr(), x2.shape[0], C, _ptr(w), _ptr(b), float(eps), out.data_ptr(),
+                                    ctypes.byref(sink), _stream())
+    _check(code, "ll_layer_norm")
     return out.view(x.shape)
 
 

@@ -134,6 +134,71 @@ __global__ __launch_bounds__(kRowThreads) void adaln_kernel(const uint16_t* __re
   }
 }
 
+// ----------------------------------------------------------------------------- LayerNorm with weight and bias
+// wan_5b/modules/model.py:101-111 (nn.LayerNorm on bf16 tensors: statistics and the affine map in fp32, one
+// rounding to bf16 at the end).  One wave = one row.
+template <int NCH>
+__global__ __launch_bounds__(kRowThreads) void layernorm_kernel(const uint16_t* __restrict__ x, int64_t rows, int C,
+                                                                const uint16_t* __restrict__ w,
+                                                                const uint16_t* __restrict__ b, float eps,
+                                                                uint16_t* __restrict__ out, AmaxSink sink) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const uint16_t* xr = x + row * (int64_t)C;
+  const int nchunks = C >> 3;
+  float v[NCH][8];
+  uint4 wraw[NCH], braw[NCH];  // requested up front: their latency runs under the two reductions
+  float sum = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunks) {
+      unpack8(*reinterpret_cast<const uint4*>(xr + c * 8), v[i]);
+      wraw[i] = w ? *reinterpret_cast<const uint4*>(w + c * 8) : make_uint4(0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u);
+      braw[i] = b ? *reinterpret_cast<const uint4*>(b + c * 8) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sum += v[i][j];
+    }
+  }
+  const float inv_c = 1.0f / (float)C;
+  const float mean = wave_sum_dpp(sum) * inv_c;
+  float sq = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunks) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[i][j] -= mean;
+        sq += v[i][j] * v[i][j];
+      }
+    }
+  }
+  const float var = wave_sum_dpp(sq) * inv_c;
+  const float rstd = 1.0f / sqrtf(var + eps);
+  uint16_t* orow = out + row * (int64_t)C;
+  float out_max = 0.0f;
+#pragma unroll
+  for (int i = 0; i < NCH; ++i) {
+    const int c = lane + i * 64;
+    if (c < nchunks) {
+      float w8[8], b8[8], y[8];
+      unpack8(wraw[i], w8);
+      unpack8(braw[i], b8);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = (v[i][j] * rstd) * w8[j] + b8[j];
+      const uint4 packed = pack8(y);
+      *reinterpret_cast<uint4*>(orow + c * 8) = packed;
+      out_max = abs_max_bf16x8(packed, out_max);
+    }
+  }
+  if (sink.parts) {
+    out_max = wave_max(out_max);
+    if (lane == 0) amax_sink_update(sink, (uint32_t)row, out_max);
+  }
+}
+
 // ----------------------------------------------------------------------------- RMSNorm
 // wan_5b/modules/model.py:82-98.
 template <int NCH>
@@ -346,6 +411,37 @@ extern "C" int ll_adaln_modulate_amax(const void* x, int64_t B, int64_t L, int C
   }
 #undef LL_LAUNCH_ADALN
   LL_CHECK_LAUNCH("adaln_kernel");
+  return LL_OK;
+}
+
+extern "C" int ll_layer_norm(const void* x, int64_t rows, int C, const void* weight, const void* bias, float eps,
+                             void* out, const ll_amax_sink* amax_sink, void* stream) {
+  using namespace ll;
+  LL_REQUIRE(x && out, "ll_layer_norm: null pointer");
+  LL_REQUIRE(rows > 0 && rows <= 0x7FFFFFFF && C > 0 && C % 8 == 0 && C <= kMaxRowLength,
+             "ll_layer_norm: bad shape rows=%lld C=%d", (long long)rows, C);
+  LL_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(bias) |
+               reinterpret_cast<uintptr_t>(out)) & 15) == 0,
+             "ll_layer_norm: pointers must be 16-byte aligned");
+  AmaxSink sink{};
+  if (amax_sink && amax_sink->parts) {
+    LL_REQUIRE((reinterpret_cast<uintptr_t>(amax_sink->parts) & 7) == 0 && amax_sink->epoch != 0,
+               "ll_layer_norm: amax sink needs 8-byte alignment and a non-zero epoch");
+    sink.parts = reinterpret_cast<unsigned long long*>(amax_sink->parts);
+    sink.epoch = amax_sink->epoch;
+  }
+  const dim3 grid((unsigned)((rows + kRowsPerWg - 1) / kRowsPerWg));
+#define LL_LAUNCH_LN(NCH)                                                                                        \
+  hipLaunchKernelGGL(layernorm_kernel<NCH>, grid, dim3(kRowThreads), 0, static_cast<hipStream_t>(stream),        \
+                     static_cast<const uint16_t*>(x), rows, C, static_cast<const uint16_t*>(weight),             \
+                     static_cast<const uint16_t*>(bias), eps, static_cast<uint16_t*>(out), sink)
+  if (C <= 64 * 6 * 8) {
+    LL_LAUNCH_LN(6);
+  } else {
+    LL_LAUNCH_LN(kMaxChunks);
+  }
+#undef LL_LAUNCH_LN
+  LL_CHECK_LAUNCH("layernorm_kernel");
   return LL_OK;
 }
 

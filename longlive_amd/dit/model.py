@@ -60,7 +60,13 @@ class WanLayerNorm(nn.LayerNorm):
     def __init__(self, dim: int, eps: float = 1e-6, elementwise_affine: bool = False) -> None:
         super().__init__(dim, elementwise_affine=elementwise_affine, eps=eps)
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, amax_out=None) -> torch.Tensor:
+        """``amax_out``: an amax ticket that receives the absolute maximum of the result (device kernel only)."""
+        if x.is_cuda and x.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0 and \
+                (self.weight is None or self.weight.dtype == torch.bfloat16):
+            return _native.layer_norm(x, self.weight, self.bias, self.eps, amax_out=amax_out)
+        if amax_out is not None:
+            raise ValueError("amax_out needs the device kernel (bfloat16 CUDA input)")
         return super().forward(x).type_as(x)
 
 
@@ -172,14 +178,15 @@ class CrossAttention(nn.Module):
         self.q, self.k, self.v, self.o = (nn.Linear(dim, dim) for _ in range(4))
         self.norm_q, self.norm_k = WanRMSNorm(dim, eps), WanRMSNorm(dim, eps)
 
-    def forward(self, x, context, crossattn_cache: dict | None = None, *, residual=None):
+    def forward(self, x, context, crossattn_cache: dict | None = None, *, residual=None, input_amax=None):
         """``residual`` [B, L, C] turns the result into ``residual + out`` (folded into the output projection).
+        ``input_amax``: the amax ticket the producer of ``x`` was given, if any.
         ``crossattn_cache`` ({"is_init": bool, "k": ..., "v": ...}, the reference's interface,
         wan_5b/modules/causal_model.py:199-206) keeps the projected K / V of a prompt's text context between
         calls; the reference has the argument but recomputes on every call (:229-235), which gives the same
         tensors.  Without a cache K / V are recomputed here too."""
         b, n, d = x.shape[0], self.num_heads, self.head_dim
-        q = self.norm_q(self.q(x)).view(b, -1, n, d)
+        q = self.norm_q(_project_shared(x, [self.q], amax=input_amax)[0]).view(b, -1, n, d)
         if crossattn_cache is not None and crossattn_cache.get("is_init"):
             k, v = crossattn_cache["k"], crossattn_cache["v"]
         else:
@@ -232,7 +239,8 @@ class DiTBlock(nn.Module):
         x, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size,
                                    input_amax=y_amax, residual=x, gate=gates[0], gate_rows=frame_seqlen,
                                    global_sink_tokens=global_sink_tokens, rope_fn=rope_fn)
-        x = self.cross_attn(self.norm3(x), context, crossattn_cache, residual=x)
+        y_amax = _native.amax_ticket(x.device) if isinstance(self.cross_attn.q, FourOverSixLinear) else None
+        x = self.cross_attn(self.norm3(x, amax_out=y_amax), context, crossattn_cache, residual=x, input_amax=y_amax)
         y_amax = _native.amax_ticket(x.device) if isinstance(self.ffn[0], FourOverSixLinear) else None
         y = adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps, amax_out=y_amax)
         x = self._feed_forward(y, y_amax, x, gates[1], frame_seqlen)

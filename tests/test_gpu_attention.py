@@ -271,6 +271,36 @@ def test_rms_norm_against_oracle(gpu):
     assert diff.max() <= 2 ** -5 and (diff != 0).mean() < 5e-3
 
 
+@pytest.mark.parametrize("L,C,affine", [(37, 256, True), (2640, 3072, True), (10, 4096, False), (5, 1000, True)])
+def test_layer_norm_against_oracle_and_torch(gpu, L, C, affine):
+    """LayerNorm with weight and bias (the norm ahead of cross-attention): fp32 statistics, one rounding.  Against
+    the float64 oracle and against torch's own bf16 layer_norm, each within one bf16 step; the amax it leaves in
+    the sink is the maximum of what it wrote."""
+    import dit_oracle
+
+    x = _randn((1, L, C), 41, 3.0) + 0.5
+    w = (_randn((C,), 42, 0.2) + 1.0) if affine else None
+    b = _randn((C,), 43, 0.3) if affine else None
+    ticket = _native.amax_ticket(gpu)
+    y = _native.layer_norm(x.to(gpu), None if w is None else w.to(gpu), None if b is None else b.to(gpu), 1e-6,
+                           amax_out=ticket)
+    got = y[0].float().cpu().numpy()
+    wn = np.ones(C, np.float32) if w is None else w.float().numpy()
+    bn = np.zeros(C, np.float32) if b is None else b.float().numpy()
+    ref = dit_oracle.layer_norm_affine(x[0].float().numpy(), wn, bn, 1e-6)
+    # one bf16 step at the magnitude of the value, plus the fp32 error of the two terms where they cancel
+    step = np.abs(ref) * 2.0 ** -7 + 4e-6 * (np.abs(bn) + 6.0 * np.abs(wn))[None, :]
+    assert (np.abs(got - ref) <= step).all()
+    assert (got == ref).mean() > 0.98
+    t = torch.nn.functional.layer_norm(x.to(gpu), (C,), None if w is None else w.to(gpu), None if b is None else b.to(gpu),
+                                       1e-6)[0].float().cpu().numpy()
+    assert (np.abs(got - t) <= step).all()
+    xq_sink = quantize_to_fp4(y[0], CFG, amax=ticket)
+    xq_pass = quantize_to_fp4(y[0], CFG)
+    assert float(xq_sink.amax) == float(xq_pass.amax) == np.abs(got).max()
+    assert torch.equal(xq_sink.values, xq_pass.values)
+
+
 def test_config3_full_size_fused_decode_equals_attention_over_the_dequantized_cache(gpu):
     """Benchmark shape (24 heads, 2640 queries, 4 FP4 slots of 2640 tokens + the bf16 chunk = 13200 keys):
     the kernel that decodes FP4 on load must agree with plain bf16 attention over the cache dequantized by
