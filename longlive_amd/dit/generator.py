@@ -12,6 +12,8 @@ the stream become a global sink that is never evicted, and the first chunk of ev
 is pinned after its clean-context pass, so that the new scene attends its own opening frames instead of the
 previous scene's; ``shot_clean_recache`` additionally forgets everything but the global sink before that pass.
 ``use_relative_rope`` (:149, 316) caches K without RoPE and rotates the attended window by its own frame positions.
+``multi_shot_rope_offset`` (:108-112, 439-442, 545-549) shifts the temporal RoPE positions of every scene by
+``scene index * offset`` frames, which moves scenes apart in position space.
 
 Two samplers: ``"euler"`` steps the flow prediction over the given timesteps (the fixed 1000/750/500/250
 schedule of the benchmark configuration); ``"unipc"`` is the reference pipeline's own choice (:566-612,
@@ -33,7 +35,7 @@ class StreamingGenerator:
                  model_quant: dict | None = None, kv_scale_rule: str = "mse", cache_text_kv: bool = True,
                  skip_dead_cache_writes: bool = True, sampler: str = "euler", sample_shift: float = 5.0,
                  multi_shot_sink: bool = False, shot_clean_recache: bool = False,
-                 use_relative_rope: bool = False) -> None:
+                 use_relative_rope: bool = False, multi_shot_rope_offset: float = 0.0) -> None:
         if sampler not in ("euler", "unipc"):
             raise ValueError(f"unknown sampler {sampler!r}")
         self.cfg, self.device = cfg, torch.device(device)
@@ -53,6 +55,7 @@ class StreamingGenerator:
         self.model.kv_quant_config = self.kv_quant_config
         self.kv_cache = None
         self.multi_shot_sink, self.shot_clean_recache = multi_shot_sink, shot_clean_recache
+        self.multi_shot_rope_offset = float(multi_shot_rope_offset)
         self.global_sink_size = cfg.sink_size if multi_shot_sink else 0   # :107
         self.model.global_sink_size = self.global_sink_size
         for block in self.model.blocks:                                   # :316
@@ -84,6 +87,8 @@ class StreamingGenerator:
         xcache = [{"is_init": False} for _ in range(cfg.num_layers)] if self.cache_text_kv else None
         contexts = list(context) if isinstance(context, (list, tuple)) else None
         scene_cuts = {int(c) for c in scene_cuts}
+        shot_index = 0
+        self.model.rope_temporal_offset = 0.0
         sigmas = [t / 1000.0 for t in self.timesteps] + [0.0]
         for ci, start in enumerate(range(0, F, nb)):
             x = noise[0, start:start + nb].transpose(0, 1).contiguous()  # [C, f, H, W]
@@ -92,6 +97,9 @@ class StreamingGenerator:
                 if ci > 0 and contexts[ci] is not contexts[ci - 1] and xcache is not None:
                     xcache = [{"is_init": False} for _ in range(cfg.num_layers)]  # new prompt: re-project its K / V
                 context = contexts[ci]
+            if ci > 0 and ci in scene_cuts and self.multi_shot_rope_offset != 0.0:
+                shot_index += 1
+                self.model.rope_temporal_offset = shot_index * self.multi_shot_rope_offset
             is_scene_cut = self.multi_shot_sink and cfg.sink_size > 0 and ci > 0 and ci in scene_cuts
             if self.sampler == "unipc":
                 scheduler = FlowUniPCMultistepScheduler(num_train_timesteps=1000, shift=1)

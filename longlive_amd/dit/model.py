@@ -280,6 +280,7 @@ class CausalDiT(nn.Module):
         self.head = CausalHead(cfg.dim, cfg.out_dim, cfg.patch_size, cfg.eps)
         self.rope_angles = build_rope_angles(cfg.dim // cfg.num_heads)
         self.global_sink_size = cfg.global_sink_size  # frames; the generator overrides it like the reference pipeline
+        self.rope_temporal_offset = 0.0               # frames added to every temporal position (causal_model.py:1097)
         self.kv_quant_config = None
         self._rope_cache: dict = {}
         self.init_weights()
@@ -300,12 +301,13 @@ class CausalDiT(nn.Module):
                     nn.init.normal_(m.weight, std=0.02)
         nn.init.normal_(self.head.head.weight, std=0.02)
 
-    def _rope(self, f: int, h: int, w: int, start_frame: int, device) -> tuple[torch.Tensor, torch.Tensor]:
-        key = (f, h, w, start_frame, str(device))
+    def _rope(self, f: int, h: int, w: int, start_frame: int, device, temporal_offset: float = 0.0):
+        key = (f, h, w, start_frame, str(device), float(temporal_offset))
         if key not in self._rope_cache:
             if len(self._rope_cache) > 64:
                 self._rope_cache.clear()
-            self._rope_cache[key] = rope_cos_sin(self.rope_angles, f, h, w, start_frame, device)
+            self._rope_cache[key] = rope_cos_sin(self.rope_angles, f, h, w, start_frame, device,
+                                                 temporal_offset=float(temporal_offset))
         return self._rope_cache[key]
 
     def unpatchify(self, x: torch.Tensor, grid) -> torch.Tensor:
@@ -333,7 +335,8 @@ class CausalDiT(nn.Module):
         e0 = self.time_projection(e).unflatten(2, (6, cfg.dim))
         ctx = torch.cat([context, context.new_zeros(cfg.text_len - context.size(0), context.size(1))]).unsqueeze(0)
         ctx = self.text_embedding(ctx)
-        cos, sin = self._rope(f, h, w, current_start // frame_seqlen, x.device)
+        # the multi-shot phase offset applies to absolute positions only (causal_model.py:478-486, 1588)
+        cos, sin = self._rope(f, h, w, current_start // frame_seqlen, x.device, self.rope_temporal_offset)
         sink_tokens = cfg.sink_size * frame_seqlen
         max_attn = cfg.local_attn_size * frame_seqlen
         updates = []

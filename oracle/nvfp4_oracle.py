@@ -358,13 +358,18 @@ def rope_table(max_pos: int = 1024, head_dim: int = 128, theta: float = 10000.0)
     return cols  # three arrays [max_pos, 22], [max_pos, 21], [max_pos, 21]
 
 
-def rope_cos_sin(f, h, w, start_frame=0, head_dim=128):
+def rope_cos_sin(f, h, w, start_frame=0, head_dim=128, t_scale=1.0, temporal_offset=0.0):
     """fp32 cos/sin [f*h*w, head_dim/2], token order (f, h, w) row-major
-    (causal_model.py:161-178, utils/rope_triton.py:84-91)."""
+    (causal_model.py:161-178, utils/rope_triton.py:84-91).  Temporal position of frame i:
+    (start_frame + i + temporal_offset) * t_scale (utils/position_embedding_utils.py:55-107; the offset is a
+    number or one value per frame of the chunk)."""
     tf, th, tw = rope_table(head_dim=head_dim)
+    pos = (np.arange(f, dtype=np.float64) + start_frame + np.asarray(temporal_offset, dtype=np.float64)) * t_scale
+    inv = tf[1]                      # angle per unit of position
+    ang_t = pos[:, None] * inv[None, :]
     ang = np.concatenate(
         [
-            np.broadcast_to(tf[start_frame : start_frame + f][:, None, None, :], (f, h, w, tf.shape[1])),
+            np.broadcast_to(ang_t[:, None, None, :], (f, h, w, tf.shape[1])),
             np.broadcast_to(th[:h][None, :, None, :], (f, h, w, th.shape[1])),
             np.broadcast_to(tw[:w][None, None, :, :], (f, h, w, tw.shape[1])),
         ],

@@ -291,6 +291,38 @@ def test_streaming_generator_multi_shot_sink(gpu, clean):
     assert st["pinned_start"] == blk or clean                     # the pinned chunk ends up right behind the sink
 
 
+def test_streaming_generator_multi_shot_rope_offset(gpu):
+    """The temporal RoPE positions of every scene after a cut are shifted by scene index x offset: nothing changes
+    before the first cut, the model's offset ends at (number of cuts) x offset, and a forward of the model with the
+    offset equals a forward at the shifted frame position when the offset is a whole number of frames."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    g = torch.Generator().manual_seed(9)
+    noise = torch.randn(1, 10, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    gen = StreamingGenerator(cfg, gpu, seed=4, multi_shot_rope_offset=8.0)
+    out = gen.generate(noise, ctx, scene_cuts=(2, 4))
+    plain = StreamingGenerator(cfg, gpu, seed=4).generate(noise, ctx)
+    assert torch.isfinite(out.float()).all()
+    assert gen.model.rope_temporal_offset == 16.0
+    assert torch.equal(out[:, :4], plain[:, :4]) and not torch.equal(out[:, 4:], plain[:, 4:])
+    # one forward on an empty cache: offset 8 at frame 0 == no offset at frame 8 (tables agree to float32 rounding)
+    m = gen.model
+    x = noise[0, :2].transpose(0, 1).contiguous()
+    t = torch.full((1, 2), 500.0, device=gpu)
+    fs = 64
+    def fresh():
+        return kvc.initialize_kv_cache(cfg.num_layers, 2 * fs, 3, cfg.num_heads, 128, gen.kv_quant_config, gpu)
+    m.rope_temporal_offset = 8.0
+    a = m(x, t, ctx, fresh(), 0)
+    m.rope_temporal_offset = 0.0
+    cache = fresh()
+    for c in cache:   # an empty cache whose stream position is frame 8
+        c["_global_end"], c["_local_end"] = 8 * fs, 0
+    b = m(x, t, ctx, cache, 8 * fs, apply_cache_updates=False)
+    assert (a.float() - b.float()).abs().max() <= 0.02 * b.float().abs().max()
+
+
 def test_streaming_generator_relative_rope(gpu):
     """While the window still starts at frame 0 of the stream, relative and absolute positions coincide, so the
     two modes may only differ by the bf16 rounding of cached-then-rotated keys."""
