@@ -4,8 +4,10 @@ Mirror of the chunk / denoise loop of the reference pipeline
 (pipeline/causal_diffusion_inference.py:532-705): every chunk of ``num_frame_per_block`` latent
 frames is denoised with a few flow-matching steps against the cached context and is then run once
 more at timestep 0 so that the cache holds the clean chunk's K / V (:639-647).  The cache keeps
-``sink_size`` frames plus a sliding window, ``local_attn_size`` frames in total (:775-783).  VAE,
-text encoder and classifier-free guidance are outside this path.
+``sink_size`` frames plus a sliding window, ``local_attn_size`` frames in total (:775-783).  VAE and
+text encoder are outside this path.  Classifier-free guidance (:215, 579-602, 648-657) runs every forward a
+second time on the negative prompt against a KV cache of its own and steps with
+``uncond + guidance_scale * (cond - uncond)``.
 
 Multi-shot generation (:104-107, 630-665, 974-1043): with ``multi_shot_sink`` the first ``sink_size`` frames of
 the stream become a global sink that is never evicted, and the first chunk of every later scene (``scene_cuts``)
@@ -35,7 +37,8 @@ class StreamingGenerator:
                  model_quant: dict | None = None, kv_scale_rule: str = "mse", cache_text_kv: bool = True,
                  skip_dead_cache_writes: bool = True, sampler: str = "euler", sample_shift: float = 5.0,
                  multi_shot_sink: bool = False, shot_clean_recache: bool = False,
-                 use_relative_rope: bool = False, multi_shot_rope_offset: float = 0.0) -> None:
+                 use_relative_rope: bool = False, multi_shot_rope_offset: float = 0.0,
+                 guidance_scale: float = 1.0) -> None:
         if sampler not in ("euler", "unipc"):
             raise ValueError(f"unknown sampler {sampler!r}")
         self.cfg, self.device = cfg, torch.device(device)
@@ -56,6 +59,8 @@ class StreamingGenerator:
         self.kv_cache = None
         self.multi_shot_sink, self.shot_clean_recache = multi_shot_sink, shot_clean_recache
         self.multi_shot_rope_offset = float(multi_shot_rope_offset)
+        self.guidance_scale = float(guidance_scale)
+        self.kv_cache_neg = None
         self.global_sink_size = cfg.sink_size if multi_shot_sink else 0   # :107
         self.model.global_sink_size = self.global_sink_size
         for block in self.model.blocks:                                   # :316
@@ -69,18 +74,29 @@ class StreamingGenerator:
         max_blocks = (cfg.local_attn_size * frame_seq_length) // block_token_size
         self.kv_cache = kvc.initialize_kv_cache(cfg.num_layers, block_token_size, max_blocks, cfg.num_heads,
                                                 cfg.dim // cfg.num_heads, self.kv_quant_config, self.device)
+        self.kv_cache_neg = None
+        if self.guidance_scale != 1.0:
+            self.kv_cache_neg = kvc.initialize_kv_cache(cfg.num_layers, block_token_size, max_blocks, cfg.num_heads,
+                                                        cfg.dim // cfg.num_heads, self.kv_quant_config, self.device)
 
     @torch.no_grad()
-    def generate(self, noise: torch.Tensor, context, on_chunk=None, scene_cuts=()) -> torch.Tensor:
+    def generate(self, noise: torch.Tensor, context, on_chunk=None, scene_cuts=(),
+                 negative_context: torch.Tensor | None = None) -> torch.Tensor:
         """noise [1, F, C, H, W] bf16 latents, context [L, text_dim] bf16 (or one such tensor per chunk) ->
         denoised latents of the same shape.  ``on_chunk(index)`` is called after each chunk (timing hooks).
         ``scene_cuts``: indices of the chunks that open a new scene (the reference recognises them by a prefix
-        of the chunk's prompt, :974-996); they matter in multi-shot mode only."""
+        of the chunk's prompt, :974-996); they matter in multi-shot mode only.  ``negative_context`` [L, text_dim]:
+        the negative prompt, needed when ``guidance_scale`` is not 1."""
         cfg = self.cfg
         _, F, C, H, W = noise.shape
         fs = (H // cfg.patch_size[1]) * (W // cfg.patch_size[2])
-        if self.kv_cache is None:
+        use_cfg = self.guidance_scale != 1.0
+        if use_cfg and negative_context is None:
+            raise ValueError("guidance_scale != 1 needs negative_context")
+        if self.kv_cache is None or (use_cfg and self.kv_cache_neg is None):
             self.reset_cache(fs)
+        caches = [self.kv_cache] + ([self.kv_cache_neg] if use_cfg else [])
+        xcache_neg = [{"is_init": False} for _ in range(cfg.num_layers)] if (use_cfg and self.cache_text_kv) else None
         out = torch.empty_like(noise)
         nb = cfg.num_frame_per_block
         # projected text K / V per layer: one prompt per call, so they are computed by the first forward only
@@ -114,18 +130,22 @@ class StreamingGenerator:
                 # clean-context pass below writes; the cache after the chunk is the same either way.
                 flow = self.model(x, tt, context, self.kv_cache, start * fs, crossattn_cache=xcache,
                                   apply_cache_updates=not self.skip_dead_cache_writes)
+                if use_cfg:
+                    uncond = self.model(x, tt, negative_context, self.kv_cache_neg, start * fs, crossattn_cache=xcache_neg,
+                                        apply_cache_updates=not self.skip_dead_cache_writes)
+                    flow = uncond + self.guidance_scale * (flow - uncond)
                 if scheduler is not None:
                     x = scheduler.step(flow, t, x, return_dict=False)[0]
                 else:
                     x = (x.float() + (sigmas[si + 1] - sigmas[si]) * flow.float()).to(noise.dtype)
             out[0, start:start + f] = x.transpose(0, 1)
             # clean-context pass: rewrites this chunk's K / V in the cache
-            if is_scene_cut and self.shot_clean_recache:
-                kvc.zero_kv_data(self.kv_cache, start * fs, self.global_sink_size * fs)
-            self.model(x, torch.zeros((1, f), device=self.device), context, self.kv_cache, start * fs,
-                       crossattn_cache=xcache)
-            if is_scene_cut:
-                kvc.pin_current_chunk(self.kv_cache, f * fs, cfg.sink_size * fs)
+            for cache, text, xc in zip(caches, (context, negative_context), (xcache, xcache_neg)):
+                if is_scene_cut and self.shot_clean_recache:
+                    kvc.zero_kv_data(cache, start * fs, self.global_sink_size * fs)
+                self.model(x, torch.zeros((1, f), device=self.device), text, cache, start * fs, crossattn_cache=xc)
+                if is_scene_cut:
+                    kvc.pin_current_chunk(cache, f * fs, cfg.sink_size * fs)
             if on_chunk is not None:
                 on_chunk(ci)
         return out

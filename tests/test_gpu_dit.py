@@ -323,6 +323,29 @@ def test_streaming_generator_multi_shot_rope_offset(gpu):
     assert (a.float() - b.float()).abs().max() <= 0.02 * b.float().abs().max()
 
 
+def test_streaming_generator_classifier_free_guidance(gpu):
+    """guidance_scale != 1: every forward runs on the prompt and on the negative prompt with a cache each, the flow
+    is uncond + s (cond - uncond).  With the negative prompt equal to the prompt the two forwards agree, so the
+    result equals the unguided run up to the bf16 rounding of the combination; both caches end in the same state."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    g = torch.Generator().manual_seed(10)
+    noise = torch.randn(1, 8, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx, neg = (torch.randn(10, 64, generator=g).bfloat16().to(gpu) for _ in range(2))
+    plain = StreamingGenerator(cfg, gpu, seed=4).generate(noise, ctx)
+    gen = StreamingGenerator(cfg, gpu, seed=4, guidance_scale=3.0)
+    with pytest.raises(ValueError):
+        gen.generate(noise, ctx)
+    same = gen.generate(noise, ctx, negative_context=ctx)
+    assert (same.float() - plain.float()).abs().max() <= 0.05 * plain.float().abs().max()
+    for a, b in zip(gen.kv_cache, gen.kv_cache_neg):
+        assert a["_local_end"] == b["_local_end"] == 3 * 128 and a["_global_end"] == b["_global_end"] == 8 * 64
+        assert torch.equal(a["k"][1].values, b["k"][1].values)
+    gen.kv_cache = None
+    guided = gen.generate(noise, ctx, negative_context=neg)
+    assert torch.isfinite(guided.float()).all() and not torch.equal(guided, same)
+
+
 def test_streaming_generator_relative_rope(gpu):
     """While the window still starts at frame 0 of the stream, relative and absolute positions coincide, so the
     two modes may only differ by the bf16 rounding of cached-then-rotated keys."""
