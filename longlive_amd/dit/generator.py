@@ -81,12 +81,17 @@ class StreamingGenerator:
 
     @torch.no_grad()
     def generate(self, noise: torch.Tensor, context, on_chunk=None, scene_cuts=(),
-                 negative_context: torch.Tensor | None = None) -> torch.Tensor:
+                 negative_context: torch.Tensor | None = None,
+                 initial_latent: torch.Tensor | None = None) -> torch.Tensor:
         """noise [1, F, C, H, W] bf16 latents, context [L, text_dim] bf16 (or one such tensor per chunk) ->
         denoised latents of the same shape.  ``on_chunk(index)`` is called after each chunk (timing hooks).
         ``scene_cuts``: indices of the chunks that open a new scene (the reference recognises them by a prefix
         of the chunk's prompt, :974-996); they matter in multi-shot mode only.  ``negative_context`` [L, text_dim]:
-        the negative prompt, needed when ``guidance_scale`` is not 1."""
+        the negative prompt, needed when ``guidance_scale`` is not 1.  ``initial_latent`` [1, F0, C, H, W]: clean
+        latents of frames that precede the generated ones (image / video continuation, :375-432): they are run
+        through the model at timestep 0 block by block to fill the cache and are returned in front of the generated
+        frames; F0 must be a whole number of blocks (the reference's single independent first frame is not
+        supported by the block-wise FP4 cache)."""
         cfg = self.cfg
         _, F, C, H, W = noise.shape
         fs = (H // cfg.patch_size[1]) * (W // cfg.patch_size[2])
@@ -97,8 +102,17 @@ class StreamingGenerator:
             self.reset_cache(fs)
         caches = [self.kv_cache] + ([self.kv_cache_neg] if use_cfg else [])
         xcache_neg = [{"is_init": False} for _ in range(cfg.num_layers)] if (use_cfg and self.cache_text_kv) else None
-        out = torch.empty_like(noise)
         nb = cfg.num_frame_per_block
+        f0 = 0 if initial_latent is None else initial_latent.shape[1]
+        if f0 % nb:
+            raise NotImplementedError(f"initial_latent must hold whole blocks of {nb} frames")
+        out = noise.new_empty((1, f0 + F) + tuple(noise.shape[2:]))
+        first_text = context[0] if isinstance(context, (list, tuple)) else context
+        for start in range(0, f0, nb):   # context blocks: clean latents, timestep 0, cache writes only
+            x = initial_latent[0, start:start + nb].transpose(0, 1).contiguous()
+            out[0, start:start + nb] = initial_latent[0, start:start + nb]
+            for cache, text in zip(caches, (first_text, negative_context)):
+                self.model(x, torch.zeros((1, nb), device=self.device), text, cache, start * fs)
         # projected text K / V per layer: one prompt per call, so they are computed by the first forward only
         xcache = [{"is_init": False} for _ in range(cfg.num_layers)] if self.cache_text_kv else None
         contexts = list(context) if isinstance(context, (list, tuple)) else None
@@ -106,8 +120,9 @@ class StreamingGenerator:
         shot_index = 0
         self.model.rope_temporal_offset = 0.0
         sigmas = [t / 1000.0 for t in self.timesteps] + [0.0]
-        for ci, start in enumerate(range(0, F, nb)):
-            x = noise[0, start:start + nb].transpose(0, 1).contiguous()  # [C, f, H, W]
+        for ci, src in enumerate(range(0, F, nb)):
+            start = f0 + src                                              # position of the chunk in the stream
+            x = noise[0, src:src + nb].transpose(0, 1).contiguous()      # [C, f, H, W]
             f = x.shape[1]
             if contexts is not None:
                 if ci > 0 and contexts[ci] is not contexts[ci - 1] and xcache is not None:

@@ -346,6 +346,24 @@ def test_streaming_generator_classifier_free_guidance(gpu):
     assert torch.isfinite(guided.float()).all() and not torch.equal(guided, same)
 
 
+def test_streaming_generator_continues_from_initial_latents(gpu):
+    """Clean context frames fill the cache at timestep 0 exactly like the clean-context pass of a generated chunk,
+    so continuing from the first chunk of a run reproduces the rest of that run bit for bit."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    g = torch.Generator().manual_seed(11)
+    noise = torch.randn(1, 10, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    full = StreamingGenerator(cfg, gpu, seed=4).generate(noise, ctx)
+    gen = StreamingGenerator(cfg, gpu, seed=4)
+    cont = gen.generate(noise[:, 4:], ctx, initial_latent=full[:, :4])
+    assert cont.shape == full.shape and torch.equal(cont[:, :4], full[:, :4])
+    assert torch.equal(cont[:, 4:], full[:, 4:])
+    assert gen.kv_cache[0]["_global_end"] == 10 * 64
+    with pytest.raises(NotImplementedError):
+        gen.generate(noise[:, 4:], ctx, initial_latent=full[:, :3])
+
+
 def test_streaming_generator_relative_rope(gpu):
     """While the window still starts at frame 0 of the stream, relative and absolute positions coincide, so the
     two modes may only differ by the bf16 rounding of cached-then-rotated keys."""
