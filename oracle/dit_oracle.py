@@ -2,8 +2,12 @@
 
 Composition of the functions in ``nvfp4_oracle`` in the order of the reference block forward
 (wan_5b/modules/causal_model.py:862-930, 362-368, 477-487, 557-671, 197-262), with a bf16 rounding
-wherever the eager bf16 graph of the reference rounds.  Parity of the composition is "unpinned" in
-the sense that the reference ships no golden vector for a block; every component is pinned on its own.
+wherever the eager bf16 graph of the reference rounds.  The reference ships no golden vector for a block, so
+the composition is **parity unpinned** against the reference itself; what pins it here is that every component is
+pinned on its own and that structural special cases hold (tests/test_dit_oracle.py: closed gates are the
+identity, each gate opens exactly its own branch, scale / shift slots feed the norm of their own branch and
+frame, cross-attention is added ungated and token by token, cached keys are attended as a set) - the cases a
+dropped term, a swapped modulation slot or a transposed operand would fail.
 """
 from __future__ import annotations
 
