@@ -36,7 +36,7 @@ LINEAR_SET = [
 PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak (the GEMM runs v_mfma_f32_32x32x16_f16)
 # HBM-side bytes of one FFN-up GEMM launch from the rocprofv3 counter runs kept under profiles/:
 # FETCH_SIZE 82078 KiB x 2.0 (the factor a 256 MiB copy calibrates) + WRITE_SIZE 73920 KiB x 1.0
-FFN_UP_TRAFFIC_BYTES = (92575.8 * 2.0 + 73927.3) * 1024  # FETCH_SIZE x 2.00 (copy yardstick) + WRITE_SIZE, KiB per launch
+FFN_UP_TRAFFIC_BYTES = (75334.7 * 2.0 + 73927.3) * 1024  # FETCH_SIZE x 2.00 (copy yardstick) + WRITE_SIZE, KiB per launch
 
 
 def step_flops() -> float:
