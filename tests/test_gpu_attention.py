@@ -333,6 +333,38 @@ def test_config3_full_size_fused_decode_equals_attention_over_the_dequantized_ca
     assert (out_c.float() - 0.75).abs().max().item() <= 2 ** -7
 
 
+def test_release_shape_rolling_window_equals_attention_over_the_dequantized_slots(gpu):
+    """Shapes of the reference's released NVFP4 configuration (configs/nvfp4/inference_nvfp4.yaml:3-7: chunks of 8
+    frames = 7040 tokens, window 32 frames = 4 blocks, sink 8 frames = 1 block), streamed past the point where
+    the window rolls: in chunks 4 and 5 the kernel attends the sink block, the two most recent cached blocks and
+    the chunk itself (28160 keys).  Checked against plain bf16 attention over exactly those slots dequantized by
+    the separate kernel, and against the oracle's fp64 softmax on a sample of queries of three heads."""
+    from longlive_amd.utils.quant import k_smooth
+    H, T, blocks = 24, 7040, 4
+    g = torch.Generator().manual_seed(7)
+    cache = kvc.initialize_kv_cache(1, T, blocks, H, 128, CFG, gpu)[0]
+    for c in range(6):
+        q, k, v = (torch.randn(1, T, H, 128, generator=g).bfloat16().to(gpu) for _ in range(3))
+        slot_ids, _, _ = kvc.plan_cache_step(cache, c * T, T, T, blocks * T)
+        out, (ce, le, info) = kvc.kv_cache_attention(q, k, v, cache, c * T, sink_tokens=T, max_attention_size=blocks * T)
+        if c >= 4:
+            assert info["action"] == "roll_and_insert" and len(slot_ids) == blocks - 1 and slot_ids[0] == 0
+            kd = dequantize_kv_cache(cache["k"], blocks, H, T, torch.bfloat16, gpu)[0].view(blocks, T, H, 128)
+            vd = dequantize_kv_cache(cache["v"], blocks, H, T, torch.bfloat16, gpu)[0].view(blocks, T, H, 128)
+            k_all = torch.cat([kd[i] for i in slot_ids] + [k_smooth(k)[0]]).contiguous()
+            v_all = torch.cat([vd[i] for i in slot_ids] + [v[0]]).contiguous()
+            assert k_all.shape == (blocks * T, H, 128)
+            ref = _native.attention_bf16(q[0].contiguous(), k_all, v_all, 128 ** -0.5)
+            assert (out[0].float() - ref.float()).abs().max().item() <= 4e-3
+            for h in (0, 13, 23):
+                rows = slice(7000, 7016)   # the ragged last query tile (7040 = 55 * 128)
+                want = o.attention(q[0, rows, h:h + 1].float().cpu().numpy(), k_all[:, h:h + 1].float().cpu().numpy(),
+                                   v_all[:, h:h + 1].float().cpu().numpy())
+                assert np.abs(out[0, rows, h:h + 1].float().cpu().numpy() - want).max() <= 2e-2
+            del kd, vd, k_all, v_all, ref
+        kvc.apply_cache_update(cache, ce, le, info, CFG)
+
+
 def test_gate_residual_bit_exact_against_oracle_and_eager(gpu):
     from longlive_amd.utils.adaln import gate_residual
     L, C, fs = 48, 3072, 16

@@ -97,7 +97,18 @@ def test_ffn_shapes_linearity_property(gpu):
     """Benchmark configuration 2, FFN shapes (too large for a CPU matmul in a unit test): the GEMM is linear in
     the tensor scale of A, so doubling amax_a doubles every output exactly (power of two), and rows of
     A that are zero give zero rows."""
-    for M, N, K in ((2640, 14336, 3072), (2640, 3072, 14336)):
+    _ffn_shape_checks(gpu, ((2640, 14336, 3072), (2640, 3072, 14336)))
+
+
+def test_release_chunk_shapes_linearity_property(gpu):
+    """The same checks at the token count of the reference's released configuration (chunks of 8 frames =
+    7040 tokens, configs/nvfp4/inference_nvfp4.yaml:5): 55 row tiles of 128 or 27.5 of 256, so other tile
+    choices and a ragged last row tile."""
+    _ffn_shape_checks(gpu, ((7040, 3072, 3072), (7040, 14336, 3072), (7040, 3072, 14336)))
+
+
+def _ffn_shape_checks(gpu, shapes):
+    for M, N, K in shapes:
         x, w = activations((M, K), 1).to(gpu), weights((N, K), 1).to(gpu)
         x[5] = 0
         xq, wq = quantize_to_fp4(x), quantize_to_fp4(w)
