@@ -508,16 +508,8 @@ static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
   AttnParams p = p_in;
   p.n_qtiles = (int)((p.Lq + kWgQueries - 1) / kWgQueries);
   const size_t smem = 2 * kStageBytes + sizeof(SlotTable);
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&kv_attention_kernel),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) {
-      set_error("ll_kv_attention: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-      return LL_ELAUNCH;
-    }
-    configured = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&kv_attention_kernel), smem, lds_allowed, "ll_kv_attention")) return rc;
   hipLaunchKernelGGL(kv_attention_kernel, dim3((unsigned)(p.H * p.n_qtiles)), dim3(kAttnThreads), smem, stream, p);
   LL_CHECK_LAUNCH("kv_attention_kernel");
   return LL_OK;

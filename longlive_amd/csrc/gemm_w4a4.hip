@@ -437,16 +437,8 @@ int launch_gemm(const uint8_t* Av, const uint8_t* As, const uint8_t* Bv, const u
   using S = GemmSmem<FA, FB>;
   const int tiles_m = (M + S::BM - 1) / S::BM, tiles_n = (N + S::BN - 1) / S::BN;
   const size_t smem = 2 * S::kStage;
-  static bool configured = false;
-  if (!configured) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_w4a4_kernel<FA, FB>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    if (e != hipSuccess) {
-      set_error("ll_nvfp4_gemm_tnt: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-      return LL_ELAUNCH;
-    }
-    configured = true;
-  }
+  static std::atomic<uint64_t> lds_allowed{0};  // one per tile configuration
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_w4a4_kernel<FA, FB>), smem, lds_allowed, "ll_nvfp4_gemm_tnt")) return rc;
   hipLaunchKernelGGL((gemm_w4a4_kernel<FA, FB>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kGemmThreads), smem, stream,
                      Av, As, Bv, Bs, alpha, amax_a, amax_b, 1.0f / denom_a, 1.0f / denom_b, M, N, Mp, Np, Kp,
                      static_cast<uint16_t*>(D), ldd, tiles_m, tiles_n, epi);

@@ -4,6 +4,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <atomic>
+
 #include "../../include/ll_nvfp4.h"
 
 namespace ll {
@@ -29,6 +31,27 @@ void set_error(const char* fmt, ...);
   } while (0)
 
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+// Kernels that need more than 64 KB of dynamic LDS have to be told so with hipFuncSetAttribute, and that setting
+// holds per device.  `done` (one per kernel, zero-initialised) keeps one bit per device ordinal so that the call
+// is made once for every device the kernel is launched on; two threads racing here both make the same call.
+inline int allow_dynamic_lds(const void* kernel, size_t bytes, std::atomic<uint64_t>& done, const char* what) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_error("%s: hipGetDevice failed: %s", what, hipGetErrorString(e));
+    return LL_ELAUNCH;
+  }
+  const uint64_t bit = 1ull << (dev & 63);
+  if (dev < 64 && (done.load(std::memory_order_acquire) & bit)) return LL_OK;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) {
+    set_error("%s: cannot reserve %zu bytes of LDS: %s", what, bytes, hipGetErrorString(e));
+    return LL_ELAUNCH;
+  }
+  if (dev < 64) done.fetch_or(bit, std::memory_order_release);
+  return LL_OK;
+}
 
 // ----------------------------------------------------------------------------- formats
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
