@@ -333,6 +333,38 @@ def test_config3_full_size_fused_decode_equals_attention_over_the_dequantized_ca
     assert (out_c.float() - 0.75).abs().max().item() <= 2 ** -7
 
 
+@pytest.mark.parametrize("H,bts,n_cached,n_new,Lq", [(4, 96, 232, 77, 50), (2, 64, 129, 0, 130), (2, 192, 200, 300, 33),
+                                                     (8, 16, 40, 5, 7)])
+def test_kernel_accepts_any_number_of_cached_tokens(gpu, H, bts, n_cached, n_new, Lq):
+    """The entry point promises any n_cached >= 0: the last slot may be only partly attended, and neither the slot
+    size nor n_cached need be a multiple of the kernel's 64- and 128-key tiles.  Checked against the oracle's
+    attention over the oracle's dequantization of the attended part of the slots plus the bf16 tail."""
+    from longlive_amd.utils.quant import SlotPointerTable
+    n_slots = -(-n_cached // bts)
+    ks, vs, kq, vq = [], [], [], []
+    for i in range(n_slots):
+        k, v = _randn((bts, H, 128), 900 + i, 1.0 + 0.25 * i), _randn((bts, H, 128), 950 + i, 0.5 + 0.25 * i)  # amax differs per slot
+        ks.append(_oracle_slot(k)[0])
+        vs.append(_oracle_slot(v)[0])
+        kq.append(quantize_to_fp4(k.reshape(-1, 128).to(gpu), CFG))
+        vq.append(quantize_to_fp4(v.reshape(-1, 128).to(gpu), CFG))
+    kt, vt = SlotPointerTable(kq), SlotPointerTable(vq)
+    tables = [kt.values, kt.scales, kt.amax, vt.values, vt.scales, vt.amax]
+    q = _randn((Lq, H, 128), 990)
+    k_new = _randn((n_new, H, 128), 991) if n_new else None
+    v_new = _randn((n_new, H, 128), 992) if n_new else None
+    out = _native.kv_attention(q.to(gpu), tables, n_cached, bts, 6.0, 256.0, k_new.to(gpu) if n_new else None,
+                               v_new.to(gpu) if n_new else None, 128 ** -0.5)
+    k_all = np.concatenate(ks)[:n_cached]
+    v_all = np.concatenate(vs)[:n_cached]
+    if n_new:
+        k_all = np.concatenate([k_all, k_new.float().numpy()])
+        v_all = np.concatenate([v_all, v_new.float().numpy()])
+    ref = o.attention(q.float().numpy(), k_all, v_all)
+    err = np.abs(out.float().cpu().numpy() - ref).max()
+    assert err <= 2e-2, err
+
+
 def test_release_shape_rolling_window_equals_attention_over_the_dequantized_slots(gpu):
     """Shapes of the reference's released NVFP4 configuration (configs/nvfp4/inference_nvfp4.yaml:3-7: chunks of 8
     frames = 7040 tokens, window 32 frames = 4 blocks, sink 8 frames = 1 block), streamed past the point where
