@@ -145,6 +145,40 @@ def run_block(torch, dev, steps):
             "workload": "configs[3]: one NVFP4 DiT block forward, 1228.2 GFLOP (783.4 linears + 428.2 self-attn + 16.6 cross-attn)"}
 
 
+def run_block_release(torch, dev, steps):
+    """One DiT block at the shapes of the reference's released NVFP4 configuration (chunks of 8 latent frames =
+    7040 tokens, window of 32 frames = 4 cache blocks, sink 8 frames): the chunk attends the sink block, two
+    cached blocks and itself, 28160 keys.  Not one of the benchmark configurations; reported beside them."""
+    from longlive_amd.dit import DiTBlock
+    from longlive_amd.fouroversix import ModelQuantizationConfig, QuantizationConfig
+    from longlive_amd.utils import kv_cache as kvc
+    from longlive_amd.utils.quant import quantize_model_with_filter
+    from longlive_amd.utils.rope import build_rope_angles, rope_cos_sin
+
+    tokens, blocks = 8 * 880, 4
+    g = torch.Generator().manual_seed(5)
+    kv_cfg = QuantizationConfig(scale_rule="mse")
+    cache = kvc.initialize_kv_cache(1, tokens, blocks, HEADS, 128, kv_cfg, dev)[0]
+    for chunk in range(blocks):
+        q, k, v = (torch.randn(1, tokens, HEADS, 128, generator=g).bfloat16().to(dev) for _ in range(3))
+        _, (g_end, l_end, info) = kvc.kv_cache_attention(q, k, v, cache, chunk * tokens, sink_tokens=tokens)
+        kvc.apply_cache_update(cache, g_end, l_end, info, kv_cfg)
+    torch.manual_seed(5)
+    block = DiTBlock(DIM, FFN, HEADS).to(dev)
+    block, _ = quantize_model_with_filter(block, ModelQuantizationConfig(), use_default_filtered_modules=True,
+                                          materialize_for_inference=True, verbose=False)
+    x = torch.randn(1, tokens, DIM, generator=g).bfloat16().to(dev)
+    e0 = torch.randn(1, 8, 6, DIM, generator=g).bfloat16().to(dev)
+    ctx = torch.randn(1, M_TEXT, DIM, generator=g).bfloat16().to(dev)
+    cos, sin = rope_cos_sin(build_rope_angles(128), 8, 22, 40, 32, dev)
+    with torch.no_grad():
+        ms = _time_events(torch, lambda: block(x, e0, cos, sin, ctx, cache, blocks * tokens, sink_tokens=tokens), steps)
+    gflop = (2.0 * tokens * (8 * DIM * DIM + 2 * DIM * FFN) - 2 * 2.0 * (tokens - M_TEXT) * DIM * DIM  # k/v of cross-attention run on the text
+             + 4.0 * tokens * (blocks * tokens) * 128 * HEADS + 4.0 * tokens * M_TEXT * 128 * HEADS) / 1e9
+    return {"block_ms": ms, "block_TFLOPs": gflop / ms, "gflop": gflop,
+            "workload": "released configuration: one NVFP4 DiT block forward, 7040 tokens, 28160 keys (3 FP4 slots + bf16 chunk)"}
+
+
 def run_e2e(torch, dev):
     """configs[4]: 30 blocks, 10 chunks of 3 latent frames, 4 denoising forwards + 1 cache-rewrite forward each."""
     from longlive_amd.dit import DiTConfig, StreamingGenerator
@@ -205,7 +239,7 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the attention / block / end-to-end figures")
-    ap.add_argument("--workload", choices=["linears", "attention", "block", "e2e", "copy"], default="linears")
+    ap.add_argument("--workload", choices=["linears", "attention", "block", "block_release", "e2e", "copy"], default="linears")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives are part of this path); use --gpus 1")
@@ -228,6 +262,7 @@ def main() -> None:
         return
     if args.workload != "linears":
         res = {"attention": lambda: run_attention(torch, dev, args.steps), "block": lambda: run_block(torch, dev, args.steps),
+               "block_release": lambda: run_block_release(torch, dev, args.steps),
                "e2e": lambda: run_e2e(torch, dev)}[args.workload]()
         print(json.dumps(res))
         return
@@ -342,6 +377,7 @@ def main() -> None:
         extras = {}
         for key, fn in (("gemm_shapes", lambda: run_gemm_shapes(torch, dev, work, cfg, 10)),
                         ("attention", lambda: run_attention(torch, dev, 10)), ("block", lambda: run_block(torch, dev, 10)),
+                        ("block_release_shapes", lambda: run_block_release(torch, dev, 5)),
                         ("e2e", lambda: run_e2e(torch, dev))):
             try:
                 extras[key] = fn()
