@@ -35,6 +35,7 @@ enum {
 
 enum { LL_RULE_STATIC_6 = 0, LL_RULE_STATIC_4 = 1, LL_RULE_MAE = 2, LL_RULE_MSE = 3, LL_RULE_ABS_MAX = 4 };
 enum { LL_ACT_NONE = 0, LL_ACT_GELU_TANH = 1 };
+#define LL_AMAX_PARTS 1024 /* partial maxima per tensor: size of the quantizer's scratch and of an amax sink */
 enum { LL_DTYPE_BF16 = 0, LL_DTYPE_F16 = 1, LL_DTYPE_F32 = 2 }; /* utils/kernel/kv_dequant.py:18-25 */
 
 const char* ll_last_error(void);
@@ -67,7 +68,6 @@ int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ldx, int rule
  * ll_nvfp4_quantize_from_sink reads the slots of that epoch.  Calls that share a buffer must be ordered
  * (one stream).
  */
-#define LL_AMAX_PARTS 1024
 typedef struct ll_amax_sink {
   uint64_t* parts;   /* device memory, LL_AMAX_PARTS entries, 8-byte aligned */
   uint32_t epoch;    /* > 0 */
@@ -141,10 +141,13 @@ int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A_scales, co
 
 /*
  * Replaces torch.ops.longlive_kernels.dequantize_kv_cache_fp4 (utils/kernel/kv_dequant.cpp:14,
- * utils/kernel/kv_dequant_cuda.cu:59-239) and the Triton fp4_dequantize it falls back to
- * (utils/nvfp4_kernel.py:40-176): n_blocks cache slots, each NVFP4 [rows_padded, 128] holding
+ * utils/kernel/kv_dequant_cuda.cu:59-239): n_blocks cache slots, each NVFP4 [rows_padded, 128] holding
  * block_token_size*num_heads logical rows, are dequantized to out[1, n_blocks*block_token_size, num_heads, 128]
- * as f32(e2m1) * f32(scale) * (amax / (e2m1_max*e4m3_max)).
+ * as cast((f32(e2m1) * f32(scale)) * gs) with the slot scale gs = amax * f32(1.0 / (e2m1_max*e4m3_max)), the
+ * reciprocal formed in double (kv_dequant_cuda.cu:95-106, 216).  The Triton routine the reference falls back to
+ * when its extension is not built (utils/nvfp4_kernel.py:40-176 with utils/quant.py:753-756) divides amax by the
+ * denominator instead, which moves gs by at most one fp32 ulp; the fused path is the one followed here, by this
+ * entry point and by ll_kv_attention alike.
  *   values_ptrs / scales_ptrs / amax_ptrs: DEVICE arrays of n_blocks device pointers.
  */
 int ll_kv_dequantize_blocks(const uint64_t* values_ptrs, const uint64_t* scales_ptrs, const uint64_t* amax_ptrs,
@@ -156,6 +159,8 @@ int ll_kv_dequantize_blocks(const uint64_t* values_ptrs, const uint64_t* scales_
  * (wan_5b/modules/causal_model.py:557-567, 628-671, 673-724, 781; wan_5b/modules/attention.py:84-306):
  *   out[t, h, :] = softmax_j(q[t, h, :] . k_j[h, :] * scale) v_j   over the key list
  *       [ n_cached tokens read from the NVFP4 slots (slot = j / block_token_size) | n_new bf16 tokens ]
+ *   Cached keys and values enter the products as the bf16 values ll_kv_dequantize_blocks(..., LL_DTYPE_BF16)
+ *   returns for the same slots, bit for bit.
  *   q bf16 [Lq, H, 128]; k_new, v_new bf16 [n_new, H, 128] (the caller passes the smoothed K of the
  *   current chunk, utils/quant.py:797-798); out bf16 [Lq, H, 128].  No mask (causal_model.py:781).
  *   k_* / v_* pointer arrays: DEVICE arrays of device pointers, one per slot, slot layout as above
@@ -239,10 +244,6 @@ int ll_qk_norm_rope(const void* x, int64_t rows, int num_heads, const void* weig
 int ll_qk_norm_rope_pair(const void* q, const void* k, int64_t rows, int num_heads, const void* q_weight,
                          const void* k_weight, float eps, const float* cos, const float* sin, int64_t seq_len,
                          void* q_out, void* k_out, void* k_out_smooth, void* stream);
-
-/* Test hooks: hardware fp32->e4m3 / fp32->e2m1 conversions applied to n floats (used by the GPU tests to
- * check the instructions the fast paths rely on against the software codecs). mode 0: e4m3, 1: e2m1. */
-int ll_debug_convert(const float* in, int64_t n, int mode, uint8_t* out, void* stream);
 
 #ifdef __cplusplus
 }

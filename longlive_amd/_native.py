@@ -65,7 +65,6 @@ _SIGNATURES = {
                                  c_void_p, c_void_p]),
     "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
     "ll_layer_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p]),
-    "ll_debug_convert": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p]),
 }
 
 
@@ -471,11 +470,3 @@ def layer_norm(x, weight, bias, eps=1e-6, amax_out=None):
                                     ctypes.byref(sink), _stream())
     _check(code, "ll_layer_norm")
     return out.view(x.shape)
-
-
-def debug_convert(x: torch.Tensor, mode: int) -> torch.Tensor:
-    x = x.contiguous().float()
-    out = torch.empty(x.numel(), dtype=torch.uint8, device=x.device)
-    code = load().ll_debug_convert(x.data_ptr(), x.numel(), mode, out.data_ptr(), _stream())
-    _check(code, "ll_debug_convert")
-    return out

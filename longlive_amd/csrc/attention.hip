@@ -9,7 +9,8 @@
 // 256 registers (64 for O^T, 32 for S^T, 32 for its Q fragments, the rest for tile fragments, raw FP4 data
 // and addressing), which is what lets two waves share a SIMD: while one wave converts FP4 data or evaluates
 // exponentials, the other one's MFMAs run.  Per iteration all 512 threads decode 128 keys of K and V
-// (e2m1 x e4m3 x amax/(6*256) -> bf16, the values the reference's dequantized bf16 cache holds) into LDS, both
+// ((e2m1 x e4m3) x slot scale -> bf16: bit for bit the values the reference's fused cache dequantization and
+// ll_kv_dequantize_blocks produce, utils/kernel/kv_dequant_cuda.cu:95-106) into LDS, both
 // row-major (one row per key), with the same thread layout and the same byte offsets for K and V.  The MFMAs
 // compute S^T = K Q^T and O^T = V^T P^T (v_mfma_f32_32x32x16_bf16), so every lane owns one query column: row max /
 // row sum need no cross-lane traffic beyond one swap between the wave halves, and the online-softmax rescale is
@@ -70,21 +71,42 @@ __device__ __forceinline__ float max_over_wave_halves(float v) {
   return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
-__device__ __forceinline__ float fp8_byte_to_f32(uint32_t word, int byte) {
-  typedef float float2v_ __attribute__((ext_vector_type(2)));
-  const float2v_ lo = __builtin_amdgcn_cvt_pk_f32_fp8((int)word, false);
-  const float2v_ hi = __builtin_amdgcn_cvt_pk_f32_fp8((int)word, true);
-  return byte == 0 ? lo[0] : byte == 1 ? lo[1] : byte == 2 ? hi[0] : hi[1];
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+
+// The two e4m3 block scales in the low 16 bits of `word`, as f16 pairs (s, s) ready for a packed multiply.
+__device__ __forceinline__ void block_scales_f16(uint32_t word, half2v (&s2)[2]) {
+  const half2v sc = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(word, 1.0f, false);
+  s2[0] = half2v{sc[0], sc[0]};
+  s2[1] = half2v{sc[1], sc[1]};
 }
 
-// 8 e2m1 codes (one dword) times sf -> 8 floats
-__device__ __forceinline__ void fp4x8_to_f32(uint32_t w, float sf, float (&o)[8]) {
-  const float2v q0 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0);
-  const float2v q1 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1);
-  const float2v q2 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2);
-  const float2v q3 = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3);
-  o[0] = q0[0] * sf; o[1] = q0[1] * sf; o[2] = q1[0] * sf; o[3] = q1[1] * sf;
-  o[4] = q2[0] * sf; o[5] = q2[1] * sf; o[6] = q3[0] * sf; o[7] = q3[1] * sf;
+// f32(t.lo) * g and f32(t.hi) * g with one instruction each: the mixed-precision fused multiply-add widens
+// the selected f16 half on the way in (op_sel_hi marks source 0 as f16, op_sel picks its upper half).  The
+// addend is -0, which leaves the product untouched, signed zeros included.
+__device__ __forceinline__ float widen_mul_lo(half2v t, float g) {
+  float r;
+  asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel_hi:[1,0,0]" : "=v"(r) : "v"(t), "v"(g), "s"(-0.0f));
+  return r;
+}
+__device__ __forceinline__ float widen_mul_hi(half2v t, float g) {
+  float r;
+  asm("v_fma_mix_f32 %0, %1, %2, %3 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(r) : "v"(t), "v"(g), "s"(-0.0f));
+  return r;
+}
+
+// 8 e2m1 codes (one dword) of a block with scale s2 = (s, s) and slot scale gs -> the 8 fp32 values
+// (code * s) * gs, the expression of the reference's fused cache dequantization (utils/kernel/kv_dequant_cuda.cu:
+// 97-106).  code * s has at most six significant bits and lies within [2^-10, 2688], so the packed f16 product is
+// exact; the multiplication by gs is the only rounding, done in fp32.
+__device__ __forceinline__ void fp4x8_to_f32(uint32_t w, half2v s2, float gs, float (&o)[8]) {
+  const half2v t0 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 0) * s2;
+  const half2v t1 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 1) * s2;
+  const half2v t2 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 2) * s2;
+  const half2v t3 = __builtin_amdgcn_cvt_scalef32_pk_f16_fp4(w, 1.0f, 3) * s2;
+  o[0] = widen_mul_lo(t0, gs); o[1] = widen_mul_hi(t0, gs);
+  o[2] = widen_mul_lo(t1, gs); o[3] = widen_mul_hi(t1, gs);
+  o[4] = widen_mul_lo(t2, gs); o[5] = widen_mul_hi(t2, gs);
+  o[6] = widen_mul_lo(t3, gs); o[7] = widen_mul_hi(t3, gs);
 }
 
 // Raw FP4 data prefetched one iteration ahead.  Only packed bytes and scale bytes are held in registers
@@ -127,16 +149,17 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
 }
 
 // Decode 32 elements of one key (K or V) to bf16 and store the 64 bytes into the key's LDS row.
-// kind: 0 = fp4 slot data in f (gs = slot amax / (e2m1_max * e4m3_max)), 1 = bf16 row at src, 2 = zeros.
+// kind: 0 = fp4 slot data in f (gs = slot amax * f32(1 / (e2m1_max * e4m3_max))), 1 = bf16 row at src, 2 = zeros.
 __device__ __forceinline__ void store_row(const KRaw& f, int kind, float gs, const uint4* src, uint8_t* dst) {
   uint4* d4 = reinterpret_cast<uint4*>(dst);
   if (kind == 0) {
     const uint32_t w[4] = {f.v.x, f.v.y, f.v.z, f.v.w};
+    half2v s2[2];
+    block_scales_f16(f.scales, s2);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const float sf = fp8_byte_to_f32(f.scales, j >> 1) * gs;
       float v8[8];
-      fp4x8_to_f32(w[j], sf, v8);
+      fp4x8_to_f32(w[j], s2[j >> 1], gs, v8);
       d4[j] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]), pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
     }
   } else if (kind == 1) {
@@ -209,7 +232,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   int iter_base = 0;
   int k_slot = k_local / p.bts, k_off = k_local - k_slot * p.bts;
   uint32_t k_vo, k_so;
-  float k_gs, v_gs;  // slot scale amax / (e2m1_max * e4m3_max) of the thread's key, for K and for V
+  float k_gs, v_gs;  // slot scale amax * f32(1 / (e2m1_max * e4m3_max)) of the thread's key, for K and for V
   auto locate = [&]() __attribute__((always_inline)) {
     const int64_t row = (int64_t)k_off * p.H + head;
     k_vo = (uint32_t)row * 64u + k_quarter * 16u;
@@ -359,6 +382,9 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     float16v sc[2];
     {
       const uint32_t wk[4] = {kf.v.x, kf.v.y, kf.v.z, kf.v.w}, wv[4] = {vf.v.x, vf.v.y, vf.v.z, vf.v.w};
+      half2v ks2[2], vs2[2];
+      block_scales_f16(kf.scales, ks2);
+      block_scales_f16(vf.scales, vs2);
       uint8_t* kdst = nxt + k_dst_off;
       uint8_t* vdst = nxt + v_dst_off;
       const uint8_t* krow0 = cur + kp * kKTileBytes + l32 * kKPitch + lh * 16;
@@ -381,9 +407,8 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
         {  // one dword (8 elements) of the prefetched row per step: K in the even steps, V in the odd ones
           const int j = ks >> 1;
           const bool is_k = (ks & 1) == 0;
-          const float sf = fp8_byte_to_f32(is_k ? kf.scales : vf.scales, j >> 1) * (is_k ? k_gs : v_gs);
           float v8[8];
-          fp4x8_to_f32(is_k ? wk[j] : wv[j], sf, v8);
+          fp4x8_to_f32(is_k ? wk[j] : wv[j], is_k ? ks2[j >> 1] : vs2[j >> 1], is_k ? k_gs : v_gs, v8);
           reinterpret_cast<uint4*>(is_k ? kdst : vdst)[j] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
                                                                        pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
         }
@@ -567,7 +592,7 @@ extern "C" int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads, co
   p.n_new = n_new;
   p.bts = n_cached > 0 ? block_token_size : (1 << 30);
   p.n_slots = n_slots;
-  p.inv_denom = n_cached > 0 ? 1.0f / (e2m1_max * e4m3_max) : 0.f;
+  p.inv_denom = n_cached > 0 ? kv_inverse_denominator(e2m1_max, e4m3_max) : 0.f;
   p.k_new = static_cast<const uint16_t*>(k_new);
   p.v_new = static_cast<const uint16_t*>(v_new);
   p.scale_log2 = softmax_scale * 1.4426950408889634f;

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(256) void kv_dequantize_kernel(const uint64_t* __re
                                                             const uint64_t* __restrict__ scales_ptrs,
                                                             const uint64_t* __restrict__ amax_ptrs,
                                                             int64_t rows_per_slot, int64_t total_groups,
-                                                            float denom, void* __restrict__ out) {
+                                                            float inv_denom, void* __restrict__ out) {
   const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;  // group of 8 elements; 16 groups per row
   if (g >= total_groups) return;
   const int64_t grow = g >> 4;
@@ -90,7 +90,10 @@ __global__ __launch_bounds__(256) void kv_dequantize_kernel(const uint64_t* __re
   const float amax = *reinterpret_cast<const float*>(amax_ptrs[slot]);
   const uint32_t packed = *reinterpret_cast<const uint32_t*>(values + r * 64 + (c >> 1));
   const float s = e4m3_to_f32(scales[blocked_scale_offset(r, c >> 4, 8)]);
-  const float gs = amax / denom;  // global scale formed first (utils/quant.py:753-756)
+  // The slot scale as the reference's fused path forms it: amax * f32(1 / (e2m1_max * e4m3_max))
+  // (utils/kernel/kv_dequant_cuda.cu:95, 216), then (code * scale) * gs left to right (:97-106): the first product
+  // is exact, so every value carries one fp32 rounding.  kv_attention_kernel decodes with the same expression.
+  const float gs = amax * inv_denom;
   float v[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) v[i] = (kE2M1[(packed >> (4 * i)) & 0xF] * s) * gs;
@@ -144,20 +147,20 @@ extern "C" int ll_kv_dequantize_blocks(const uint64_t* values_ptrs, const uint64
   const int64_t rows_per_slot = (int64_t)num_heads * block_token_size;
   const int64_t groups = rows_per_slot * n_blocks * 16;
   const dim3 grid((unsigned)((groups + 255) / 256));
-  const float denom = e2m1_max * e4m3_max;
+  const float inv_denom = kv_inverse_denominator(e2m1_max, e4m3_max);
   hipStream_t s = static_cast<hipStream_t>(stream);
   switch (out_dtype) {
     case LL_DTYPE_BF16:
       hipLaunchKernelGGL(kv_dequantize_kernel<LL_DTYPE_BF16>, grid, dim3(256), 0, s, values_ptrs, scales_ptrs,
-                         amax_ptrs, rows_per_slot, groups, denom, out);
+                         amax_ptrs, rows_per_slot, groups, inv_denom, out);
       break;
     case LL_DTYPE_F16:
       hipLaunchKernelGGL(kv_dequantize_kernel<LL_DTYPE_F16>, grid, dim3(256), 0, s, values_ptrs, scales_ptrs,
-                         amax_ptrs, rows_per_slot, groups, denom, out);
+                         amax_ptrs, rows_per_slot, groups, inv_denom, out);
       break;
     case LL_DTYPE_F32:
       hipLaunchKernelGGL(kv_dequantize_kernel<LL_DTYPE_F32>, grid, dim3(256), 0, s, values_ptrs, scales_ptrs,
-                         amax_ptrs, rows_per_slot, groups, denom, out);
+                         amax_ptrs, rows_per_slot, groups, inv_denom, out);
       break;
     default:
       LL_REQUIRE(false, "ll_kv_dequantize_blocks: unknown dtype code %d", out_dtype);

@@ -542,10 +542,13 @@ extern "C" int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A
   // work per MFMA, but four times the workgroups) finish sooner.  Configuration 3 (64x128) is only reachable
   // through the override below.
   if (((M + 127) / 128) * ((N + 127) / 128) <= 128) best = 4;
-  if (const char* force = getenv("LL_GEMM_TILE")) {  // tuning aid: 0..4 selects a tile configuration
-    const int f = atoi(force);
-    if (f >= 0 && f < 5) best = f;
-  }
+  // Tuning aid: LL_GEMM_TILE=0..4 in the environment when the library is first used pins one tile configuration.
+  static const int forced_tile = [] {
+    const char* force = getenv("LL_GEMM_TILE");
+    const int f = force ? atoi(force) : -1;
+    return (f >= 0 && f < 5) ? f : -1;
+  }();
+  if (forced_tile >= 0) best = forced_tile;
 #define LL_GEMM_ARGS A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, (int)M, (int)N, \
                      (int)Mp, (int)Np, (int)Kp, D, ldd, epi, s
   switch (best) {

@@ -113,6 +113,12 @@ __host__ __device__ __forceinline__ void rule_limits(int rule, float& e2, float&
   e4 = (rule == LL_RULE_STATIC_6 || rule == LL_RULE_STATIC_4) ? 448.0f : 256.0f;
 }
 
+// 1 / (e2m1_max * e4m3_max) of a KV-cache slot as the reference's fused dequantization forms it: the reciprocal
+// in double, rounded to fp32 once (utils/kernel/kv_dequant_cuda.cu:216); the slot scale is amax times this.
+inline float kv_inverse_denominator(float e2m1_max, float e4m3_max) {
+  return static_cast<float>(1.0 / (static_cast<double>(e2m1_max) * static_cast<double>(e4m3_max)));
+}
+
 // ----------------------------------------------------------------------------- wave helpers
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll

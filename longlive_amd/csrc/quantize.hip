@@ -460,18 +460,6 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
   }
 }
 
-// ----------------------------------------------------------------------------- hardware codec probe
-__global__ void debug_convert_kernel(const float* __restrict__ in, int64_t n, int mode, uint8_t* __restrict__ out) {
-  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const float v = in[i];
-  if (mode == 0) {
-    out[i] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(v, 0.0f, 0, false) & 0xFF);
-  } else {
-    out[i] = (uint8_t)(__builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, v, 0.0f, 1.0f, 0) & 0xF);
-  }
-}
-
 }  // namespace ll
 
 extern "C" size_t ll_nvfp4_quantize_workspace_floats(void) { return ll::kAmaxParts; }
@@ -530,13 +518,4 @@ extern "C" int ll_nvfp4_quantize_from_sink(const void* x, int64_t M, int64_t K, 
   using namespace ll;
   LL_REQUIRE(amax_sink, "ll_nvfp4_quantize_from_sink: null amax sink");
   return quantize_impl(x, M, K, ldx, rule, values, scales, amax, 0, nullptr, amax_sink, stream);
-}
-
-extern "C" int ll_debug_convert(const float* in, int64_t n, int mode, uint8_t* out, void* stream) {
-  using namespace ll;
-  LL_REQUIRE(in && out && n > 0 && (mode == 0 || mode == 1), "ll_debug_convert: bad arguments");
-  hipLaunchKernelGGL(debug_convert_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), in, n, mode, out);
-  LL_CHECK_LAUNCH("debug_convert_kernel");
-  return LL_OK;
 }

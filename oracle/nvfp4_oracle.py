@@ -17,7 +17,8 @@ Reference files followed (paths relative to the reference checkout):
                   fouroversix/src/fouroversix/quantize/quantized_tensor.py:10-18
 * dequantize      fouroversix/src/fouroversix/quantize/quantized_tensor.py:21-53,184-214
 * matmul          fouroversix/src/fouroversix/matmul/pytorch.py:22-41
-* KV dequant      utils/nvfp4_kernel.py:40-176, utils/quant.py:731-768
+* KV dequant      utils/kernel/kv_dequant_cuda.cu:59-107, 216 (the path the reference takes when its extension is
+                  built), utils/nvfp4_kernel.py:40-176 + utils/quant.py:731-768 (its fallback)
 * KV attention    wan_5b/modules/causal_model.py:491-724,781 ; wan_5b/modules/attention.py:260-306
 * RoPE            utils/rope_triton.py:36-135 ; wan_5b/modules/model.py:29-36 ;
                   wan_5b/modules/causal_model.py:90-194
@@ -32,9 +33,16 @@ Pinning status (what independent evidence fixes each function):
 * quantize mse/mae/abs_max    selection invariant in fp64 + golden vectors written by the
                               reference's own PyTorch backend (tests/golden/)
 * dequantize / matmul         exhaustive code x scale table; fp64 brute force; integer special case
+* kv_dequantize               exact rational arithmetic, torch float32/float8/bfloat16 evaluation of the same
+                              expression, and the golden-pinned dequantize (within one bf16 ulp, equal away
+                              from rounding boundaries)
+* k_smooth                    bit-exact against torch's bf16 `k - k.mean(-1, keepdim=True)`
 * attention / RoPE / adaLN    fp64 textbook forms, torch library routines (layer_norm,
                               complex multiply), norm preservation
-* gate_residual / gelu_tanh   the two eager bf16 operations / torch.nn.functional.gelu(approximate="tanh")
+* gate_residual               the two eager bf16 operations
+* gelu_tanh                   torch.nn.functional.gelu(approximate="tanh") on every bf16 value of [-8, 8] (equal
+                              outside the negative tail, where torch's fp32 `1 + tanh` cancels; there within
+                              the cancellation bound) and the algebraically equal logistic form in fp64
 
 Parity unpinned: the reference's production matmul is a CUTLASS kernel (fouroversix/.gitmodules, submodule
 absent, no pinned commit) and its attention is flash-attn 2.8.3 (not installed); neither result is
@@ -308,16 +316,35 @@ def fp4_matmul(a, b, out_bf16=True):
     return round_bf16(out) if out_bf16 else out
 
 
-def kv_dequantize(values, scales_blocked, amax, rule="mse"):
-    """utils/nvfp4_kernel.py:125-133: f32(e2m1) * f32(scale) * (amax / (6*256)) -> bf16.
-    The global scale is formed first (utils/quant.py:753-756)."""
+def kv_global_scale(amax, rule="mse", path="fused"):
+    """fp32 per-slot scale of the KV cache.  The reference has two code paths that differ in this one value:
+
+    * "fused"  the CUDA extension, the path taken whenever it is built:
+               amax * f32(1.0 / (e2m1_max * e4m3_max)), the reciprocal formed in double on the host
+               (utils/kernel/kv_dequant_cuda.cu:95, 216);
+    * "triton" the per-block fallback: amax / (e2m1_max * e4m3_max), an fp32 division (utils/quant.py:753-756).
+
+    The two agree except where the rounded reciprocal tips the product over a rounding boundary (1 ulp)."""
+    e2, e4 = rule_limits(rule)
+    if path == "fused":
+        return F32(F32(amax) * F32(1.0 / (e2 * e4)))
+    if path == "triton":
+        return F32(F32(amax) / F32(e2 * e4))
+    raise ValueError(path)
+
+
+def kv_dequantize(values, scales_blocked, amax, rule="mse", path="fused", dtype="bf16"):
+    """One cache slot -> its dequantized values: (f32(e2m1) * f32(scale)) * global_scale, evaluated left to
+    right in fp32 and cast (utils/kernel/kv_dequant_cuda.cu:97-106; utils/nvfp4_kernel.py:125-133 has the same
+    expression).  The product of code and scale is exact, so the fp32 value carries one rounding.
+    ``path`` selects how the global scale is formed (see kv_global_scale); dtype "bf16" or "f32"."""
     Mp = values.shape[0]
     Kp = values.shape[1] * 2
     v = unpack_e2m1(values)
     s = e4m3_decode(from_blocked(np.asarray(scales_blocked, dtype=np.uint8), (Mp, Kp // 16)))
-    e2, e4 = rule_limits(rule)
-    g = F32(amax) / F32(e2 * e4)
-    return round_bf16((v * np.repeat(s, 16, axis=1)) * g)
+    g = kv_global_scale(amax, rule, path)
+    res = ((v * np.repeat(s, 16, axis=1)) * g).astype(F32)
+    return round_bf16(res) if dtype == "bf16" else res
 
 
 # --------------------------------------------------------------------------- attention

@@ -33,3 +33,25 @@ def weights(shape, seed) -> torch.Tensor:
 
 def u8(t: torch.Tensor) -> np.ndarray:
     return t.detach().cpu().contiguous().view(torch.uint8).numpy().copy()
+
+
+def hardware_convert(x: torch.Tensor, mode: int) -> torch.Tensor:
+    """fp32 -> e4m3 byte (mode 0) or e2m1 nibble (mode 1) with the gfx950 conversion instructions, through the
+    test-only library built next to the product library (longlive_amd/csrc/test_hooks.hip)."""
+    import ctypes
+    import os
+
+    from longlive_amd import _native
+
+    path = os.path.join(os.path.dirname(_native.LIB_PATH), "libll_nvfp4_testhooks.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: run `make -C longlive_amd/csrc`")
+    lib = ctypes.CDLL(path)
+    lib.ll_test_convert.restype = ctypes.c_int
+    lib.ll_test_convert.argtypes = [ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    x = x.contiguous().float()
+    out = torch.empty(x.numel(), dtype=torch.uint8, device=x.device)
+    code = lib.ll_test_convert(x.data_ptr(), x.numel(), mode, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    if code != 0:
+        raise RuntimeError(f"ll_test_convert failed with {code}")
+    return out

@@ -474,3 +474,102 @@ def test_norm_rope_of_q_and_k_in_one_launch_equals_two_launches(gpu, S, H):
     assert torch.equal(rk, one_k) and torch.equal(sk, one_s)
     with pytest.raises(ValueError):
         _native.qk_norm_rope_pair(q, k[:-1], wq, wk, 1e-6, cos, sin, H)
+
+
+# --------------------------------------------------------------------------- cached values, bit for bit
+# Slot amax values for which the order of the three factors of a cached value is visible in bf16.  A cached
+# value is (code * scale) * gs with gs = amax * f32(1/1536) (utils/kernel/kv_dequant_cuda.cu:95-106, 216).
+# For the first group, (scale * gs) * code rounds to a different bf16 number for dozens of (scale, code)
+# pairs; for the second group the Triton fallback's gs = amax / 1536 (utils/quant.py:753-756) does.  Found by
+# enumerating all 2^23 fp32 mantissas of gs on the CPU; the test re-checks both properties before relying on them.
+ORDER_SENSITIVE_AMAX = [3.0625, 3.4375, 1.53125, 3.106250047683716, 6.145832538604736, 3.009615421295166]
+DIVISION_SENSITIVE_AMAX = [4.34375, 6.640625476837158, 2.0484375953674316, 5.642045021057129]
+
+
+def _raw_slots(n_slots, rows, amaxes, seed, gpu):
+    """Slots of random bytes: every e2m1 code (both zeros included) under every finite e4m3 scale byte."""
+    rng = np.random.default_rng(seed)
+    host, dev = [], []
+    for i in range(n_slots):
+        values = rng.integers(0, 256, size=(rows, 64), dtype=np.uint8)
+        sb = rng.integers(0, 127, size=(rows, 8), dtype=np.uint8) | (rng.integers(0, 2, size=(rows, 8), dtype=np.uint8) << 7)
+        scales = o.to_blocked(sb)
+        amax = np.float32(amaxes[i % len(amaxes)])
+        host.append((values, scales, amax))
+        dev.append((torch.from_numpy(values).to(gpu), torch.from_numpy(scales).to(gpu),
+                    torch.tensor([amax], dtype=torch.float32, device=gpu)))
+    return host, dev
+
+
+def _table(dev_slots, gpu):
+    t = torch.tensor([[s[j].data_ptr() for s in dev_slots] for j in range(3)], dtype=torch.int64).to(gpu)
+    return t[0], t[1], t[2]
+
+
+@pytest.mark.parametrize("n_cached,n_new", [(384, 0), (360, 0), (64, 0), (384, 100), (200, 128)])
+def test_attention_reads_cached_values_bit_for_bit(gpu, n_cached, n_new):
+    """The value the attention kernel decodes for a cached token is the bf16 number ll_kv_dequantize_blocks
+    returns for it, which is the oracle's (reference: utils/kernel/kv_dequant_cuda.cu:95-106).  Read back
+    through the kernel itself: the K slots hold two-hot keys (position t % 64 and 64 + t / 64) and query t is
+    the matching two-hot vector, so the score of key t exceeds every other by > 500 in the exponent, the softmax
+    is exactly one-hot, and out[t] = 1.0 * V[t] / 1.0.  The V slots are random bytes under slot amax values chosen
+    so that any other order of the three factors, or the fallback's divided slot scale, shows in bf16."""
+    H, T = 2, 64
+    n_slots = (n_cached + T - 1) // T
+    amaxes = ORDER_SENSITIVE_AMAX + DIVISION_SENSITIVE_AMAX
+    host_v, dev_v = _raw_slots(n_slots, T * H, amaxes, seed=n_cached + n_new, gpu=gpu)
+    # keys: token t of the cache -> 64 * (e[t % 64] + e[64 + t // 64]), the same in both heads
+    tok = np.arange(n_slots * T)
+    kmat = np.zeros((n_slots * T, H, 128), dtype=np.float32)
+    kmat[tok, :, tok % 64] = 64.0
+    kmat[tok, :, 64 + tok // 64] = 64.0
+    k_slots = [quantize_to_fp4(torch.from_numpy(kmat[i * T:(i + 1) * T]).bfloat16().reshape(-1, 128).to(gpu), CFG)
+               for i in range(n_slots)]
+    dev_k = [(s.values, s.scale_factors.view(torch.uint8), s.amax) for s in k_slots]
+    q = torch.from_numpy(kmat[:n_cached]).bfloat16().to(gpu)
+    if n_new:  # the chunk's own keys point away from every query, its values are large: any leak would show
+        k_new = torch.zeros(n_new, H, 128, dtype=torch.bfloat16, device=gpu)
+        k_new[:, :, 127] = -64.0
+        v_new = torch.full((n_new, H, 128), 1000.0, dtype=torch.bfloat16, device=gpu)
+    else:
+        k_new = v_new = None
+    tables = _table(dev_k, gpu) + _table(dev_v, gpu)
+    out = _native.kv_attention(q, tables, n_cached, T, 6.0, 256.0, k_new, v_new, 128 ** -0.5)
+    vt = _table(dev_v, gpu)
+    deq = _native.kv_dequantize_blocks(vt[0], vt[1], vt[2], n_slots, H, T, torch.bfloat16, 6.0, 256.0)[0][:n_cached]
+    # the sign of a zero does not survive the accumulation (1.0 * -0 + 0 = +0): zeros compare as equal
+    ob, db = bits_of(out), bits_of(deq)
+    ob[ob == 0x8000] = 0
+    db[db == 0x8000] = 0
+    assert np.array_equal(ob, db), f"{(ob != db).sum()} of {ob.size} values differ"
+    ref = np.concatenate([o.kv_dequantize(v, s, a).reshape(T, H, 128) for v, s, a in host_v])[:n_cached]
+    assert np.array_equal(bits_of(deq), o.f32_to_bf16(ref))
+    # the inputs do tell the candidate expressions apart
+    n_order = n_div = 0
+    for v, s, a in host_v:
+        if float(a) in ORDER_SENSITIVE_AMAX:
+            gs = o.kv_global_scale(a)
+            sf = np.repeat(o.e4m3_decode(o.from_blocked(s, (T * H, 8))), 16, axis=1)
+            other = o.f32_to_bf16((sf * gs).astype(np.float32) * o.unpack_e2m1(v))
+            n_order += int((other != o.f32_to_bf16(o.kv_dequantize(v, s, a))).sum())
+        else:
+            n_div += int((o.f32_to_bf16(o.kv_dequantize(v, s, a, path="triton")) != o.f32_to_bf16(o.kv_dequantize(v, s, a))).sum())
+    if n_slots >= 4:
+        assert n_order >= 50
+    if n_slots >= len(amaxes) - 3:
+        assert n_div >= 10
+
+
+def test_kv_dequantize_blocks_every_code_and_scale(gpu):
+    """ll_kv_dequantize_blocks on random bytes (all codes, all finite scale bytes, both signs) and slot amax values
+    sensitive to the factor order, in all three output types, against the oracle."""
+    H, T = 4, 96
+    host, dev = _raw_slots(5, T * H, ORDER_SENSITIVE_AMAX + DIVISION_SENSITIVE_AMAX, seed=9, gpu=gpu)
+    t = _table(dev, gpu)
+    ref32 = np.concatenate([o.kv_dequantize(v, s, a, dtype="f32").reshape(T, H, 128) for v, s, a in host])
+    got32 = _native.kv_dequantize_blocks(t[0], t[1], t[2], 5, H, T, torch.float32, 6.0, 256.0)[0].cpu().numpy()
+    assert np.array_equal(got32.view(np.uint32), ref32.view(np.uint32))
+    got16 = _native.kv_dequantize_blocks(t[0], t[1], t[2], 5, H, T, torch.bfloat16, 6.0, 256.0)[0]
+    assert np.array_equal(bits_of(got16), o.f32_to_bf16(ref32))
+    gotf16 = _native.kv_dequantize_blocks(t[0], t[1], t[2], 5, H, T, torch.float16, 6.0, 256.0)[0]
+    assert torch.equal(gotf16.cpu(), torch.from_numpy(ref32).half())

@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import nvfp4_oracle as o
-from helpers import activations, bits_of, from_bits, u8, weights
+from helpers import activations, bits_of, from_bits, hardware_convert, u8, weights
 from longlive_amd import _native
 from longlive_amd.fouroversix import QuantizationConfig, QuantizedTensor, quantize_to_fp4
 
@@ -29,14 +29,14 @@ def test_hardware_e4m3_conversion_matches_software_codec(gpu):
     x = np.concatenate([np.linspace(0, 448, 200001, dtype=np.float32),
                         o.e4m3_decode(np.arange(127, dtype=np.uint8)),
                         np.array([2**-10, 2**-10 * 1.001, 3 * 2**-10, 2**-9 * 2.5, 17.0, 19.0, 27.0], dtype=np.float32)])
-    got = _native.debug_convert(torch.from_numpy(x).to(gpu), 0).cpu().numpy()
+    got = hardware_convert(torch.from_numpy(x).to(gpu), 0).cpu().numpy()
     assert np.array_equal(got, o.e4m3_encode(x))
 
 
 def test_hardware_e2m1_conversion_matches_reference_rounding(gpu):
     x = np.concatenate([np.linspace(-6.9, 6.9, 400001, dtype=np.float32),
                         np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, -0.25, -2.5, -5.0, -0.1, 0.0], dtype=np.float32)])
-    got = _native.debug_convert(torch.from_numpy(x).to(gpu), 1).cpu().numpy()
+    got = hardware_convert(torch.from_numpy(x).to(gpu), 1).cpu().numpy()
     ref = o._codes_from_fake_quantized(o._fake_quantize_e2m1(x))
     assert np.array_equal(got, ref)
 
