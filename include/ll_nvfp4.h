@@ -59,6 +59,20 @@ int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ldx, int rule
                       float* workspace, void* stream);
 
 /*
+ * ll_nvfp4_quantize (amax computed by the call) for callers that cannot allocate device memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.
+ * The scratch ll_nvfp4_quantize takes as `workspace` lives in a fixed array of LL_AMAX_PARTS floats that every GPU
+ * the library runs on holds until the process ends; the call allocates and frees nothing.  Same outputs, bit for
+ * bit, as ll_nvfp4_quantize with amax_given == 0.  Limits: M * K <= LL_NOALLOC_MAX_ELEMENTS (larger inputs are
+ * refused with LL_EINVAL); all calls on one GPU share the array, so calls that overlap in time on one GPU (two
+ * streams, two threads) race -- serialize them, or use ll_nvfp4_quantize with one workspace per stream.
+ */
+#define LL_NOALLOC_MAX_ELEMENTS (1ll << 32)
+int64_t ll_nvfp4_quantize_noalloc_max_elements(void);
+int ll_nvfp4_quantize_noalloc(const void* x, int64_t M, int64_t K, int64_t ldx, int rule,
+                              uint8_t* values, uint8_t* scales, float* amax, void* stream);
+
+/*
  * Amax sink.  The tensor-wide absolute maximum that NVFP4 quantization starts from
  * (quantize/pytorch/reference.py:242-255, x.abs().max()) costs a pass over the tensor.  A kernel of this
  * library that writes the tensor can leave the maximum behind instead: it raises LL_AMAX_PARTS 64-bit slots,

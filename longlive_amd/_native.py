@@ -65,6 +65,9 @@ _SIGNATURES = {
                                  c_void_p, c_void_p]),
     "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
     "ll_layer_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p]),
+    "ll_nvfp4_quantize_noalloc_max_elements": (c_int64, []),
+    "ll_nvfp4_quantize_noalloc": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p,
+                                          c_void_p]),
 }
 
 

@@ -519,3 +519,56 @@ extern "C" int ll_nvfp4_quantize_from_sink(const void* x, int64_t M, int64_t K, 
   LL_REQUIRE(amax_sink, "ll_nvfp4_quantize_from_sink: null amax sink");
   return quantize_impl(x, M, K, ldx, rule, values, scales, amax, 0, nullptr, amax_sink, stream);
 }
+
+// ----------------------------------------------------------------------------- entry point that allocates nothing
+// ll_nvfp4_quantize needs kAmaxParts floats of device scratch for the partial maxima of its amax pass.  For callers
+// that cannot allocate, the same floats exist once per GPU as a file-scope device array.  In host code the array's
+// name is only a handle: its device address is looked up once per device (hipGetSymbolAddress, with that device
+// current) and kept; kernels receive that address like any other workspace pointer.
+static __device__ __align__(256) float scratch[LL_AMAX_PARTS];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<float*> g_scratch_ptr[kMaxDevices];
+
+int scratch_address(float** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    ll::set_error("ll_nvfp4_quantize_noalloc: hipGetDevice failed: %s", hipGetErrorString(e));
+    return LL_ELAUNCH;
+  }
+  if (dev < 0 || dev >= kMaxDevices) {
+    ll::set_error("ll_nvfp4_quantize_noalloc: device ordinal %d not supported (at most %d devices)", dev, kMaxDevices);
+    return LL_ENOSUP;
+  }
+  float* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    void* addr = nullptr;
+    e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !addr) {
+      ll::set_error("ll_nvfp4_quantize_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+      return LL_ELAUNCH;
+    }
+    p = static_cast<float*>(addr);
+    g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing threads store the same address
+  }
+  *out = p;
+  return LL_OK;
+}
+}  // namespace
+
+extern "C" int64_t ll_nvfp4_quantize_noalloc_max_elements(void) { return LL_NOALLOC_MAX_ELEMENTS; }
+
+extern "C" int ll_nvfp4_quantize_noalloc(const void* x, int64_t M, int64_t K, int64_t ldx, int rule, uint8_t* values,
+                                         uint8_t* scales, float* amax, void* stream) {
+  using namespace ll;
+  LL_REQUIRE(M > 0 && K > 0, "ll_nvfp4_quantize_noalloc: bad shape M=%lld K=%lld", (long long)M, (long long)K);
+  LL_REQUIRE(K <= LL_NOALLOC_MAX_ELEMENTS && M <= LL_NOALLOC_MAX_ELEMENTS / K,
+             "ll_nvfp4_quantize_noalloc: %lld x %lld elements exceed the limit of %lld of this entry point; use "
+             "ll_nvfp4_quantize with a caller-provided workspace",
+             (long long)M, (long long)K, (long long)LL_NOALLOC_MAX_ELEMENTS);
+  float* ws = nullptr;
+  if (int rc = scratch_address(&ws)) return rc;
+  return quantize_impl(x, M, K, ldx, rule, values, scales, amax, 0, ws, nullptr, stream);
+}

@@ -42,6 +42,15 @@ def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
     assert ctypes.sizeof(_native.GemmEpilogue) == 72 and ctypes.sizeof(_native.AmaxSinkStruct) == 16
 
 
+def test_noalloc_quantize_refuses_inputs_beyond_its_limit_before_touching_the_gpu():
+    lib = _native.load()
+    limit = lib.ll_nvfp4_quantize_noalloc_max_elements()
+    assert limit == 1 << 32
+    assert lib.ll_nvfp4_quantize_noalloc(None, limit // 64 + 1, 64, 64, 3, None, None, None, None) == -1
+    assert b"exceed the limit" in lib.ll_last_error()
+    assert lib.ll_nvfp4_quantize_noalloc(None, 0, 64, 64, 3, None, None, None, None) == -1
+
+
 def test_scale_rule_tables():
     assert [ScaleRule(r).cuda_id() for r in ("static_6", "static_4", "mae", "mse", "abs_max")] == [0, 1, 2, 3, 4]
     assert ScaleRule.mse.max_allowed_e4m3_value() == 256 and ScaleRule.static_4.max_allowed_e2m1_value() == 4
