@@ -55,3 +55,35 @@ def hardware_convert(x: torch.Tensor, mode: int) -> torch.Tensor:
     if code != 0:
         raise RuntimeError(f"ll_test_convert failed with {code}")
     return out
+
+
+def block_oracle_params(block) -> dict:
+    """Parameters of a (quantized) DiTBlock in the form oracle/dit_oracle.block_forward takes."""
+    f = lambda t: t.detach().float().cpu().numpy()
+    p = {"modulation": f(block.modulation)[0]}
+    for name in ("self_attn.q", "self_attn.k", "self_attn.v", "self_attn.o", "cross_attn.q", "cross_attn.k",
+                 "cross_attn.v", "cross_attn.o", "ffn.0", "ffn.2"):
+        lin = block.get_submodule(name)
+        qw = lin.quantized_weight()
+        p[name + ".w"] = dict(values=u8(qw.values), scales=u8(qw.scale_factors), amax=np.float32(qw.amax.item()),
+                              rule=qw.scale_rule.value, padded=tuple(qw.padded_shape), orig=tuple(qw.original_shape))
+        p[name + ".b"] = f(lin.bias)
+    for name in ("self_attn.norm_q", "self_attn.norm_k", "cross_attn.norm_q", "cross_attn.norm_k"):
+        p[name] = f(block.get_submodule(name).weight)
+    p["norm3.w"], p["norm3.b"] = f(block.norm3.weight), f(block.norm3.bias)
+    return p
+
+
+def generator_oracle_params(model) -> dict:
+    """Parameters of a quantized CausalDiT in the form oracle/generator_oracle takes: bf16 CPU tensors for the
+    embeddings and the head, block_oracle_params per block."""
+    c = lambda t: t.detach().cpu().bfloat16()
+    P = {"patch_embedding.weight": c(model.patch_embedding.weight), "patch_embedding.bias": c(model.patch_embedding.bias),
+         "head.modulation": c(model.head.modulation), "head.head.weight": c(model.head.head.weight),
+         "head.head.bias": c(model.head.head.bias)}
+    for name, seq, idx in (("time_embedding", model.time_embedding, (0, 2)), ("text_embedding", model.text_embedding, (0, 2)),
+                           ("time_projection", model.time_projection, (1,))):
+        for i in idx:
+            P[f"{name}.{i}.weight"], P[f"{name}.{i}.bias"] = c(seq[i].weight), c(seq[i].bias)
+    P["blocks"] = [block_oracle_params(b) for b in model.blocks]
+    return P

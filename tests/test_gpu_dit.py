@@ -20,19 +20,7 @@ def _f(t):
     return t.detach().float().cpu().numpy()
 
 
-def _oracle_params(block):
-    p = {"modulation": _f(block.modulation)[0]}
-    for name in ("self_attn.q", "self_attn.k", "self_attn.v", "self_attn.o", "cross_attn.q", "cross_attn.k",
-                 "cross_attn.v", "cross_attn.o", "ffn.0", "ffn.2"):
-        lin = block.get_submodule(name)
-        qw = lin.quantized_weight()
-        p[name + ".w"] = dict(values=u8(qw.values), scales=u8(qw.scale_factors), amax=np.float32(qw.amax.item()),
-                              rule="mse", padded=qw.padded_shape, orig=qw.original_shape)
-        p[name + ".b"] = _f(lin.bias)
-    for name in ("self_attn.norm_q", "self_attn.norm_k", "cross_attn.norm_q", "cross_attn.norm_k"):
-        p[name] = _f(block.get_submodule(name).weight)
-    p["norm3.w"], p["norm3.b"] = _f(block.norm3.weight), _f(block.norm3.bias)
-    return p
+from helpers import block_oracle_params as _oracle_params  # noqa: E402
 
 
 def _rel(a, b):
@@ -496,3 +484,147 @@ def test_generator_with_the_unipc_sampler_follows_a_hand_stepped_scheduler(gpu):
     # bf16 latents: the generator rounds after every step, the hand-stepped copy once per step as well
     diff = (out[0, :2].transpose(0, 1).float() - x.float()).abs().max().item()
     assert diff <= 2 * 2.0 ** -7 * out.float().abs().max().item(), diff  # two bf16 ulps of the largest latent
+
+
+@pytest.mark.parametrize("time_gain,disp_tol,latent_tol", [(1.0, 4e-2, 1.5e-2), (40.0, 1e-1, 6e-2)])
+def test_streaming_generator_against_the_chunk_loop_oracle(gpu, time_gain, disp_tol, latent_tol):
+    """The generator on the GPU against the CPU restatement of the reference's chunk loop (oracle/generator_oracle.py:
+    model forward around the blocks, four Euler / flow steps at 1000/750/500/250, timestep-0 recache, cache fill and
+    roll), latent by latent.  2 layers, dim 256, 6 chunks of 2 frames (128 tokens), cache of 3 blocks with a 1-block
+    sink, so chunks 3-5 each roll the window.
+
+    Tolerance, per chunk: relative Frobenius error of the displacement (latent - noise, the integral of the
+    predicted flow) <= 4e-2 and of the latent itself <= 1.5e-2 (measured 1.5e-2 and 4.5e-3: the FP4
+    re-quantization of activations that differ in the last bf16 bit flips a few codes per forward).
+    With the random initialisation the model barely reacts to the timestep, so a second case multiplies the first
+    time-embedding weight by 40: the modulation then dominates, the errors grow with it (tolerance 1e-1 / 6e-2,
+    measured 6.4e-2 / 3.8e-2), and leaving the timestep-0 pass out of the oracle moves every later chunk by more
+    than 2e-1 (measured 2.7e-1 to 3.3e-1) -- the control that the comparison sees that pass."""
+    import generator_oracle as go
+    from helpers import generator_oracle_params
+    from longlive_amd.utils.quant import dequantize_kv_cache
+
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    gen = StreamingGenerator(cfg, gpu, seed=4)
+    with torch.no_grad():
+        gen.model.time_embedding[0].weight.mul_(time_gain)
+    g = torch.Generator().manual_seed(4)
+    noise = torch.randn(1, 12, 8, 16, 16, generator=g).bfloat16()
+    ctx = torch.randn(10, 64, generator=g).bfloat16()
+    out = gen.generate(noise.to(gpu), ctx.to(gpu)).cpu()
+    P = generator_oracle_params(gen.model)
+    ref, caches = go.generate(P, cfg, noise, ctx)
+
+    def err(a, b, c):
+        sl = slice(2 * c, 2 * c + 2)
+        a, b, n = _f(a[0, sl]), _f(b[0, sl]), _f(noise[0, sl])
+        return _rel(a - n, b - n), _rel(a, b)
+
+    for c in range(6):
+        d_err, l_err = err(out, ref, c)
+        assert d_err <= disp_tol and l_err <= latent_tol, (c, d_err, l_err)
+    if time_gain > 1:
+        control, _ = go.generate(P, cfg, noise, ctx, recache=False)
+        for c in range(1, 6):
+            assert err(control, ref, c)[0] > 2e-1, c
+    # cache state: same bookkeeping, and the slots hold what the oracle's cache holds: slot amax within 3 % (10 % in the amplified case), content
+    # within 0.2 relative Frobenius (two FP4 quantizations of inputs that differ in the last bf16 bits differ by
+    # whole e2m1 steps where a value sits next to a rounding boundary or the block's 4-or-6 choice flips; the
+    # quantization noise of NVFP4 itself is about 0.1)
+    blk = 128
+    for layer, (cache, oc) in enumerate(zip(gen.kv_cache, caches)):
+        st = oc["policy"]
+        assert (cache["_global_end"], cache["_local_end"]) == (st["global_end"], st["local_end"]) == (12 * 64, 3 * blk)
+        for name in ("k", "v"):
+            got = _f(dequantize_kv_cache(cache[name], 3, 2, blk, torch.bfloat16, gpu)[0])
+            for slot in range(3):
+                chunk = int(st["buf"][slot * blk]) // blk
+                assert _rel(got[slot * blk:(slot + 1) * blk], oc[name][chunk]) <= 0.2, (layer, name, slot)
+                assert abs(float(cache[name][slot].amax) / oc[name + "_amax"][chunk] - 1) <= max(0.03, disp_tol), (layer, name, slot)
+        assert [int(st["buf"][s * blk]) // blk for s in range(3)] == [0, 4, 5]
+
+
+def test_config5_full_size_generator_fills_and_rolls_the_window(gpu, monkeypatch):
+    """Benchmark configuration 5 at full size (30 blocks, dim 3072, 24 heads, FFN 14336, chunks of 3 latent frames
+    = 2640 tokens, FP4 cache of 5 blocks = sink 3 + window 12 frames, timesteps 1000/750/500/250 + the timestep-0
+    recache pass), run for 6 chunks: five fill the cache, the sixth rolls it.  The CPU oracle of the whole loop is
+    out of reach at this size (184 TFLOP per chunk), so the checks are: finite, non-trivial latents; per-layer cache
+    bookkeeping equal to the token-level policy oracle's; every slot of layer 0 holding, bit for bit, the bytes
+    written for the chunk the policy oracle places there; and the newest slot's bytes equal to the CPU oracle's
+    quantization of the rotated K (and of V) the model produced for that chunk in its recache pass."""
+    import cache_policy_oracle as cpo
+    from longlive_amd.dit import model as dit_model
+
+    cfg = DiTConfig()
+    gen = StreamingGenerator(cfg, gpu, seed=4)
+    g = torch.Generator().manual_seed(4)
+    n_chunks, fs, blk = 6, 880, 2640
+    noise = torch.randn(1, 3 * n_chunks, 48, 44, 80, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(512, 4096, generator=g).bfloat16().to(gpu)
+
+    written = {}          # chunk -> (K bytes, V bytes, K amax) of layer 0 right after the chunk's recache pass
+    produced = {}         # chunk -> (rotated K, V) bf16 handed to the cache update of layer 0
+    real_update = kvc.apply_cache_update
+
+    def recording_update(cache, current_end, local_end_index, info, kv_cfg):
+        real_update(cache, current_end, local_end_index, info, kv_cfg)
+        if cache is gen.kv_cache[0] and info is not None:
+            chunk = current_end // blk - 1
+            slot = info["local_start_index"] // blk
+            written[chunk] = (cache["k"][slot].values.clone(), cache["v"][slot].values.clone(),
+                              cache["k"][slot].scale_factors.clone(), float(cache["k"][slot].amax))
+            produced[chunk] = (info["new_k"], info["new_v"])
+
+    monkeypatch.setattr(dit_model.kvc, "apply_cache_update", recording_update)
+    out = gen.generate(noise, ctx)
+    assert out.shape == noise.shape and torch.isfinite(out.float()).all()
+    moved = (out.float() - noise.float()).norm() / noise.float().norm()
+    assert 0.01 < float(moved) < 10.0
+    assert sorted(written) == list(range(n_chunks))
+
+    # policy oracle: five forwards per chunk, each applying its update, as the reference does
+    st = cpo.new_state(5 * blk)
+    for c in range(n_chunks):
+        for _ in range(5):
+            ids, upd = cpo.attend(st, c * blk, blk, cfg.sink_size * fs, 0, cfg.local_attn_size * fs)
+            cpo.apply(st, upd)
+    holds = [int(st["buf"][s * blk]) // blk for s in range(5)]
+    assert holds == [0, 2, 3, 4, 5]
+    for cache in gen.kv_cache:
+        assert (cache["_global_end"], cache["_local_end"]) == (st["global_end"], st["local_end"])
+        assert int(cache["global_end_index"]) == st["global_end"] and int(cache["local_end_index"]) == st["local_end"]
+    c0 = gen.kv_cache[0]
+    for slot, chunk in enumerate(holds):
+        kb, vb, ksb, kam = written[chunk]
+        assert torch.equal(c0["k"][slot].values, kb) and torch.equal(c0["v"][slot].values, vb), (slot, chunk)
+        assert torch.equal(c0["k"][slot].scale_factors.view(torch.uint8), ksb.view(torch.uint8))
+        assert float(c0["k"][slot].amax) == kam == float(produced[chunk][0].float().abs().max())
+    # newest slot against the CPU oracle's quantization of what the model produced
+    for name, t in zip(("k", "v"), produced[n_chunks - 1]):
+        vals, sc, am, _ = o.quantize_to_fp4(bits_of(t[0].reshape(-1, 128)), "mse")
+        slot = c0[name][4]
+        assert float(slot.amax) == float(am)
+        assert np.array_equal(u8(slot.scale_factors), sc) and np.array_equal(u8(slot.values), vals), name
+
+
+@pytest.mark.parametrize("clean", [False, True])
+def test_skipping_dead_cache_writes_is_invisible_in_multi_shot_mode(gpu, clean):
+    """Leaving out the cache writes of the denoising forwards (which the timestep-0 pass overwrites) must not
+    change a bit of the latents or of the final cache in multi-shot mode either: global sink, scene cuts at
+    chunks 2 and 5 (pinned chunks that float to the front while the window rolls), with and without the clean
+    recache."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=8, sink_size=2)
+    g = torch.Generator().manual_seed(12)
+    noise = torch.randn(1, 16, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    gens = [StreamingGenerator(cfg, gpu, seed=4, multi_shot_sink=True, shot_clean_recache=clean,
+                               skip_dead_cache_writes=skip) for skip in (True, False)]
+    a, b = (gen.generate(noise, ctx, scene_cuts=(2, 5)) for gen in gens)
+    assert torch.equal(a, b)
+    for la, lb in zip(gens[0].kv_cache, gens[1].kv_cache):
+        for key in ("_global_end", "_local_end", "_pinned_start", "_pinned_len"):
+            assert la[key] == lb[key], key
+        for sa, sb in zip(la["k"] + la["v"], lb["k"] + lb["v"]):
+            assert torch.equal(sa.values, sb.values) and torch.equal(sa.amax, sb.amax)
