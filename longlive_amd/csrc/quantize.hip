@@ -130,18 +130,16 @@ __device__ __forceinline__ float candidate_error(const float (&X)[16], const Can
 }
 
 // Quantize one block of 16 values; returns the 8 packed bytes (lo, hi) and the scale byte.
+// enc = (E2 * E4) / amax and dec = 1 / enc do not depend on the block; the kernel forms them once.
 template <int RULE>
-__device__ __forceinline__ void quantize_block(const float (&X)[16], float amax, uint32_t& lo, uint32_t& hi,
-                                               uint32_t& scale_byte) {
+__device__ __forceinline__ void quantize_block(const float (&X)[16], float amax, float enc, float dec, uint32_t& lo,
+                                               uint32_t& hi, uint32_t& scale_byte) {
   constexpr bool kStatic = (RULE == LL_RULE_STATIC_6 || RULE == LL_RULE_STATIC_4);
   constexpr float E2 = (RULE == LL_RULE_STATIC_4) ? 4.0f : 6.0f;
-  constexpr float E4 = kStatic ? 448.0f : 256.0f;
   float bmax = fabsf(X[0]);
 #pragma unroll
   for (int i = 1; i < 16; ++i) bmax = fmaxf(bmax, fabsf(X[i]));
-  const float enc = (E2 * E4) / amax;
   const float hp = (amax == 0.0f) ? 0.0f : (bmax / E2) * enc;
-  const float dec = 1.0f / enc;
 
   Candidate c6;
   make_candidate(X, hp, dec, c6);
@@ -181,7 +179,7 @@ __device__ __forceinline__ void quantize_block(const float (&X)[16], float amax,
 //  * bmax / 6 = fma(fma(-6, q0, bmax), 1/6, q0) with q0 = bmax * (1/6) is the correctly rounded
 //    quotient for every fp32 bmax (verified exhaustively on the CPU).
 struct ScaleEntry {
-  float r, d1, d3, pad;
+  float r, d1, d3, w;  // w = d1 * d1
 };
 
 typedef float float2v __attribute__((ext_vector_type(2)));
@@ -271,38 +269,45 @@ __device__ __forceinline__ float exact_error(const float (&X)[16], const ScaleEn
 }
 
 // Four-over-six choice.  The reference compares the two candidates' errors as it computes them in fp32
-// (exact_error).  The estimates of encode_candidate, multiplied by the candidate's step d1 (squared for
-// mse), are the same quantities up to rounding: y carries at most 5 roundings (|y| < 7), the reference's
-// dequantized value 2, its difference, square and 16-term sum a few more.  With u = 2^-24 each estimate E = a w
-// (a in step units, w = d1 or d1^2) and the reference's value both lie within
-//     mse: (320 u sqrt(a) + 32 u a) w     mae: (640 u + 32 u a) w     abs_max: (40 u + 8 u a) w
-// of the exact real-number error, plus 8 u E for the rounding of d1 itself.  When the two estimates differ by
-// more than four times the sum of these bounds the reference's comparison has the same outcome; otherwise
-// (a few blocks in 10^4 of Gaussian data) the block is decided by exact_error.  `approx_ok` is false when the tensor amax is so
-// small or large that squares could leave the normal fp32 range; then every block is decided by exact_error.
+// (exact_error).  The estimates of encode_candidate, multiplied by the candidate's weight w (the step d1 of the
+// candidate, squared for mse), are the same quantities up to rounding.  With u = 2^-24, D the real-number step
+// s * amax / 1536 and a* = sum (q - x / D)^2 the real-number error in step units:
+//   * y = fl(x * r) carries five roundings (1536 / amax, its reciprocal, the product with s, the reciprocal of
+//     that, the product with x) and |y| < 7, so |y - x / D| <= 35 u and the estimate a = sum (q - y)^2, 17 more
+//     roundings of its own, lies within 2 * 35 u * sum |q - x / D| + 18 u a* <= 280 u sqrt(a*) + 18 u a* of a*
+//     (Cauchy-Schwarz over the 16 terms);
+//   * the reference's dequantized value q D (1 + 2u) (q * s is exact, two roundings follow) gives errors
+//     D (q - x / D + q eps) with |q eps| <= 12 u, so its sum of squares, 18 more roundings, lies within
+//     D^2 (96 u sqrt(a*) + 19 u a*) of D^2 a*;
+//   * w = fl(d1 * d1) = D^2 (1 + 5u) and E = fl(a * w) add 6 u E.
+// Hence both E and the reference's value lie within B = (320 u sqrt(a) + 32 u a) w + 8 u E of the real-number
+// error D^2 a*, and when |E4 - E6| exceeds 2 (B4 + B6) the reference's comparison has the same outcome.  The
+// kernel asks for twice that and bounds the square root by 2 sqrt(a) <= 1 + a, which gives the margin
+//     mse: 640 u (w4 + w6) + 800 u (E4 + E6)
+// (mae, whose terms are |q - y| instead of squares: B = (640 u + 32 u a) w + 8 u E, the same derivation with
+// sum |.| <= 16 * 35 u in place of the Cauchy-Schwarz step).  Blocks inside the margin (a few in 10^4 of
+// Gaussian data) are decided by exact_error.  `approx_ok` is false when the tensor amax is so small or large
+// that squares could leave the normal fp32 range; then every block is decided by exact_error.
 template <int RULE>
 __device__ __forceinline__ bool pick_four(const float (&X)[16], const ScaleEntry& e6, const ScaleEntry& e4, float a6,
                                           float a4, uint32_t lo6, uint32_t hi6, uint32_t lo4, uint32_t hi4,
                                           bool approx_ok) {
   constexpr float u = 0x1p-24f;
-  const float w6 = (RULE == LL_RULE_MSE) ? e6.d1 * e6.d1 : e6.d1;
-  const float w4 = (RULE == LL_RULE_MSE) ? e4.d1 * e4.d1 : e4.d1;
-  const float E6 = a6 * w6, E4 = a4 * w4;
-  float b6, b4;
-  if (RULE == LL_RULE_MSE) {
-    b6 = 320.0f * u * __builtin_sqrtf(a6) + 32.0f * u * a6;
-    b4 = 320.0f * u * __builtin_sqrtf(a4) + 32.0f * u * a4;
-  } else if (RULE == LL_RULE_MAE) {
-    b6 = 640.0f * u + 32.0f * u * a6;
-    b4 = 640.0f * u + 32.0f * u * a4;
-  } else {
-    b6 = 40.0f * u + 8.0f * u * a6;
-    b4 = 40.0f * u + 8.0f * u * a4;
-  }
-  const float margin = 4.0f * (b6 * w6 + b4 * w4 + 8.0f * u * (E6 + E4)) + 0x1p-100f;
   // abs_max compares two maxima over values that sit on a coarse grid (bf16 inputs): exact ties are common
   // (a few percent of the blocks), so that rule always takes the reference's arithmetic.
-  if (RULE != LL_RULE_ABS_MAX && approx_ok && fabsf(E4 - E6) > margin) return E4 < E6;
+  if (RULE != LL_RULE_ABS_MAX) {
+    const float w6 = (RULE == LL_RULE_MSE) ? e6.w : e6.d1;
+    const float w4 = (RULE == LL_RULE_MSE) ? e4.w : e4.d1;
+    const float E6 = a6 * w6, E4 = a4 * w4;
+    float margin;
+    if (RULE == LL_RULE_MSE) {
+      margin = __builtin_fmaf(800.0f * u, E6 + E4, (640.0f * u) * (w6 + w4)) + 0x1p-100f;
+    } else {
+      const float b6 = 640.0f * u + 32.0f * u * a6, b4 = 640.0f * u + 32.0f * u * a4;
+      margin = 4.0f * (b6 * w6 + b4 * w4 + 8.0f * u * (E6 + E4)) + 0x1p-100f;
+    }
+    if (approx_ok && fabsf(E4 - E6) > margin) return E4 < E6;
+  }
   return exact_error<RULE>(X, e4, lo4, hi4) < exact_error<RULE>(X, e6, lo6, hi6);
 }
 
@@ -351,7 +356,10 @@ __device__ __forceinline__ bool quantize_block_fast(const float (&X)[16], float 
 // ----------------------------------------------------------------------------- quantize kernel
 // One workgroup = a 128-row x 64-column tile = 512 blocks of 16 = one 512-byte tile of the blocked
 // scale layout, which is staged in LDS and written with coalesced 4-byte stores.
-template <int RULE>
+// GENERIC = false: x is 16-byte aligned with ldx a multiple of 8 and K a multiple of 64, so every block is two
+// whole 16-byte pieces and only rows beyond M need care (zeros).  GENERIC = true handles any K, ldx and
+// alignment element by element at the edges.
+template <int RULE, bool GENERIC>
 __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
                                                             int64_t ldx, int64_t Kp, uint8_t* __restrict__ values,
                                                             uint8_t* __restrict__ scales, float* __restrict__ amax_io,
@@ -360,14 +368,17 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
                                                             const unsigned long long* __restrict__ sink_parts,
                                                             uint32_t sink_epoch) {
   __shared__ float s_red[kThreads / 64];
-  __shared__ float s_amax;
-  __shared__ uint32_t s_scales[128];  // 512 bytes in blocked order
+  __shared__ uint32_t s_scales[2][128];  // two staged 512-byte scale tiles in blocked order
   __shared__ ScaleEntry s_tab[128];
+  static_assert(kThreads == 256 && kAmaxParts == 4 * kThreads, "four waves, four partial maxima per thread");
 
+  // ---- tensor amax: given, or the maximum of the kAmaxParts partial maxima (every wave folds its share, the four
+  // wave results meet in LDS and every thread folds those itself: one barrier)
+  float amax;
   if (amax_given) {
-    if (threadIdx.x == 0) s_amax = amax_io[0];
+    amax = amax_io[0];
   } else {
-    float4 p;  // kAmaxParts == 4 * kThreads
+    float4 p;
     if (sink_parts) {
       p = make_float4(amax_sink_read(sink_parts, sink_epoch, 4 * threadIdx.x),
                       amax_sink_read(sink_parts, sink_epoch, 4 * threadIdx.x + 1),
@@ -376,18 +387,12 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
     } else {
       p = reinterpret_cast<const float4*>(parts)[threadIdx.x];
     }
-    float m = wave_max(fmaxf(fmaxf(p.x, p.y), fmaxf(p.z, p.w)));
+    const float m = wave_max(fmaxf(fmaxf(p.x, p.y), fmaxf(p.z, p.w)));
     if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = m;
     __syncthreads();
-    if (threadIdx.x == 0) {
-      float r = s_red[0];
-      for (int i = 1; i < kThreads / 64; ++i) r = fmaxf(r, s_red[i]);
-      s_amax = r;
-      if (blockIdx.x == 0) amax_io[0] = r;
-    }
+    amax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    if (blockIdx.x == 0 && threadIdx.x == 0) amax_io[0] = amax;
   }
-  __syncthreads();
-  const float amax = s_amax;
 
   // The fast path needs amax to be the true maximum (so block scales stay within e4m3 range) and far
   // from the ends of the fp32 range (so powers of two scale exactly); otherwise every block takes the
@@ -398,20 +403,22 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
   const bool fast = !amax_given && amax >= 0x1p-100f && amax <= 0x1p100f;
   const bool approx_ok = amax >= 0x1p-30f && amax <= 0x1p30f;  // squares of errors stay normal fp32 numbers
   const float enc = (kE2 * kE4) / amax;
-  if (fast && threadIdx.x < 128) {
-    const float dec = 1.0f / enc;
-    const float sf = e4m3_to_f32(threadIdx.x);
-    ScaleEntry e;
-    e.r = (threadIdx.x == 0 || threadIdx.x == 127) ? 0.0f : 1.0f / (dec * sf);
-    e.d1 = (sf * amax) / 1536.0f;
-    e.d3 = ((1.5f * sf) * amax) / 1536.0f;
-    e.pad = 0.0f;
-    s_tab[threadIdx.x] = e;
+  const float dec = 1.0f / enc;
+  if (fast) {  // table entry threadIdx.x % 128: the lower half of the workgroup fills r, d1 and w, the upper half d3
+    const uint32_t idx = threadIdx.x & 127;
+    const float sf = e4m3_to_f32(idx);
+    if (threadIdx.x < 128) {
+      const float d1 = (sf * amax) / 1536.0f;
+      s_tab[idx].r = (idx == 0 || idx == 127) ? 0.0f : 1.0f / (dec * sf);
+      s_tab[idx].d1 = d1;
+      s_tab[idx].w = d1 * d1;
+    } else if (!kStaticRule) {
+      s_tab[idx].d3 = ((1.5f * sf) * amax) / 1536.0f;
+    }
   }
   __syncthreads();
 
   const bool vec = ((ldx & 7) == 0) && ((reinterpret_cast<uintptr_t>(x) & 15) == 0);
-  uint8_t* s_bytes = reinterpret_cast<uint8_t*>(s_scales);
   const uint32_t tiles_x = (uint32_t)(Kp >> 6);
 
   // Tiles are dealt to the resident workgroups round-robin, so the prologue above (amax reduction,
@@ -420,49 +427,140 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
   // the lines are consecutive in tile order.  Consecutive workgroup ids are dealt round-robin to the 8 XCDs,
   // each with an L2 of its own, so the four tiles go to workgroups v, v + 8, v + 16, v + 24, which start on
   // the same XCD at about the same time and let that L2 merge the partial lines before they are written back.
-  // (The grid is a multiple of 32 workgroups; v runs over all of them in every round.)
-  const uint32_t n_tiles = (uint32_t)total_tiles;  // 32-bit: cheap division
-#pragma unroll 1
-  for (uint32_t v = blockIdx.x; v < ((n_tiles + 31u) & ~31u); v += gridDim.x) {
-  const uint32_t tile = ((v >> 5) * 8u + (v & 7u)) * 4u + ((v >> 3) & 3u);
-  if (tile >= n_tiles) continue;  // uniform over the workgroup
-  const uint32_t tile_y = tile / tiles_x;
-  const int64_t row0 = (int64_t)tile_y * 128;
-  const int64_t col0 = (int64_t)(tile - tile_y * tiles_x) * 64;
-#pragma unroll 1
-  for (int it = 0; it < 2; ++it) {
-    const int b = threadIdx.x + it * kThreads;  // block within the tile
-    const int r = b >> 2, cb = b & 3;
-    const int64_t row = row0 + r, col = col0 + cb * 16;
-    float X[16];
-    if (row < M && col + 16 <= K && vec) {
-      const uint4* p = reinterpret_cast<const uint4*>(x + row * ldx + col);
-      const uint4 v0 = p[0], v1 = p[1];
-      const uint32_t w[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        X[2 * i] = __uint_as_float(w[i] << 16);
-        X[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
+  // The grid is a multiple of 32 workgroups, so a workgroup's next tile is its current one plus the grid size:
+  // the tile's row and column advance by constants, and no division is left in the loop.
+  const uint32_t n_tiles = (uint32_t)total_tiles;
+  const uint32_t grid = gridDim.x, wg = blockIdx.x;
+  const uint32_t first_tile = ((wg >> 5) * 8u + (wg & 7u)) * 4u + ((wg >> 3) & 3u);
+  const uint32_t step_y = grid / tiles_x, step_x = grid - step_y * tiles_x;
+
+  // The thread's two blocks of a tile: block b = threadIdx.x + it * kThreads, row b / 4, column block b % 4.
+  const int r0 = threadIdx.x >> 2, cb = threadIdx.x & 3;
+  const int64_t vrow = Kp >> 1;                                   // bytes per row of packed values
+  const int64_t thread_x = (int64_t)r0 * ldx + cb * 16;           // elements, from the tile's first element
+  const int64_t thread_v = (int64_t)r0 * vrow + cb * 8;           // bytes, from the tile's first packed byte
+  const int s_off0 = (r0 & 31) * 16 + (r0 >> 5) * 4 + cb;         // staged scale byte of the block of it = 0; it = 1: + 8
+  // The 32 bytes of one block as they lie in memory (16 bf16 values); blocks that stick out of the tensor are
+  // completed with zeros, like the reference's zero padding.
+  struct Raw {
+    uint4 lo, hi;
+  };
+  struct Tile {
+    uint32_t index, ty, tx;
+  };
+  auto load_block = [&](const Tile& t, int it, Raw& raw) {
+    const int64_t row0 = (int64_t)t.ty * 128, col0 = (int64_t)t.tx * 64;
+    if (!GENERIC || (vec && col0 + 64 <= K)) {  // whole 16-byte pieces; rows beyond M are zeros
+      if (row0 + r0 + it * 64 < M) {
+        const uint4* p = reinterpret_cast<const uint4*>(x + (row0 * ldx + col0) + thread_x + (int64_t)it * 64 * ldx);
+        raw.lo = p[0];
+        raw.hi = p[1];
+      } else {
+        raw.lo = raw.hi = make_uint4(0u, 0u, 0u, 0u);
       }
     } else {
+      const int64_t row = row0 + r0 + it * 64, col = col0 + cb * 16;
+      uint32_t w[8];
 #pragma unroll
-      for (int i = 0; i < 16; ++i)
-        X[i] = (row < M && col + i < K) ? bf16_bits_to_f32(x[row * ldx + col + i]) : 0.0f;
+      for (int i = 0; i < 8; ++i) {
+        const uint32_t e0 = (row < M && col + 2 * i < K) ? x[row * ldx + col + 2 * i] : 0u;
+        const uint32_t e1 = (row < M && col + 2 * i + 1 < K) ? x[row * ldx + col + 2 * i + 1] : 0u;
+        w[i] = e0 | (e1 << 16);
+      }
+      raw.lo = make_uint4(w[0], w[1], w[2], w[3]);
+      raw.hi = make_uint4(w[4], w[5], w[6], w[7]);
+    }
+  };
+  // Quantize one block and store its 8 packed bytes; the scale byte goes to the staged 128x4 scale tile.
+  auto quantize_store = [&](const Tile& t, int it, const Raw& raw, uint8_t* s_bytes) {
+    const uint32_t w[8] = {raw.lo.x, raw.lo.y, raw.lo.z, raw.lo.w, raw.hi.x, raw.hi.y, raw.hi.z, raw.hi.w};
+    float X[16];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      X[2 * i] = __uint_as_float(w[i] << 16);
+      X[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
     }
     uint32_t lo, hi, sb;
-    if (!fast || !quantize_block_fast<RULE>(X, enc, s_tab, approx_ok, lo, hi, sb)) quantize_block<RULE>(X, amax, lo, hi, sb);
-    *reinterpret_cast<uint2*>(values + row * (Kp >> 1) + (col >> 1)) = make_uint2(lo, hi);
-    s_bytes[(r & 31) * 16 + (r >> 5) * 4 + cb] = (uint8_t)sb;
-  }
-  __syncthreads();
-  if (threadIdx.x < 128) reinterpret_cast<uint32_t*>(scales)[(int64_t)tile * 128 + threadIdx.x] = s_scales[threadIdx.x];
-  __syncthreads();  // the staged scale tile is rewritten by the next tile
+    if (!fast || !quantize_block_fast<RULE>(X, enc, s_tab, approx_ok, lo, hi, sb)) quantize_block<RULE>(X, amax, enc, dec, lo, hi, sb);
+    uint8_t* dst = values + ((int64_t)t.ty * 128 * vrow + (int64_t)t.tx * 32) + thread_v + (int64_t)it * 64 * vrow;
+    *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
+    s_bytes[s_off0 + it * 8] = (uint8_t)sb;
+  };
+  auto advance = [&](Tile& t) {
+    t.index += grid;
+    t.ty += step_y;
+    t.tx += step_x;
+    if (t.tx >= tiles_x) {
+      t.tx -= tiles_x;
+      ++t.ty;
+    }
+  };
+
+  // One barrier per tile: the staged scale tile is double-buffered.
+  Tile cur;
+  cur.index = first_tile;
+  cur.ty = first_tile / tiles_x;
+  cur.tx = first_tile - cur.ty * tiles_x;
+  int parity = 0;
+#pragma unroll 1
+  while (cur.index < n_tiles) {
+    uint8_t* s_bytes = reinterpret_cast<uint8_t*>(s_scales[parity]);
+#pragma unroll 1
+    for (int it = 0; it < 2; ++it) {
+      Raw raw;
+      load_block(cur, it, raw);
+      quantize_store(cur, it, raw, s_bytes);
+    }
+    __syncthreads();
+    if (threadIdx.x < 128)
+      reinterpret_cast<uint32_t*>(scales)[(int64_t)cur.index * 128 + threadIdx.x] = s_scales[parity][threadIdx.x];
+    parity ^= 1;  // the next tile stages into the other buffer; this one is rewritten two barriers from now
+    advance(cur);
   }
 }
 
 }  // namespace ll
 
 extern "C" size_t ll_nvfp4_quantize_workspace_floats(void) { return ll::kAmaxParts; }
+
+// Workgroups of quantize_kernel<rule, generic> that fit on the current device at once (occupancy per CU from the
+// runtime, times the CU count), looked up once per device and kernel.
+static int resident_workgroups(int rule, bool generic, int64_t* out) {
+  using namespace ll;
+  static std::atomic<int> cache[64][5][2];
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    set_error("ll_nvfp4_quantize: hipGetDevice failed: %s", hipGetErrorString(e));
+    return LL_ELAUNCH;
+  }
+  std::atomic<int>* slot = (dev >= 0 && dev < 64) ? &cache[dev][rule][generic ? 1 : 0] : nullptr;
+  int n = slot ? slot->load(std::memory_order_relaxed) : 0;
+  if (n == 0) {
+    int per_cu = 0, cus = 0;
+#define LL_OCC(R)                                                                                                        \
+  e = generic ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, quantize_kernel<R, true>, kThreads, 0)            \
+              : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, quantize_kernel<R, false>, kThreads, 0)
+    switch (rule) {
+      case LL_RULE_STATIC_6: LL_OCC(LL_RULE_STATIC_6); break;
+      case LL_RULE_STATIC_4: LL_OCC(LL_RULE_STATIC_4); break;
+      case LL_RULE_MAE: LL_OCC(LL_RULE_MAE); break;
+      case LL_RULE_MSE: LL_OCC(LL_RULE_MSE); break;
+      default: LL_OCC(LL_RULE_ABS_MAX); break;
+    }
+#undef LL_OCC
+    if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+    if (e != hipSuccess || per_cu <= 0 || cus <= 0) {
+      set_error("ll_nvfp4_quantize: occupancy query failed: %s", hipGetErrorString(e));
+      return LL_ELAUNCH;
+    }
+    n = per_cu * cus;
+    if (n < 32) n = 32;
+    if (slot) slot->store(n, std::memory_order_relaxed);
+  }
+  *out = n;
+  return LL_OK;
+}
 
 static int quantize_impl(const void* x, int64_t M, int64_t K, int64_t ldx, int rule, uint8_t* values, uint8_t* scales,
                          float* amax, int amax_given, float* workspace, const ll_amax_sink* sink, void* stream) {
@@ -487,14 +585,23 @@ static int quantize_impl(const void* x, int64_t M, int64_t K, int64_t ldx, int r
   }
   const unsigned long long* sink_parts = sink ? reinterpret_cast<const unsigned long long*>(sink->parts) : nullptr;
   const uint32_t sink_epoch = sink ? sink->epoch : 0u;
-  // one workgroup per tile up to what the chip holds at once (256 CUs x 8 for the static rules,
-  // x 4 for the rules that evaluate two candidates and need twice the registers)
-  const int64_t resident = (rule == LL_RULE_STATIC_6 || rule == LL_RULE_STATIC_4) ? 2048 : 1024;
+  const bool generic = (K % 64) != 0 || (ldx % 8) != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0;
+  // One workgroup per tile up to what the chip holds at once (the launch is persistent: every workgroup has to be
+  // resident from the start, or the ones that wait would run after the others have finished).
+  int64_t resident = 0;
+  if (int rc = resident_workgroups(rule, generic, &resident)) return rc;
   const int64_t padded_tiles = (total_tiles + 31) & ~(int64_t)31;  // whole groups of 32 for the XCD-aware tile order
-  const dim3 grid((unsigned)(padded_tiles < resident ? padded_tiles : resident));
-#define LL_LAUNCH_Q(R)                                                                                          \
-  hipLaunchKernelGGL(quantize_kernel<R>, grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales, amax, \
-                     workspace, amax_given, total_tiles, sink_parts, sink_epoch)
+  const int64_t resident32 = resident & ~(int64_t)31;
+  const dim3 grid((unsigned)(padded_tiles < resident32 ? padded_tiles : resident32));
+#define LL_LAUNCH_Q(R)                                                                                                  \
+  do {                                                                                                                  \
+    if (generic)                                                                                                        \
+      hipLaunchKernelGGL((quantize_kernel<R, true>), grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales,    \
+                         amax, workspace, amax_given, total_tiles, sink_parts, sink_epoch);                            \
+    else                                                                                                                \
+      hipLaunchKernelGGL((quantize_kernel<R, false>), grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales,   \
+                         amax, workspace, amax_given, total_tiles, sink_parts, sink_epoch);                            \
+  } while (0)
   switch (rule) {
     case LL_RULE_STATIC_6: LL_LAUNCH_Q(LL_RULE_STATIC_6); break;
     case LL_RULE_STATIC_4: LL_LAUNCH_Q(LL_RULE_STATIC_4); break;

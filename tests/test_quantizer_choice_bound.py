@@ -31,14 +31,17 @@ def _estimates(X, amax, rule):
         d1 = ((sf * amax) / F32(1536)).astype(F32)
         w = (d1 * d1).astype(F32) if rule == "mse" else d1
         if rule == "mse":
-            b = F32(320) * U * np.sqrt(a) + F32(32) * U * a
+            b = None  # the mse margin is formed from the sums below
         elif rule == "mae":
             b = F32(640) * U + F32(32) * U * a
         else:
             b = F32(40) * U + F32(8) * U * a
-        out.append((a * w, b * w, sb, q, sf))
-    (E6, B6, sb6, q6, sf6), (E4, B4, sb4, q4, sf4) = out
-    margin = F32(4) * (B6 + B4 + F32(8) * U * (E6 + E4)) + F32(2.0 ** -100)
+        out.append(((a * w).astype(F32), None if b is None else b * w, sb, q, sf, w))
+    (E6, B6, sb6, q6, sf6, w6), (E4, B4, sb4, q4, sf4, w4) = out
+    if rule == "mse":  # quantize.hip, pick_four: 640 u (w4 + w6) + 800 u (E4 + E6)
+        margin = ((F32(800) * U) * (E6 + E4) + (F32(640) * U) * (w6 + w4)).astype(F32) + F32(2.0 ** -100)
+    else:
+        margin = F32(4) * (B6 + B4 + F32(8) * U * (E6 + E4)) + F32(2.0 ** -100)
     same = sb4 == sb6  # identical candidates: the kernel keeps "6" without looking at errors
     sure = ((np.abs(E4 - E6) > margin) & (sb6 != 0)) | same
     # the oracle's own comparison (reference.py:175-239 as restated in quantize_blocks)
