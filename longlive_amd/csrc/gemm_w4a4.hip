@@ -315,26 +315,73 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
       }
       if (wave_has_output) mma(o[1]);
     } else {
-      // The large tiles need all registers for accumulators and fragments; there two workgroups share a CU and
-      // the hardware overlaps one wave's decode (VALU) with another wave's MFMAs.
+      // Large tiles (8 fragments pairs per wave): the same software pipeline, with the packed dwords read from LDS
+      // one sub-step ahead instead of a whole K step at a time, which is what lets it fit 256 registers.
+      struct Raw {
+        uint32_t a[FA], b[FB];
+      };
+      struct Scales {
+        half2v a[FA][2], b[FB][2];
+      };
+      auto read_scales = [&](Scales& sc, int stage, int cc) {
+        const uint8_t* base = smem + stage * S::kStage;
+#pragma unroll
+        for (int f = 0; f < FA; ++f) {
+          const uint32_t sb = *reinterpret_cast<const uint16_t*>(base + a_soff[f] + 512 * cc);
+          const half2v v = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(sb, 1.0f, false);
+          sc.a[f][0] = half2v{v[0], v[0]};
+          sc.a[f][1] = half2v{v[1], v[1]};
+        }
+#pragma unroll
+        for (int g = 0; g < FB; ++g) {
+          const uint32_t sb = *reinterpret_cast<const uint16_t*>(base + b_soff[g] + 512 * cc);
+          const half2v v = __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(sb, 1.0f, false);
+          sc.b[g][0] = half2v{v[0], v[0]};
+          sc.b[g][1] = half2v{v[1], v[1]};
+        }
+      };
+      auto read_raw = [&](Raw& r, int stage, int j) {  // j = 0..7: half j / 4, dword j % 4 of the lane's 16-byte piece
+        const uint8_t* base = smem + stage * S::kStage + 4 * (j & 3);
+        const int flip = 32 * (j >> 2);
+#pragma unroll
+        for (int f = 0; f < FA; ++f) r.a[f] = *reinterpret_cast<const uint32_t*>(base + (a_voff[f] ^ flip));
+#pragma unroll
+        for (int g = 0; g < FB; ++g) r.b[g] = *reinterpret_cast<const uint32_t*>(base + (b_voff[g] ^ flip));
+      };
+      auto decode_raw = [&](Operands& o, const Raw& r, const Scales& sc, int jj) {
+#pragma unroll
+        for (int f = 0; f < FA; ++f) o.a[f] = decode8(r.a[f], sc.a[f][jj >> 1]);
+#pragma unroll
+        for (int g = 0; g < FB; ++g) o.b[g] = decode8(r.b[g], sc.b[g][jj >> 1]);
+      };
+      Operands o[2];
       for (int t = 0; t < nk; ++t) {
         if (t + 1 < nk) load_step(t + 1, (t + 1) & 1);
         if (wave_has_output) {
+          Scales sc[2];
+          Raw raw[2];
+          read_raw(raw[0], t & 1, 0);
+          read_scales(sc[0], t & 1, 0);
+          read_raw(raw[1], t & 1, 1);
+          read_scales(sc[1], t & 1, 1);
+          if (t > 0) mma(o[1]);
+          decode_raw(o[0], raw[0], sc[0], 0);
 #pragma unroll
-          for (int cc = 0; cc < 2; ++cc) {
-            Half h;
-            read_half(h, t & 1, cc);
+          for (int j = 0; j < 7; ++j) {
+            if (j + 2 < 8) read_raw(raw[j & 1], t & 1, j + 2);
+            decode_raw(o[(j + 1) & 1], raw[(j + 1) & 1], sc[(j + 1) >> 2], (j + 1) & 3);
+            mma(o[j & 1]);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              Operands o;
-              decode(o, h, j);
-              mma(o);
+            for (int g = 0; g < FA * FB; ++g) {
+              __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+              __builtin_amdgcn_sched_group_barrier(0x002, (8 * (FA + FB) + FA * FB - 1) / (FA * FB), 0);  // its share of the decode
             }
           }
         }
         __builtin_amdgcn_s_waitcnt(0x0F70);
         __syncthreads();
       }
+      if (wave_has_output) mma(o[1]);
     }
   }
 
