@@ -34,10 +34,55 @@ LINEAR_SET = [
     ("ffn_down", M_TOKENS, FFN, DIM, 1),
 ]
 PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak (the GEMM runs v_mfma_f32_32x32x16_f16)
-# HBM-side bytes of one FFN-up GEMM launch from the rocprofv3 counter runs kept under profiles/:
-# FETCH_SIZE 82078 KiB x 2.0 (the factor a 256 MiB copy calibrates) + WRITE_SIZE 73920 KiB x 1.0
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak
 PREWARM_SECONDS = 0.5  # untimed load ahead of the warm-up steps (clock ramp-up), reported as config.prewarm_s
-FFN_UP_TRAFFIC_BYTES = (75334.7 * 2.0 + 73927.3) * 1024  # FETCH_SIZE x 2.00 (copy yardstick) + WRITE_SIZE, KiB per launch
+# rocprofv3 counter summary of the FFN-up GEMM launch (FETCH_SIZE / WRITE_SIZE per dispatch and the factors a plain
+# copy of known size calibrates); roofline.traffic is computed from the numbers in that file, or null without it
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_w4a4_ffn_up_hbm_traffic.txt")
+
+
+def measured_traffic_bytes():
+    """HBM bytes of one FFN-up GEMM launch = FETCH_SIZE x fetch factor + WRITE_SIZE x write factor, read from the
+    `key = value` lines of the counter summary under profiles/ (None when the file or a key is missing)."""
+    keys = {"fetch_size_kib_per_launch": None, "fetch_scale": None, "write_size_kib_per_launch": None, "write_scale": None}
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                name, sep, value = line.partition("=")
+                if sep and name.strip() in keys:
+                    keys[name.strip()] = float(value.split()[0])
+    except (OSError, ValueError):
+        return None
+    if any(v is None for v in keys.values()):
+        return None
+    return (keys["fetch_size_kib_per_launch"] * keys["fetch_scale"]
+            + keys["write_size_kib_per_launch"] * keys["write_scale"]) * 1024.0
+
+
+def physical_cores() -> int:
+    """Physical cores this process may use: distinct (package, core) pairs of /proc/cpuinfo among the CPUs of the
+    affinity mask, capped by OMP_NUM_THREADS (the share of the machine a one-GPU job is given)."""
+    try:
+        allowed = os.sched_getaffinity(0)
+    except AttributeError:
+        allowed = set(range(os.cpu_count() or 1))
+    cores, cpu, phys = set(), None, "0"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                key, _, val = line.partition(":")
+                key, val = key.strip(), val.strip()
+                if key == "processor":
+                    cpu, phys = int(val), "0"
+                elif key == "physical id":
+                    phys = val
+                elif key == "core id" and cpu in allowed:
+                    cores.add((phys, val))
+    except OSError:
+        pass
+    n = len(cores) or len(allowed)
+    cap = os.environ.get("OMP_NUM_THREADS")
+    return max(1, min(n, int(cap)) if cap and cap.isdigit() else n)
 
 
 def step_flops() -> float:
@@ -54,23 +99,28 @@ def cpu_baseline(work) -> dict:
     import torch
     from helpers import bits_of
 
+    from threadpoolctl import threadpool_limits
+
+    cores = physical_cores()
     host = []
     for _, x, wq in work:
         wd = dict(values=wq.values.cpu().numpy(), scales=wq.scale_factors.cpu().view(torch.uint8).numpy(),
                   amax=np.float32(wq.amax.item()), rule="mse", padded=tuple(wq.padded_shape), orig=tuple(wq.original_shape))
         host.append((bits_of(x.cpu()), wd))
-    t0 = time.perf_counter()
     n_steps = 0
-    while n_steps < 1 or (time.perf_counter() - t0 < 10.0 and n_steps < 8):  # about 10-30 s of CPU work
-        for xb, wd in host:
-            v, sc, a, pad = o.quantize_to_fp4(xb, "mse")
-            y = o.fp4_matmul(dict(values=v, scales=sc, amax=a, rule="mse", padded=pad, orig=xb.shape), wd)
-        n_steps += 1
-    dt = time.perf_counter() - t0
+    with threadpool_limits(limits=cores):  # BLAS threads of the fp32 matmul = physical cores; the rest is numpy
+        t0 = time.perf_counter()
+        while n_steps < 1 or (time.perf_counter() - t0 < 10.0 and n_steps < 8):  # about 10-30 s of CPU work
+            for xb, wd in host:
+                v, sc, a, pad = o.quantize_to_fp4(xb, "mse")
+                y = o.fp4_matmul(dict(values=v, scales=sc, amax=a, rule="mse", padded=pad, orig=xb.shape), wd)
+            n_steps += 1
+        dt = time.perf_counter() - t0
     assert np.isfinite(y).all()
-    return {"value": n_steps * step_flops() / dt / 1e12, "unit": "TFLOP/s",
-            "cores": int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)), "kind": "port",
-            "sample": f"{n_steps} whole step(s) of the same workload (10 linears, 783.4 GFLOP each, weights pre-quantized), {dt:.1f} s"}
+    return {"value": n_steps * step_flops() / dt / 1e12, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{n_steps} whole step(s) of the same workload (10 linears, 783.4 GFLOP each, weights "
+                      f"pre-quantized), {dt:.1f} s; BLAS threads limited to the {cores} physical cores of the "
+                      "process's CPU share, the element-wise numpy part of the oracle is single-threaded"}
 
 
 def _time_events(torch, fn, n, warm=10, repeats=3):
@@ -208,6 +258,26 @@ def run_e2e(torch, dev):
                         "sink 3 + window 12 frames, text K/V projected once per prompt, cache written by the recache forward only (the denoising forwards' writes are dead stores); one untimed 3-frame run first; the chunks get slower until the window of 12 frames is full"}
 
 
+def run_quantize(torch, dev, steps, rule="mse"):
+    """The quantize kernel alone on the FFN-down activation shape (2640 x 14336 bf16, the tensor with the most
+    blocks), tensor amax taken from an amax sink as in the DiT block (no reduction pass): the launch the
+    `roofline_quantize` record and the instruction-count profile are about."""
+    from helpers import activations
+    from longlive_amd import _native
+    from longlive_amd.fouroversix import QuantizationConfig, quantize_to_fp4
+
+    cfg = QuantizationConfig(scale_rule=rule)
+    x = activations((M_TOKENS, FFN), 7).to(dev)
+    # what a producer kernel leaves behind: slot 0 of the sink holds (epoch << 32) | bits of max |x|
+    ticket = _native.amax_ticket(dev)
+    amax_bits = int(x.float().abs().max().view(torch.int32).item())
+    ticket.parts[0] = (ticket.epoch << 32) | amax_bits
+    ms = _time_events(torch, lambda: quantize_to_fp4(x, cfg, amax=ticket), steps)
+    gbs = 2.5625 * x.numel() / ms / 1e6
+    return {"quantize_ms": ms, "GB_per_s": gbs, "frac_of_hbm_8TBs": gbs / PEAK_HBM_GBS, "rule": rule,
+            "workload": "quantize_kernel alone, 2640 x 14336 bf16 -> NVFP4, 96.98 MB algorithmic traffic, amax from a sink"}
+
+
 def run_gemm_shapes(torch, dev, work, cfg, steps):
     """The W4A4 GEMM kernel alone on each distinct shape of the linear set (operands already quantized), with the
     vendor library's dense f16 GEMM (torch.matmul) on operands of the same shape beside it: the library kernel
@@ -240,7 +310,7 @@ def main() -> None:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the attention / block / end-to-end figures")
-    ap.add_argument("--workload", choices=["linears", "attention", "block", "block_release", "e2e", "copy"], default="linears")
+    ap.add_argument("--workload", choices=["linears", "attention", "block", "block_release", "e2e", "copy", "quantize", "quantize_static"], default="linears")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives are part of this path); use --gpus 1")
@@ -264,6 +334,8 @@ def main() -> None:
     if args.workload != "linears":
         res = {"attention": lambda: run_attention(torch, dev, args.steps), "block": lambda: run_block(torch, dev, args.steps),
                "block_release": lambda: run_block_release(torch, dev, args.steps),
+               "quantize": lambda: run_quantize(torch, dev, args.steps),
+               "quantize_static": lambda: run_quantize(torch, dev, args.steps, "static_6"),
                "e2e": lambda: run_e2e(torch, dev)}[args.workload]()
         print(json.dumps(res))
         return
@@ -371,7 +443,7 @@ def main() -> None:
                                "dim 3072, ffn 14336, rule mse, seed 1", "flop_per_step": step_flops(),
                    "prewarm_s": PREWARM_SECONDS},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_F16_TFLOPS, "traffic": FFN_UP_TRAFFIC_BYTES,
+                     "frac": achieved / PEAK_F16_TFLOPS, "traffic": measured_traffic_bytes(),
                      "kernel": "gemm_w4a4_kernel M=2640 N=14336 K=3072", "avg_ms": gemm_ms},
         "quantize": {"shape": [M_TOKENS, FFN], "avg_ms": q_ms, "GB_per_s": q_gbs, "frac_of_hbm_8TBs": q_gbs / 8000.0,
                      "note": "amax + quantize kernels, 2.5625 algorithmic bytes per element",
@@ -382,6 +454,15 @@ def main() -> None:
                                      "note": "the same kernel rotating over seven copies of its input (530 MB, more "
                                              "than the last-level cache), so every launch reads from HBM"}},
     }
+    # the same shape of record for the other two hot kernels (the contract's `roofline` stays the GEMM's)
+    q_bytes = 2.5625 * h.numel()
+    out["roofline_quantize"] = {"bound": "hbm", "achieved": qs_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                "frac": qs_gbs / PEAK_HBM_GBS, "traffic": q_bytes,
+                                "kernel": "quantize_kernel<mse> 2640x14336 (tensor amax from the producer's epilogue)",
+                                "avg_ms": qs_ms, "cold_input_frac": qc_gbs / PEAK_HBM_GBS,
+                                "with_amax_pass_frac": q_gbs / PEAK_HBM_GBS,
+                                "note": "achieved = 2.5625 algorithmic bytes per element / kernel time; traffic = the "
+                                        "same bytes (FETCH_SIZE + WRITE_SIZE of the kernel equal them, profiles/)"}
     if not args.no_extras:
         extras = {}
         for key, fn in (("gemm_shapes", lambda: run_gemm_shapes(torch, dev, work, cfg, 10)),
@@ -394,6 +475,12 @@ def main() -> None:
                 extras[key] = {"error": f"{type(exc).__name__}: {exc}"}
             torch.cuda.empty_cache()
         out["extras"] = extras
+        att = extras.get("attention", {})
+        if "attention_ms" in att:
+            out["roofline_attention"] = {"bound": "mfma", "achieved": att["attention_TFLOPs"], "peak": PEAK_F16_TFLOPS,
+                                         "unit": "TFLOP/s", "frac": att["attention_TFLOPs"] / PEAK_F16_TFLOPS,
+                                         "traffic": None, "kernel": "kv_attention_kernel Lq=2640 Lk=13200 H=24 (configs[2])",
+                                         "avg_ms": att["attention_ms"]}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(work)
     print(json.dumps(out))
