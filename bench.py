@@ -259,19 +259,20 @@ def run_e2e(torch, dev):
 
 
 def run_quantize(torch, dev, steps, rule="mse"):
-    """The quantize kernel alone on the FFN-down activation shape (2640 x 14336 bf16, the tensor with the most
-    blocks), tensor amax taken from an amax sink as in the DiT block (no reduction pass): the launch the
-    `roofline_quantize` record and the instruction-count profile are about."""
-    from helpers import activations
+    """The quantize kernel alone on the FFN-down activation (2640 x 14336 bf16, the tensor with the most blocks),
+    tensor amax taken from the amax sink its producer filled, as in the DiT block (no reduction pass): the launch
+    the `roofline_quantize` record and the instruction-count profile are about."""
+    from helpers import activations, weights
     from longlive_amd import _native
-    from longlive_amd.fouroversix import QuantizationConfig, quantize_to_fp4
+    from longlive_amd.fouroversix import QuantizationConfig, fp4_matmul, quantize_to_fp4
 
     cfg = QuantizationConfig(scale_rule=rule)
-    x = activations((M_TOKENS, FFN), 7).to(dev)
-    # what a producer kernel leaves behind: slot 0 of the sink holds (epoch << 32) | bits of max |x|
+    # the tensor the DiT block quantizes at this point: the FFN-up GEMM's GELU output, whose amax that GEMM's
+    # epilogue leaves in the sink
+    xq = quantize_to_fp4(activations((M_TOKENS, DIM), 2008).to(dev), QuantizationConfig(scale_rule="mse"))
+    wq = quantize_to_fp4(weights((FFN, DIM), 1008).to(dev), QuantizationConfig(scale_rule="mse"))
     ticket = _native.amax_ticket(dev)
-    amax_bits = int(x.float().abs().max().view(torch.int32).item())
-    ticket.parts[0] = (ticket.epoch << 32) | amax_bits
+    x = fp4_matmul(xq, wq, activation="gelu_tanh", amax_out=ticket)
     ms = _time_events(torch, lambda: quantize_to_fp4(x, cfg, amax=ticket), steps)
     gbs = 2.5625 * x.numel() / ms / 1e6
     return {"quantize_ms": ms, "GB_per_s": gbs, "frac_of_hbm_8TBs": gbs / PEAK_HBM_GBS, "rule": rule,

@@ -148,37 +148,68 @@ class AmaxTicket:
     """One use of a device's amax sink: handed to the kernel that writes a tensor (``amax_out=``) and then to
     the quantization of that tensor (``amax=``), which reads the maximum the producer left."""
 
-    __slots__ = ("parts", "epoch")
+    __slots__ = ("parts", "epoch", "key")
 
-    def __init__(self, parts: torch.Tensor, epoch: int) -> None:
-        self.parts, self.epoch = parts, epoch
+    def __init__(self, parts: torch.Tensor, epoch: int, key=None) -> None:
+        self.parts, self.epoch, self.key = parts, epoch, key
 
     def struct(self) -> AmaxSinkStruct:
         return AmaxSinkStruct(self.parts.data_ptr(), self.epoch)
 
 
+# per device: [sink buffer, last epoch issued, (epoch, stream) of the last producer launch]
 _sinks: dict = {}
 
 
 def amax_ticket(device: torch.device) -> AmaxTicket:
     """A fresh epoch on the device's amax sink buffer.  Epochs only grow, which is what lets the buffer go
-    uncleared between uses; producer and consumer must run on one stream, in that order."""
+    uncleared between uses.  All tickets of a device share the one buffer, so a ticket is good for exactly one
+    producer launch followed by the quantization(s) of its output, on one stream, with no other producer launch
+    in between: a later producer overwrites the slots.  The host side checks this (see ``_check_consumer``)."""
     device = torch.device(device)
-    key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+    index = device.index if device.index is not None else (torch.cuda.current_device() if device.type == "cuda" else 0)
+    key = (device.type, index)
     entry = _sinks.get(key)
     if entry is None or entry[1] >= 0xFFFFFFFE:
-        entry = [torch.zeros(AMAX_PARTS, dtype=torch.int64, device=device), 0]
+        entry = [torch.zeros(AMAX_PARTS, dtype=torch.int64, device=device), 0, None]
         _sinks[key] = entry
     entry[1] += 1
-    return AmaxTicket(entry[0], entry[1])
+    return AmaxTicket(entry[0], entry[1], key)
+
+
+def _stream_of(ticket: AmaxTicket) -> int:
+    return _stream() if ticket.parts.is_cuda else 0
 
 
 def _sink_struct(ticket):
+    """The struct a producer kernel is given; notes the launch as the sink's latest producer."""
     if ticket is None:
         return AmaxSinkStruct(None, 0)
     if not isinstance(ticket, AmaxTicket):
         raise TypeError("amax_out must be an AmaxTicket (see amax_ticket)")
+    entry = _sinks.get(ticket.key)
+    if entry is not None and entry[0] is ticket.parts:
+        entry[2] = (ticket.epoch, _stream_of(ticket))
     return ticket.struct()
+
+
+def _check_consumer(ticket: AmaxTicket) -> None:
+    """A quantization may read a ticket's amax only while that ticket's producer is the latest producer launch
+    on the device's sink, and on the stream the producer ran on.  Anything else (another producer launched in
+    between, the producer never launched, a different stream) would make the kernel read partial maxima of
+    another tensor or none at all and quantize against a wrong amax without any error, so it is refused here."""
+    entry = _sinks.get(ticket.key)
+    if entry is None or entry[0] is not ticket.parts:
+        raise RuntimeError("this amax ticket belongs to a sink buffer that has been replaced")
+    last = entry[2]
+    if last is None or last[0] != ticket.epoch:
+        raise RuntimeError(
+            f"amax ticket {ticket.epoch} is not the latest producer on its sink (latest: "
+            f"{'none' if last is None else last[0]}): between the kernel that was given this ticket as amax_out and "
+            "the quantization of its output no other kernel may be given a ticket of the same device")
+    if last[1] != _stream_of(ticket):
+        raise RuntimeError("the producer of this amax ticket ran on another stream than the quantization that "
+                           "reads it; both must be issued on one stream")
 
 
 # --------------------------------------------------------------------------- quantize / dequantize
@@ -189,6 +220,7 @@ def quantize(x: torch.Tensor, rule: str, amax: torch.Tensor | None = None, out=N
     given, in which case the bytes equal those of ``amax=None``."""
     ticket = amax if isinstance(amax, AmaxTicket) else None
     if ticket is not None:
+        _check_consumer(ticket)
         amax = None
     _require_cuda(x, amax)
     if x.ndim != 2:

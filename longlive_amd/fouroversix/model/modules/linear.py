@@ -85,6 +85,30 @@ class FourOverSixLinear(nn.Linear):
     def quantized_weight_transposed(self) -> None:
         return None
 
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                              error_msgs) -> None:
+        """State dicts written by the reference's module load as they are: after quantization the reference holds
+        the tensor amax as a 0-dim tensor (it registers a [1] buffer, linear.py:203-206, and replaces it with
+        ``QuantizedTensor.amax``), and values / scale factors in the padded shape (rows to 128, columns to 64)
+        where the freshly swapped module registered the unpadded one.  Buffers are brought to the incoming
+        shapes before the regular copy, so ``strict=True`` holds for such checkpoints."""
+        amax_key = prefix + "quantized_weight_amax"
+        own_amax = getattr(self, "quantized_weight_amax", None)
+        incoming = state_dict.get(amax_key)
+        if isinstance(incoming, torch.Tensor) and isinstance(own_amax, torch.Tensor) and incoming.numel() == 1 \
+                and incoming.shape != own_amax.shape:
+            state_dict[amax_key] = incoming.reshape(own_amax.shape)
+        for name in ("quantized_weight_values", "quantized_weight_scale_factors"):
+            own, incoming = getattr(self, name, None), state_dict.get(prefix + name)
+            if isinstance(own, torch.Tensor) and isinstance(incoming, torch.Tensor) and own.shape != incoming.shape \
+                    and own.dtype == incoming.dtype and incoming.numel() >= own.numel():
+                setattr(self, name, torch.zeros(incoming.shape, dtype=own.dtype, device=own.device))
+        for attr in ("_quantized_weight", "_quantized_weight_transposed"):
+            if hasattr(self, attr):
+                delattr(self, attr)
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys, unexpected_keys,
+                                      error_msgs)
+
     # ------------------------------------------------------------------ forward
     def forward(self, input: torch.Tensor) -> torch.Tensor:
         if input.requires_grad and torch.is_grad_enabled():

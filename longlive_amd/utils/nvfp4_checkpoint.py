@@ -142,6 +142,17 @@ def load_nvfp4_generator(generator: nn.Module, checkpoint, config=None, *, use_e
         raise ValueError(f"unsupported {NVFP4_CHECKPOINT_FORMAT} version {version}")
     state = clean_fsdp_state_dict_keys(unwrap_generator_state_dict(checkpoint, use_ema=use_ema))
     if is_nvfp4_state_dict(state):
+        # The packed weights were produced under one scale rule, and the rule fixes the denominator of their
+        # dequantization (6 * 256 for the four-over-six rules, 6 * 448 / 4 * 448 for the static ones): loading them
+        # under another rule would silently scale every weight.  The checkpoint records its rule; refuse a mismatch.
+        recorded = (checkpoint.get("quantization") or {}).get("scale_rule")
+        qcfg = build_model_quantization_config(config)
+        wanted = qcfg.weight_scale_rule or qcfg.scale_rule
+        wanted = getattr(wanted, "value", wanted)
+        if recorded is not None and str(recorded) != str(wanted):
+            raise ValueError(f"the checkpoint's weights were quantized with scale rule {recorded!r}, the run "
+                             f"configuration asks for {wanted!r} (model_quant_scale_rule / "
+                             "model_quant_weight_scale_rule): they must agree")
         generator, _ = quantize_model_for_fouroversix_nvfp4(generator, config, keep_master_weights=False,
                                                             verbose=verbose)
         drop_fouroversix_master_weights(generator)

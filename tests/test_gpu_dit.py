@@ -417,6 +417,9 @@ def test_packed_nvfp4_checkpoint_round_trip(gpu, tmp_path):
         ck.load_nvfp4_generator(fresh(), {"checkpoint_format": ck.TE_NVFP4_CHECKPOINT_FORMAT, "generator": {}})
     with pytest.raises(ValueError):
         ck.load_nvfp4_generator(fresh(), {**saved, "checkpoint_version": 2})
+    # a checkpoint quantized under mse must not be loaded under the default static_6 configuration
+    with pytest.raises(ValueError, match="scale rule"):
+        ck.load_nvfp4_generator(fresh(), saved, SimpleNamespace())
 
 
 def test_text_kv_cache_gives_identical_latents(gpu):

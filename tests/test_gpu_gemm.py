@@ -1,12 +1,14 @@
 """GPU parity: W4A4 GEMM and the quantized Linear against the oracle's dequantize-then-fp32-matmul.
 Bar (floating point): relative Frobenius error <= 1e-3."""
+import os
+
 import numpy as np
 import pytest
 import torch
 import torch.nn as nn
 
 import nvfp4_oracle as o
-from helpers import activations, bits_of, u8, weights
+from helpers import activations, bits_of, from_bits, u8, weights
 from longlive_amd import _native
 from longlive_amd.fouroversix import (FourOverSixLinear, ModelQuantizationConfig, QuantizationConfig,
                                       QuantizedTensor, fp4_matmul, quantize_to_fp4)
@@ -255,3 +257,90 @@ def test_ffn_down_full_size_fused_epilogue_and_sink(gpu):
     y = fp4_matmul(hq, w_down)
     fused = fp4_matmul(hq, w_down, residual=residual, gate=gate, gate_rows=frame)
     assert torch.equal(fused, residual + (y.view(M // frame, frame, D) * gate[:, None]).view(M, D))
+
+
+# --------------------------------------------------------------------------- reference-written module state
+def _fixture_state(fx, name, device):
+    state = {}
+    for key in fx[f"{name}/state_keys"]:
+        arr, dt = fx[f"{name}/state/{key}"], str(fx[f"{name}/state_dtype/{key}"])
+        if dt == "torch.bfloat16":
+            t = torch.from_numpy(arr.view(np.int16).copy()).view(torch.bfloat16)
+        elif dt == "torch.float8_e4m3fn":
+            t = torch.from_numpy(arr.copy()).view(torch.float8_e4m3fn)
+        else:
+            t = torch.from_numpy(arr.copy())
+        state[str(key)] = t.to(device)
+    return state
+
+
+@pytest.mark.parametrize("name", ["aligned_192x128", "padded_128x96"])
+def test_state_dict_written_by_the_reference_module_loads_and_runs(gpu, name):
+    """tests/golden/fouroversix_linear_state.npz holds the state dict of the reference's own FourOverSixLinear
+    (fouroversix/src/fouroversix/model/modules/linear.py:182-216, 271-307; written by
+    tests/golden/make_linear_golden.py) for two nn.Linear layers, one of them with an output dimension that is not a
+    multiple of 128, and the reference's forward on a fixed input.  (1) Quantizing the same master weight with this
+    package gives the same buffers, bit for bit.  (2) The reference's state dict loads into this package's module
+    with strict=True.  (3) The forward on the loaded module matches the reference's output (relative Frobenius
+    <= 1e-3, the GEMM bar) and the oracle's."""
+    from longlive_amd.fouroversix import FourOverSixLinear, ModuleQuantizationConfig
+    from longlive_amd.utils.quant import _materialize_quantized_weights_for_inference
+
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "fouroversix_linear_state.npz"))
+    assert name in list(fx["case_names"])
+    w = from_bits(fx[f"{name}/weight"], gpu)
+    fout, fin = w.shape
+
+    def fresh(weight, bias):
+        lin = torch.nn.Linear(fin, fout, bias=True).to(gpu).to(torch.bfloat16)
+        with torch.no_grad():
+            lin.weight.copy_(weight)
+            lin.bias.copy_(bias)
+        mod = FourOverSixLinear(lin, ModuleQuantizationConfig(scale_rule="mse"))
+        assert sorted(mod.state_dict().keys()) == sorted(str(k) for k in fx[f"{name}/registered_keys"])
+        for k, v in mod.state_dict().items():
+            assert tuple(v.shape) == tuple(fx[f"{name}/registered_shape/{k}"]), k
+        holder = torch.nn.Sequential(mod)
+        _materialize_quantized_weights_for_inference(holder)
+        return holder[0]
+
+    ref_state = _fixture_state(fx, name, gpu)
+    # (1) own quantization of the same weight
+    own = fresh(w, from_bits(fx[f"{name}/bias"], gpu))
+    own_state = own.state_dict()
+    assert sorted(own_state.keys()) == sorted(ref_state.keys())
+    for k, v in ref_state.items():
+        a, b = own_state[k], v
+        assert a.dtype == b.dtype and a.numel() == b.numel(), k
+        assert torch.equal(a.reshape(-1).view(torch.uint8), b.reshape(-1).view(torch.uint8)), k
+    # (2) strict load into a module built from other weights
+    other = fresh(torch.zeros_like(w), torch.zeros(fout, dtype=torch.bfloat16, device=gpu))
+    result = other.load_state_dict(ref_state, strict=True)
+    assert not result.missing_keys and not result.unexpected_keys
+    # the same into a freshly swapped module whose master weight was dropped without quantizing it: its buffers
+    # still have the registered (unpadded) shapes, the load brings them to the checkpoint's
+    lin = torch.nn.Linear(fin, fout, bias=True).to(gpu).to(torch.bfloat16)
+    bare = FourOverSixLinear(lin, ModuleQuantizationConfig(scale_rule="mse"))
+    bare.register_parameter("weight", None)
+    result = bare.load_state_dict(ref_state, strict=True)
+    assert not result.missing_keys and not result.unexpected_keys
+    for k, v in ref_state.items():
+        assert torch.equal(bare.state_dict()[k].reshape(-1).view(torch.uint8), v.reshape(-1).view(torch.uint8)), k
+    # (3) forward
+    x = from_bits(fx[f"{name}/x"], gpu)
+    with torch.no_grad():
+        y = other(x)
+        y_own = own(x)
+        assert torch.equal(bare(x), y)
+    assert torch.equal(y, y_own)
+    y_ref = from_bits(fx[f"{name}/y"]).float().numpy()
+    got = y.float().cpu().numpy()
+    assert got.shape == y_ref.shape
+    assert np.linalg.norm(got - y_ref) / np.linalg.norm(y_ref) <= 1e-3
+    xv, xs, xa, xpad = o.quantize_to_fp4(fx[f"{name}/x"], "mse")
+    qw = other.quantized_weight()
+    oy = o.fp4_matmul(dict(values=xv, scales=xs, amax=xa, rule="mse", padded=xpad, orig=fx[f"{name}/x"].shape),
+                      dict(values=u8(qw.values), scales=u8(qw.scale_factors), amax=np.float32(qw.amax.item()),
+                           rule="mse", padded=tuple(qw.padded_shape), orig=tuple(qw.original_shape)))
+    oy = o.round_bf16(oy + from_bits(fx[f"{name}/bias"]).float().numpy()[None, :])
+    assert np.linalg.norm(got - oy) / np.linalg.norm(oy) <= 1e-3

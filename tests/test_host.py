@@ -51,6 +51,29 @@ def test_noalloc_quantize_refuses_inputs_beyond_its_limit_before_touching_the_gp
     assert lib.ll_nvfp4_quantize_noalloc(None, 0, 64, 64, 3, None, None, None, None) == -1
 
 
+def test_amax_ticket_misuse_is_refused_on_the_host():
+    """All tickets of a device share one sink buffer.  A quantization may consume a ticket only while that
+    ticket's producer launch is the latest one on the sink; the host bookkeeping refuses anything else instead of
+    letting the kernel quantize against another tensor's (or no) maximum."""
+    cpu = torch.device("cpu")
+    a = _native.amax_ticket(cpu)
+    with pytest.raises(RuntimeError, match="not the latest producer"):   # never handed to a producer
+        _native._check_consumer(a)
+    _native._sink_struct(a)                                              # producer launch with ticket a
+    _native._check_consumer(a)                                           # its consumer: fine, also repeatedly
+    _native._check_consumer(a)
+    b = _native.amax_ticket(cpu)
+    assert b.epoch == a.epoch + 1 and b.parts is a.parts
+    _native._check_consumer(a)                                           # issuing a ticket alone changes nothing
+    _native._sink_struct(b)                                              # another producer launches in between
+    with pytest.raises(RuntimeError, match="not the latest producer"):
+        _native._check_consumer(a)
+    _native._check_consumer(b)
+    assert _native._sink_struct(None).parts is None
+    with pytest.raises(TypeError):
+        _native._sink_struct(object())
+
+
 def test_scale_rule_tables():
     assert [ScaleRule(r).cuda_id() for r in ("static_6", "static_4", "mae", "mse", "abs_max")] == [0, 1, 2, 3, 4]
     assert ScaleRule.mse.max_allowed_e4m3_value() == 256 and ScaleRule.static_4.max_allowed_e2m1_value() == 4
