@@ -257,6 +257,10 @@ class CausalHead(nn.Module):
     def forward(self, x, e):
         num_frames, frame_seqlen = e.shape[1], x.shape[1] // e.shape[1]
         e = (self.modulation.unsqueeze(1) + e).chunk(2, dim=2)
+        if x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous() and e[0].dtype == torch.bfloat16:
+            # norm(x) * (1 + e[1]) + e[0] is the adaLN modulation of the blocks, with the same bf16 roundings
+            y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.norm.eps)
+            return self.head(y.unflatten(1, (num_frames, frame_seqlen)))
         return self.head(self.norm(x).unflatten(1, (num_frames, frame_seqlen)) * (1 + e[1]) + e[0])
 
 
@@ -310,6 +314,19 @@ class CausalDiT(nn.Module):
                                                  temporal_offset=float(temporal_offset))
         return self._rope_cache[key]
 
+    def patch_embed(self, x: torch.Tensor):
+        """x [C_in, F, H, W] -> tokens [1, f*h*w, dim] and the grid (f, h, w).  The patch embedding is a Conv3d whose
+        kernel equals its stride (wan_5b/modules/causal_model.py:1052-1053, 1535): every output token is a linear map
+        of one patch, so it runs as one matrix product over the flattened patches (c, pt, ph, pw), the order of the
+        convolution weight, instead of a convolution."""
+        pt, ph, pw = self.cfg.patch_size
+        c, fr, hh, ww = x.shape
+        f, h, w = fr // pt, hh // ph, ww // pw
+        patches = x[:, :f * pt, :h * ph, :w * pw].reshape(c, f, pt, h, ph, w, pw).permute(1, 3, 5, 0, 2, 4, 6)
+        patches = patches.reshape(f * h * w, c * pt * ph * pw)
+        weight = self.patch_embedding.weight.reshape(self.patch_embedding.weight.shape[0], -1)
+        return torch.nn.functional.linear(patches, weight, self.patch_embedding.bias).unsqueeze(0), (f, h, w)
+
     def unpatchify(self, x: torch.Tensor, grid) -> torch.Tensor:
         c = self.cfg.out_dim
         f, h, w = grid
@@ -326,10 +343,8 @@ class CausalDiT(nn.Module):
         (all layers' updates applied after the last block).  ``crossattn_cache``: one dictionary per layer
         holding the projected text K / V of the current prompt (filled on first use)."""
         cfg = self.cfg
-        x = self.patch_embedding(x.unsqueeze(0))
-        f, h, w = x.shape[2:]
+        x, (f, h, w) = self.patch_embed(x)
         frame_seqlen = h * w
-        x = x.flatten(2).transpose(1, 2).contiguous()
         tt = t.flatten()
         e = self.time_embedding(sinusoidal_embedding_1d(cfg.freq_dim, tt).unflatten(0, t.shape).type_as(x))
         e0 = self.time_projection(e).unflatten(2, (6, cfg.dim))

@@ -631,3 +631,25 @@ def test_skipping_dead_cache_writes_is_invisible_in_multi_shot_mode(gpu, clean):
             assert la[key] == lb[key], key
         for sa, sb in zip(la["k"] + la["v"], lb["k"] + lb["v"]):
             assert torch.equal(sa.values, sb.values) and torch.equal(sa.amax, sb.amax)
+
+
+def test_head_modulation_through_the_adaln_kernel_matches_the_eager_graph(gpu):
+    """CausalHead (wan_5b/modules/causal_model.py:933-959): norm(x) * (1 + e[1]) + e[0] runs through the adaLN
+    kernel; against the same expression evaluated by torch's bf16 operations (each intermediate rounded to bf16) the
+    head output may differ by the last bit of the modulated activations only."""
+    from longlive_amd.dit.model import CausalHead
+
+    torch.manual_seed(5)
+    dim, F, fs = 512, 3, 40
+    head = CausalHead(dim, 8, (1, 2, 2)).to(gpu).to(torch.bfloat16)
+    torch.nn.init.normal_(head.head.weight, std=0.05)
+    g = torch.Generator().manual_seed(6)
+    x = (torch.randn(1, F * fs, dim, generator=g) * 3).bfloat16().to(gpu)
+    e = torch.randn(1, F, 1, dim, generator=g).bfloat16().to(gpu)
+    with torch.no_grad():
+        got = head(x, e)
+        em = (head.modulation.unsqueeze(1) + e).chunk(2, dim=2)
+        ln = torch.nn.functional.layer_norm(x.float(), (dim,), eps=head.norm.eps).bfloat16()
+        ref = head.head(ln.unflatten(1, (F, fs)) * (1 + em[1]) + em[0])
+    assert got.shape == ref.shape == (1, F, fs, 32)
+    assert (got.float() - ref.float()).abs().max() <= 2.0 ** -6 * ref.float().abs().max()

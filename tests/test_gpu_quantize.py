@@ -85,6 +85,14 @@ def test_benchmark_activation_full_size(gpu):
     _check(bits_of(activations((2640, 3072), 0)), "mse", gpu)
 
 
+@pytest.mark.parametrize("rule", ["mse", "mae"])
+def test_ffn_down_activation_full_size_bit_exact(gpu, rule):
+    """The activation with the most blocks, [2640, 14336] (2.4 million blocks of 16, the input of the FFN-down
+    linear), against the CPU oracle bit for bit: every block whose four-over-six choice the kernel takes from its
+    error estimate instead of the reference's arithmetic is one more chance for a wrong confident decision to show."""
+    _check(bits_of(activations((2640, 14336), 10)), rule, gpu)
+
+
 def test_strided_input_and_given_amax(gpu):
     big = activations((200, 512), 8).to(gpu)
     view = big[:, 128:384]  # row stride 512, 256 columns

@@ -74,6 +74,21 @@ def test_amax_ticket_misuse_is_refused_on_the_host():
         _native._sink_struct(object())
 
 
+def test_patch_embedding_as_matrix_product_equals_the_convolution():
+    """CausalDiT.patch_embed runs the Conv3d with kernel = stride = patch (wan_5b/modules/causal_model.py:1052-1053)
+    as one matrix product over flattened patches; fp32 on the CPU it must reproduce torch's convolution."""
+    from longlive_amd.dit.model import CausalDiT, DiTConfig
+
+    torch.manual_seed(0)
+    cfg = DiTConfig(dim=64, ffn_dim=128, num_heads=1, num_layers=0, in_dim=5, out_dim=5, text_dim=16, text_len=4)
+    m = CausalDiT(cfg)
+    x = torch.randn(5, 3, 8, 12)
+    tokens, grid = m.patch_embed(x)
+    conv = m.patch_embedding(x.unsqueeze(0))
+    assert grid == tuple(conv.shape[2:]) == (3, 4, 6)
+    assert torch.allclose(tokens, conv.flatten(2).transpose(1, 2), atol=1e-6)
+
+
 def test_scale_rule_tables():
     assert [ScaleRule(r).cuda_id() for r in ("static_6", "static_4", "mae", "mse", "abs_max")] == [0, 1, 2, 3, 4]
     assert ScaleRule.mse.max_allowed_e4m3_value() == 256 and ScaleRule.static_4.max_allowed_e2m1_value() == 4
