@@ -196,6 +196,27 @@ int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads,
                          const void* k_new, const void* v_new, int64_t n_new,
                          float softmax_scale, void* out, const ll_amax_sink* amax_sink, void* stream);
 
+/*
+ * How ll_kv_attention / ll_kv_attention_amax / ll_attention_bf16 divide a launch between workgroups.  No
+ * counterpart in the reference (it calls flash attention).  LL_ATTENTION_AUTO, the initial setting, picks per
+ * launch the cheapest of the three by a cost estimate:
+ *   LL_ATTENTION_NARROW  one workgroup per (head, 128 queries);
+ *   LL_ATTENTION_WIDE    one workgroup per (head, 256 queries): every decoded K/V tile serves twice as many MFMAs;
+ *   LL_ATTENTION_SPLIT   256-query tiles, the (tile, key range) sequence cut into one equal share per compute
+ *                        unit, so that the last round of workgroups is as full as the others.  Tiles shared by two
+ *                        workgroups pass through device memory that the library allocates on the first such
+ *                        launch on a (device, stream) pair and keeps (69 MB on a 256-CU device); launches that
+ *                        use it must not overlap on one stream's memory, which same-stream order guarantees.
+ * The three give the same result up to the order of fp32 additions (each is deterministic).  Callers that must
+ * not allocate during a launch (graph capture) select NARROW or WIDE.  The setting is process-wide.
+ */
+#define LL_ATTENTION_AUTO (-1)
+#define LL_ATTENTION_NARROW 0
+#define LL_ATTENTION_WIDE 1
+#define LL_ATTENTION_SPLIT 2
+int ll_kv_attention_set_policy(int policy); /* LL_OK, or LL_EINVAL for an unknown policy */
+int ll_kv_attention_get_policy(void);
+
 /* Plain bf16 attention (cross-attention to the text context; wan_5b/modules/causal_model.py:197-262):
  * q [Lq,H,128], k/v [Lk,H,128], out [Lq,H,128], no mask. */
 int ll_attention_bf16(const void* q, const void* k, const void* v, int64_t Lq, int64_t Lk, int num_heads,

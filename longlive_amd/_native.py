@@ -51,6 +51,8 @@ _SIGNATURES = {
                                      c_void_p, c_int64, c_int, c_float, c_float, c_void_p, c_void_p, c_int64, c_float,
                                      c_void_p, c_void_p, c_void_p]),
     "ll_attention_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_float, c_void_p, c_void_p]),
+    "ll_kv_attention_set_policy": (c_int, [c_int]),
+    "ll_kv_attention_get_policy": (c_int, []),
     "ll_rope_apply": (c_int, [c_void_p, c_int64, c_int, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int64,
                               c_void_p, c_void_p]),
     "ll_adaln_modulate": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64,
@@ -358,6 +360,28 @@ def kv_attention(q, tables, n_cached, block_token_size, e2m1_max, e4m3_max, k_ne
 
 def attention_bf16(q, k, v, softmax_scale, amax_out=None):
     return kv_attention(q, None, 0, 0, 6.0, 256.0, k, v, softmax_scale, amax_out=amax_out)
+
+
+ATTENTION_POLICIES = {"auto": -1, "narrow": 0, "wide": 1, "split": 2}
+
+
+class attention_policy:
+    """``with attention_policy("narrow"): ...`` - how the attention launches inside the block divide their work
+    between workgroups ("auto", "narrow", "wide" or "split"; process-wide, restored on exit)."""
+
+    def __init__(self, name: str):
+        if name not in ATTENTION_POLICIES:
+            raise ValueError(f"unknown attention policy {name!r}; one of {sorted(ATTENTION_POLICIES)}")
+        self.value = ATTENTION_POLICIES[name]
+
+    def __enter__(self):
+        self.previous = load().ll_kv_attention_get_policy()
+        _check(load().ll_kv_attention_set_policy(self.value), "ll_kv_attention_set_policy")
+        return self
+
+    def __exit__(self, *exc):
+        _check(load().ll_kv_attention_set_policy(self.previous), "ll_kv_attention_set_policy")
+        return False
 
 
 # --------------------------------------------------------------------------- elementwise

@@ -18,6 +18,10 @@
 // the row-major tile through ds_read_b64_tr_b16, the LDS read that transposes 16-bit elements across 16 lanes.
 #include "ll_common.h"
 
+#include <map>
+#include <mutex>
+#include <utility>
+
 namespace ll {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -36,6 +40,7 @@ constexpr int kVTileBytes = kTileKeys * kVPitch;
 constexpr int kStageBytes = 2 * kKTileBytes + 2 * kVTileBytes;
 constexpr int kMaxSlots = 64;
 constexpr int kAttnThreads = 512;
+constexpr int kPartialFloats = 8 * 66 * 64;    // a workgroup's partial result: per wave 64 O^T registers, reference point and row sum, per lane
 
 struct AttnParams {
   const uint16_t* q;
@@ -50,6 +55,13 @@ struct AttnParams {
   uint16_t* out;
   AmaxSink sink;  // receives max |out| when sink.parts is not null
   int n_qtiles;
+  // Split of the key range between workgroups (256-query kernel only).  The launch covers `units` = tiles x
+  // iterations; workgroup g of G works through the units [g * units / G, (g + 1) * units / G).  With units =
+  // G * iterations every workgroup owns exactly one tile and `partials` / `arrivals` are not touched.
+  uint32_t units;
+  uint32_t groups;  // G, the number of workgroups of the launch
+  float* partials;  // [2 G] records of kPartialFloats floats
+  int* arrivals;    // [tiles] counters, zero between launches
 };
 
 struct SlotTable {
@@ -59,6 +71,7 @@ struct SlotTable {
   const uint8_t* vs[kMaxSlots];
   float kg[kMaxSlots];
   float vg[kMaxSlots];
+  int last_arrival;  // whether this workgroup completed the tile it just left a partial result for
 };
 
 __device__ __forceinline__ uint32_t pack_bf16(float a, float b) { return pack_bf16x2(a, b); }
@@ -171,22 +184,60 @@ __device__ __forceinline__ void store_row(const KRaw& f, int kind, float gs, con
   }
 }
 
+// The kernel's arguments, read again from the argument segment at the point of use.  What is needed only between
+// two segments of work (output pointers, the split of the units) then occupies no scalar registers during the main
+// loops, which need all of them; the empty asm statement keeps the compiler from moving the reads to the kernel's start.
+__device__ __forceinline__ const __attribute__((address_space(4))) AttnParams& reread_params() {
+  const __attribute__((address_space(4))) AttnParams* a =
+      (const __attribute__((address_space(4))) AttnParams*)__builtin_amdgcn_kernarg_segment_ptr();
+  asm volatile("" : "+s"(a));
+  return *a;
+}
+// threadIdx.x as a value the compiler knows nothing about: what is derived from it inside a segment's prologue or
+// epilogue is then computed there, and not ahead of the loop over segments, where it would occupy registers
+// throughout the main loops.
+__device__ __forceinline__ int fresh_thread_index() {
+  int t = threadIdx.x;
+  asm volatile("" : "+v"(t));
+  return t;
+}
+// Partial results travel between workgroups on different XCDs, whose L2 caches do not see each other's lines.
+// Device-scope relaxed atomic accesses go past the L2 (the stores write through, the loads fetch from memory), so
+// the exchange needs no device-scope fence - a fence would write back and invalidate the XCD's whole L2, which at
+// that moment holds the K/V tiles the other 31 workgroups of the XCD are working through.
+__device__ __forceinline__ void store_shared_f32(float* ptr, float v) {
+  __hip_atomic_store(reinterpret_cast<uint32_t*>(ptr), __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_shared_f32(const float* ptr) {
+  return __uint_as_float(__hip_atomic_load(reinterpret_cast<const uint32_t*>(ptr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+// This workgroup's number in the order in which the work is handed out: consecutive hardware workgroup numbers go
+// to different XCDs; every XCD gets a contiguous range of the work instead, so that workgroups that share an L2
+// read the same heads.
+__device__ __forceinline__ uint32_t group_number(uint32_t G) {
+  uint32_t b = blockIdx.x;
+  asm volatile("" : "+s"(b));
+  return G % 8 == 0 ? (b & 7) * (G / 8) + (b >> 3) : b;
+}
+__device__ __forceinline__ uint32_t first_unit_of(uint32_t g, uint32_t units, uint32_t G) {
+  return (uint32_t)((uint64_t)g * units / G);
+}
+
+template <bool WIDE>
 __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p) {
+  constexpr int kQueries = WIDE ? 2 * kWgQueries : kWgQueries;  // queries per workgroup
+  constexpr int kHalves = WIDE ? 2 : 1;                          // 64-key tiles a wave works through per iteration
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
   SlotTable& tab = *reinterpret_cast<SlotTable*>(smem + 2 * kStageBytes);
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int l32 = lane & 31, lh = lane >> 5;
-  const int qq = wave & 3, kp = wave >> 2;  // query quarter (32 queries), key parity
-
-  int wg = blockIdx.x;
+  const int n_iter = (int)((p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys);
+  uint32_t share_end;  // end of what is left of this workgroup's share of the units
   {
-    const int total = p.H * p.n_qtiles;
-    if (total % 8 == 0) wg = (wg & 7) * (total / 8) + (wg >> 3);
+    const auto& c = reread_params();
+    share_end = first_unit_of(group_number(c.groups) + 1, c.units, c.groups);
   }
-  const int head = wg / p.n_qtiles, qtile = wg - head * p.n_qtiles;
 
-  if (tid < p.n_slots) {
+  if (const int tid = threadIdx.x; tid < p.n_slots) {
     tab.kv[tid] = reinterpret_cast<const uint8_t*>(p.kv_ptrs[tid]);
     tab.ks[tid] = reinterpret_cast<const uint8_t*>(p.ks_ptrs[tid]);
     tab.vv[tid] = reinterpret_cast<const uint8_t*>(p.vv_ptrs[tid]);
@@ -195,11 +246,38 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     tab.vg[tid] = load_global<float>(reinterpret_cast<const void*>(p.va_ptrs[tid])) * p.inv_denom;
   }
 
+  __syncthreads();
+
+  // A workgroup's share of the units is cut at tile boundaries into segments: iterations [seg_begin, seg_end) of
+  // one tile (head x group of queries).  A segment that is a whole tile ends with the normalised output; the
+  // others leave (O, reference point, row sum) in `partials`, and the workgroup that finishes a tile's last
+  // segment combines them.  The segments are taken from the share's end backwards: a share is typically the
+  // tail of one tile followed by the head of the next, and with the head (keys from 0) first and the tail
+  // (keys up to the end) last, all workgroups of the launch move through the key range together, a few
+  // iterations apart at most, which is what lets those of one head find each other's K/V lines in the L2.
+  for (;;) {
+  int tile_id, seg_begin, seg_end;
   bf16x8 qf[8];
   {
-    int64_t query = (int64_t)qtile * kWgQueries + qq * kWaveQueries + l32;
-    if (query >= p.Lq) query = p.Lq - 1;
-    const uint16_t* src = p.q + (query * p.H + head) * kHeadDim + 8 * lh;
+    const auto& c = reread_params();
+    const uint32_t share_begin = first_unit_of(group_number(c.groups), c.units, c.groups);
+    if (share_end <= share_begin) break;
+    tile_id = (int)((share_end - 1) / (uint32_t)n_iter);
+    const uint32_t tile_first_unit = (uint32_t)tile_id * (uint32_t)n_iter;
+    seg_begin = share_begin > tile_first_unit ? (int)(share_begin - tile_first_unit) : 0;
+    seg_end = (int)(share_end - tile_first_unit);
+    share_end = tile_first_unit + (uint32_t)seg_begin;
+  }
+  const int head = tile_id / p.n_qtiles, qtile = tile_id - head * p.n_qtiles;
+  // The thread's coordinates, derived anew in every segment (see fresh_thread_index).
+  const int tid = fresh_thread_index(), lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, lh = lane >> 5;
+  const int qq = WIDE ? wave : (wave & 3), kp = WIDE ? 0 : (wave >> 2);  // group of 32 queries, key parity
+  {
+    const auto& c = reread_params();
+    int64_t query = (int64_t)qtile * kQueries + qq * kWaveQueries + l32;
+    if (query >= c.Lq) query = c.Lq - 1;
+    const uint16_t* src = c.q + (query * p.H + head) * kHeadDim + 8 * lh;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) qf[ks] = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(src + 16 * ks));
   }
@@ -210,9 +288,6 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
 #pragma unroll
     for (int i = 0; i < 16; ++i) o[dt][i] = 0.0f;
   float m_run = -INFINITY, l_run = 0.0f;
-
-  const int n_iter = (int)((p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys);
-  __syncthreads();
 
   // ---- decode plan.  Thread = (key_local = tid / 4, quarter of the head dim = tid % 4), the same for K and V.
   // Schedule of iteration `it`: the MFMAs work on LDS stage it & 1 while the raw FP4 bytes of iteration
@@ -229,8 +304,8 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   const uint32_t step_so = (uint32_t)p.H * 1024u;
   const int k_dst_off = (k_local >> 6) * kKTileBytes + (k_local & 63) * kKPitch + k_quarter * 64;
   const int v_dst_off = 2 * kKTileBytes + (k_local >> 6) * kVTileBytes + (k_local & 63) * kVPitch + k_quarter * 64;
-  int iter_base = 0;
-  int k_slot = k_local / p.bts, k_off = k_local - k_slot * p.bts;
+  int iter_base = seg_begin * kIterKeys;
+  int k_slot = (iter_base + k_local) / p.bts, k_off = iter_base + k_local - k_slot * p.bts;
   uint32_t k_vo, k_so;
   float k_gs, v_gs;  // slot scale amax * f32(1 / (e2m1_max * e4m3_max)) of the thread's key, for K and for V
   auto locate = [&]() __attribute__((always_inline)) {
@@ -279,6 +354,24 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   // register r of tile kt <-> key 32 kt + 8 (r / 4) + 4 lh + r % 4), then the PV phase in four steps of 16
   // keys, the exponentials of step j + 1 computed under the four MFMAs of step j.
   auto softmax_pv = [&](float16v (&sc)[2], const uint8_t* vt_base) __attribute__((always_inline)) {
+    // V^T fragment of step `step` (16 keys), head-dim tile dt: lane l needs column d = 32 dt + l % 32 for the keys
+    // 16 step + 8 j + 4 (l / 32) + 0..3 (j = 0, 1: the order of P's registers).  One transposing read serves a
+    // 16-lane group: source lane i points at row key0 + i / 4, columns d0 + 4 (i % 4) .. + 3, and every lane of
+    // the group receives column d0 + i of the four rows.
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) bf16x4* lds_bf16x4_t;
+    const uint8_t* vt_lane = vt_base + (4 * lh + ((lane & 15) >> 2)) * kVPitch + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+    auto read_v = [&](int step, bf16x4 (&dst)[4][2]) __attribute__((always_inline)) {
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          dst[dt][j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
+              (lds_bf16x4_t)(vt_lane + (16 * step + 8 * j) * kVPitch + dt * 64));
+    };
+    bf16x4 vfr[2][4][2];
+    read_v(0, vfr[0]);
+    __builtin_amdgcn_sched_barrier(0);
     float neg;
     {
       float mx = sc[0][0];
@@ -313,29 +406,16 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       }
       dst = __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
     };
-    // V^T fragment of step `step` (16 keys), head-dim tile dt: lane l needs column d = 32 dt + l % 32 for the keys
-    // 16 step + 8 j + 4 (l / 32) + 0..3 (j = 0, 1: the order of P's registers).  One transposing read serves a
-    // 16-lane group: source lane i points at row key0 + i / 4, columns d0 + 4 (i % 4) .. + 3, and every lane of
-    // the group receives column d0 + i of the four rows.
-    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
-    typedef __attribute__((address_space(3))) bf16x4* lds_bf16x4_t;
-    const uint8_t* vt_lane = vt_base + (4 * lh + ((lane & 15) >> 2)) * kVPitch + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-    auto read_v = [&](int step, bf16x4 (&dst)[4][2]) __attribute__((always_inline)) {
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          dst[dt][j] = __builtin_amdgcn_ds_read_tr16_b64_v4bf16(
-              (lds_bf16x4_t)(vt_lane + (16 * step + 8 * j) * kVPitch + dt * 64));
-    };
+    // The scheduling barriers keep every LDS read where it is written: a whole step ahead of the MFMAs that use
+    // it.  Left alone, the compiler moves each read down to just ahead of its MFMA to shorten register live
+    // ranges, and the wave then sits out the LDS latency a dozen times per tile.
     bf16x8 pb[2];
-    bf16x4 vfr[2][4][2];
-    read_v(0, vfr[0]);
     make_p(0, pb[0]);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int step = 0; step < 4; ++step) {
       if (step < 3) read_v(step + 1, vfr[(step + 1) & 1]);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt) {
         const bf16x4(&v)[2] = vfr[step & 1][dt];
@@ -351,15 +431,16 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
           __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);  // their multiply-adds, sums and packing
         }
       }
+      __builtin_amdgcn_sched_barrier(0);
     }
     l_run += sum;
   };
 
-  // prologue: stage 0 <- iteration 0, raw registers <- iteration 1
+  // prologue: the segment's first iteration into its stage, raw registers <- the second one
   fetch_next();
-  decode_any(0);
+  decode_any(seg_begin & 1);
   advance();
-  if (n_iter > 1) fetch_next();
+  if (seg_begin + 1 < seg_end) fetch_next();
   __syncthreads();
   // Every load issued so far (Q fragments, first tiles) has to have landed before the loop: otherwise the
   // compiler's wait-count bookkeeping carries them into the loop and makes the MFMA phase wait for the
@@ -371,67 +452,74 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   // also converting one dword of the prefetched K row (even steps) or V row (odd steps) into the other LDS
   // stage.  The rest (the bf16 chunk, the tail) runs the plain
   // body in a loop of its own.
-  int n_fast = n_cached / kIterKeys - 1;
-  n_fast = n_fast < 0 ? 0 : (n_fast > n_iter ? n_iter : n_fast);
-  int it = 0;
+  const int n_fast = min(n_cached / kIterKeys, seg_end) - 1;
+  int it = seg_begin;
   for (; it < n_fast; ++it) {
     const uint8_t* cur = smem + (it & 1) * kStageBytes;
     uint8_t* nxt = smem + ((it + 1) & 1) * kStageBytes;
-    const uint8_t* vt_base = cur + 2 * kKTileBytes + kp * kVTileBytes;
-    const bool has_next2 = it + 2 < n_iter;
-    float16v sc[2];
-    {
-      const uint32_t wk[4] = {kf.v.x, kf.v.y, kf.v.z, kf.v.w}, wv[4] = {vf.v.x, vf.v.y, vf.v.z, vf.v.w};
-      half2v ks2[2], vs2[2];
-      block_scales_f16(kf.scales, ks2);
-      block_scales_f16(vf.scales, vs2);
-      uint8_t* kdst = nxt + k_dst_off;
-      uint8_t* vdst = nxt + v_dst_off;
-      const uint8_t* krow0 = cur + kp * kKTileBytes + l32 * kKPitch + lh * 16;
+    const bool has_next2 = it + 2 < seg_end;
+    const uint32_t wk[4] = {kf.v.x, kf.v.y, kf.v.z, kf.v.w}, wv[4] = {vf.v.x, vf.v.y, vf.v.z, vf.v.w};
+    half2v ks2[2], vs2[2];
+    block_scales_f16(kf.scales, ks2);
+    block_scales_f16(vf.scales, vs2);
+    uint8_t* kdst = nxt + k_dst_off;
+    uint8_t* vdst = nxt + v_dst_off;
+#pragma unroll
+    for (int h = 0; h < kHalves; ++h) {
+      const int tile = WIDE ? h : kp;
+      float16v sc[2];
+      const uint8_t* krow0 = cur + tile * kKTileBytes + l32 * kKPitch + lh * 16;
       const uint8_t* krow1 = krow0 + 32 * kKPitch;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) sc[kt][i] = 0.0f;
-      uint4 a0 = *reinterpret_cast<const uint4*>(krow0), a1 = *reinterpret_cast<const uint4*>(krow1);
+      // K fragments two steps ahead of their MFMAs, three sets in rotation, held in place by scheduling barriers.
+      uint4 fk[3][2];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        fk[ks][0] = *reinterpret_cast<const uint4*>(krow0 + ks * 32);
+        fk[ks][1] = *reinterpret_cast<const uint4*>(krow1 + ks * 32);
+      }
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
-        uint4 n0 = a0, n1 = a1;
-        if (ks < 7) {
-          n0 = *reinterpret_cast<const uint4*>(krow0 + (ks + 1) * 32);
-          n1 = *reinterpret_cast<const uint4*>(krow1 + (ks + 1) * 32);
+        if (ks < 6) {
+          fk[(ks + 2) % 3][0] = *reinterpret_cast<const uint4*>(krow0 + (ks + 2) * 32);
+          fk[(ks + 2) % 3][1] = *reinterpret_cast<const uint4*>(krow1 + (ks + 2) * 32);
         }
-        const bf16x8 fa0 = __builtin_bit_cast(bf16x8, a0), fa1 = __builtin_bit_cast(bf16x8, a1);
+        __builtin_amdgcn_sched_barrier(0);
+        const bf16x8 fa0 = __builtin_bit_cast(bf16x8, fk[ks % 3][0]), fa1 = __builtin_bit_cast(bf16x8, fk[ks % 3][1]);
         sc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, qf[ks], sc[0], 0, 0, 0);
         sc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, qf[ks], sc[1], 0, 0, 0);
-        {  // one dword (8 elements) of the prefetched row per step: K in the even steps, V in the odd ones
+        // One dword (8 elements) of the prefetched rows at a time.  One tile per wave: K in the even steps, V in the
+        // odd ones.  Two tiles per wave: every second step, K under the first tile's MFMAs and V under the second's.
+        if (!WIDE || (ks & 1) == 0) {
           const int j = ks >> 1;
-          const bool is_k = (ks & 1) == 0;
+          const bool is_k = WIDE ? h == 0 : (ks & 1) == 0;
           float v8[8];
           fp4x8_to_f32(is_k ? wk[j] : wv[j], is_k ? ks2[j >> 1] : vs2[j >> 1], is_k ? k_gs : v_gs, v8);
           reinterpret_cast<uint4*>(is_k ? kdst : vdst)[j] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
                                                                        pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
         }
-        a0 = n0;
-        a1 = n1;
+        __builtin_amdgcn_sched_barrier(0);
       }
+      if (h == kHalves - 1) {
+        advance();
+        if (has_next2) fetch_next();
+      }
+      softmax_pv(sc, cur + 2 * kKTileBytes + tile * kVTileBytes);
     }
-    advance();
-    if (has_next2) fetch_next();
-    softmax_pv(sc, vt_base);
     __syncthreads();
   }
 
   // Plain body: the S phase without interleaved conversion, masking in the last tile, and the successor tile
   // decoded after the MFMAs (or, for the chunk's own bf16 tiles, brought in ahead of them).
-  for (; it < n_iter; ++it) {
+  for (; it < seg_end; ++it) {
     const uint8_t* cur = smem + (it & 1) * kStageBytes;
-    const uint8_t* vt_base = cur + 2 * kKTileBytes + kp * kVTileBytes;
-    const int tile_base = it * kIterKeys + kp * kTileKeys;
     // A successor that lies wholly in the bf16 chunk is brought in ahead of the MFMAs: its K rows go
     // and V rows go straight from global memory into the other stage (one 256-byte row per wave instruction,
     // 16 rows of each per wave).
-    const bool next_is_chunk = iter_base >= n_cached && iter_base + kIterKeys <= Lk_i;  // iter_base = first key of tile it + 1
+    const bool next_is_chunk = it + 1 < seg_end && iter_base >= n_cached && iter_base + kIterKeys <= Lk_i;  // iter_base = first key of tile it + 1
     if (next_is_chunk) {
       uint8_t* nxt = smem + ((it + 1) & 1) * kStageBytes;
       const int64_t src_off = ((int64_t)(iter_base + wave * 16 - n_cached) * p.H + head) * kHeadDim + lane * 2;
@@ -445,20 +533,34 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
         load_to_lds_b32(p.v_new + src_off + r * src_step, vdst_lds + r * kVPitch);
       }
     }
-    if (tile_base < Lk_i) {
+#pragma unroll 1
+    for (int h = 0; h < kHalves; ++h) {
+      const int tile = WIDE ? h : kp;
+      const int tile_base = it * kIterKeys + tile * kTileKeys;
+      if (tile_base >= Lk_i) break;
       float16v sc[2];
-      const uint8_t* krow0 = cur + kp * kKTileBytes + l32 * kKPitch + lh * 16;
+      const uint8_t* krow0 = cur + tile * kKTileBytes + l32 * kKPitch + lh * 16;
       const uint8_t* krow1 = krow0 + 32 * kKPitch;
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) sc[kt][i] = 0.0f;
+      uint4 fk[3][2];  // K fragments two steps ahead, as in the loop above
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        fk[ks][0] = *reinterpret_cast<const uint4*>(krow0 + ks * 32);
+        fk[ks][1] = *reinterpret_cast<const uint4*>(krow1 + ks * 32);
+      }
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
-        const bf16x8 fa0 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow0 + ks * 32));
-        const bf16x8 fa1 = __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(krow1 + ks * 32));
-        sc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa0, qf[ks], sc[0], 0, 0, 0);
-        sc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa1, qf[ks], sc[1], 0, 0, 0);
+        if (ks < 6) {
+          fk[(ks + 2) % 3][0] = *reinterpret_cast<const uint4*>(krow0 + (ks + 2) * 32);
+          fk[(ks + 2) % 3][1] = *reinterpret_cast<const uint4*>(krow1 + (ks + 2) * 32);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        sc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fk[ks % 3][0]), qf[ks], sc[0], 0, 0, 0);
+        sc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fk[ks % 3][1]), qf[ks], sc[1], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
       }
       if (tile_base + kTileKeys > Lk_i) {
 #pragma unroll
@@ -469,78 +571,278 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
             if (key >= Lk_i) sc[kt][r] = -INFINITY;
           }
       }
-      softmax_pv(sc, vt_base);
+      softmax_pv(sc, cur + 2 * kKTileBytes + tile * kVTileBytes);
     }
     if (next_is_chunk) {
       iter_base += kIterKeys;  // the slot bookkeeping of advance() has no use beyond the cache
       __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): the rows have landed in LDS
-    } else if (it + 1 < n_iter) {
+    } else if (it + 1 < seg_end) {
       decode_any((it + 1) & 1);
       advance();
-      if (it + 2 < n_iter) fetch_next();
+      if (it + 2 < seg_end) fetch_next();
     }
     __syncthreads();
   }
 
-  // ---- merge the two key-parity halves and write out.  Row sums are per wave half so far.
-  l_run += __shfl_xor(l_run, 32, 64);
-  float* xo = reinterpret_cast<float*>(smem);   // [qq][64 regs][64 lanes]
-  float* xm = xo + 4 * 64 * 64;                  // [qq][64]
-  float* xl = xm + 4 * 64;
-  if (kp == 1) {
+  l_run += __shfl_xor(l_run, 32, 64);  // row sums were per wave half so far
+  {  // epilogue of the segment, with its own copies of the thread's coordinates (see fresh_thread_index)
+  const auto& c = reread_params();
+  const int tid = fresh_thread_index(), lane = tid & 63, wave = tid >> 6, l32 = lane & 31, lh = lane >> 5;
+  const int qq = WIDE ? wave : (wave & 3), kp = WIDE ? 0 : (wave >> 2);
+  if constexpr (WIDE) {
+    // Every wave has seen its segment of the key range for its 32 queries.
+    bool write_out = true;
+    if (seg_begin != 0 || seg_end != n_iter) {
+      // Part of a tile.  Whoever arrives last at a tile combines the parts; the others leave their state in a
+      // record (two records per workgroup: one for the first tile it touches, one for the last) and count
+      // their arrival.  The parts are combined from the end of the key range backwards whoever does it, so
+      // the result does not depend on the order of arrival.  The workgroup that holds the last part is
+      // normally also the last to arrive (the segments are walked backwards, see above): if a look at the
+      // counter shows that, it goes on from its registers without writing a record.
+      const uint32_t G = c.groups, units = c.units, wg = group_number(G);
+      auto record_of = [&](uint32_t g) {
+        const int first_tile = (int)(first_unit_of(g, units, G) / (uint32_t)n_iter);
+        return c.partials + (size_t)(2 * g + (first_tile == tile_id ? 0 : 1)) * kPartialFloats + wave * (66 * 64) + lane;
+      };
+      const uint32_t tile_first_unit = (uint32_t)tile_id * (uint32_t)n_iter;
+      const uint32_t g_first = (uint32_t)((((uint64_t)tile_first_unit + 1) * G - 1) / units);
+      const uint32_t g_last = (uint32_t)((((uint64_t)tile_first_unit + (uint32_t)n_iter) * G - 1) / units);
+      const int others = (int)(g_last - g_first);
+      if (tid == 0)
+        tab.last_arrival = wg == g_last && __hip_atomic_load(c.arrivals + tile_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
+      __syncthreads();
+      const bool from_registers = tab.last_arrival != 0;
+      write_out = from_registers;
+      if (!from_registers) {
+        float* mine = record_of(wg);
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-      for (int i = 0; i < 16; ++i) xo[(qq * 64 + dt * 16 + i) * 64 + lane] = o[dt][i];
-    xm[qq * 64 + lane] = m_run;
-    xl[qq * 64 + lane] = l_run;
-  }
-  __syncthreads();
-  if (kp == 0) {
-    float out_max = 0.0f;
-    const float m1 = xm[qq * 64 + lane], l1 = xl[qq * 64 + lane];
-    const float m = fmaxf(m_run, m1);
-    const float a0 = __builtin_amdgcn_exp2f((m_run - m) * p.scale_log2);
-    const float a1 = (m1 == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m1 - m) * p.scale_log2);
-    const float inv_l = 1.0f / (l_run * a0 + l1 * a1);
-    const int64_t query = (int64_t)qtile * kWgQueries + qq * kWaveQueries + l32;
-    if (query < p.Lq) {
-      uint16_t* dst = p.out + (query * p.H + head) * kHeadDim;
+          for (int i = 0; i < 16; ++i) store_shared_f32(mine + (dt * 16 + i) * 64, o[dt][i]);
+        store_shared_f32(mine + 64 * 64, m_run);
+        store_shared_f32(mine + 65 * 64, l_run);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the stores have left before the arrival is counted
+        __syncthreads();
+        if (tid == 0)
+          tab.last_arrival = __hip_atomic_fetch_add(c.arrivals + tile_id, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
+        __syncthreads();
+        write_out = tab.last_arrival != 0;
+      }
+      if (write_out) {
+        if (tid == 0) __hip_atomic_store(c.arrivals + tile_id, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+        if (!from_registers) {  // start from nothing; the first step below turns that into the last part exactly
+          m_run = -INFINITY;
+          l_run = 0.0f;
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[dt][i] = 0.0f;
+        }
+        for (int g = (int)g_last - (from_registers ? 1 : 0); g >= (int)g_first; --g) {
+          const float* theirs = record_of((uint32_t)g);
+          const float m1 = load_shared_f32(theirs + 64 * 64), l1 = load_shared_f32(theirs + 65 * 64);
+          const float m = fmaxf(m_run, m1);
+          const float a0 = (m_run == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m_run - m) * p.scale_log2);
+          const float a1 = (m1 == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m1 - m) * p.scale_log2);
+          l_run = l_run * a0 + l1 * a1;
+          m_run = m;
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[dt][i] = o[dt][i] * a0 + load_shared_f32(theirs + (dt * 16 + i) * 64) * a1;
+        }
+      }
+    }
+    if (write_out) {
+      float out_max = 0.0f;
+      const float inv_l = 1.0f / l_run;
+      const int64_t query = (int64_t)qtile * kQueries + qq * kWaveQueries + l32;
+      if (query < c.Lq) {
+        uint16_t* dst = c.out + (query * p.H + head) * kHeadDim;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg) {
+            const uint2 packed = make_uint2(pack_bf16(o[dt][4 * rg] * inv_l, o[dt][4 * rg + 1] * inv_l),
+                                            pack_bf16(o[dt][4 * rg + 2] * inv_l, o[dt][4 * rg + 3] * inv_l));
+            *reinterpret_cast<uint2*>(dst + dt * 32 + 8 * rg + 4 * lh) = packed;
+            out_max = abs_max_bf16x8(make_uint4(packed.x, packed.y, 0u, 0u), out_max);
+          }
+      }
+      if (c.sink.parts) {
+        out_max = wave_max(out_max);
+        if (lane == 0) amax_sink_update(AmaxSink{c.sink.parts, c.sink.epoch}, (uint32_t)tile_id * 8 + wave, out_max);
+      }
+    }
+  } else {
+    // ---- merge the two key-parity halves through LDS and write out.
+    float* xo = reinterpret_cast<float*>(smem);   // [qq][64 regs][64 lanes]
+    float* xm = xo + 4 * 64 * 64;                  // [qq][64]
+    float* xl = xm + 4 * 64;
+    if (kp == 1) {
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          float v[4];
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const float o1 = xo[(qq * 64 + dt * 16 + 4 * rg + i) * 64 + lane];
-            v[i] = (o[dt][4 * rg + i] * a0 + o1 * a1) * inv_l;
-          }
-          const int d = dt * 32 + 8 * rg + 4 * lh;
-          const uint2 packed = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
-          *reinterpret_cast<uint2*>(dst + d) = packed;
-          out_max = abs_max_bf16x8(make_uint4(packed.x, packed.y, 0u, 0u), out_max);
-        }
+        for (int i = 0; i < 16; ++i) xo[(qq * 64 + dt * 16 + i) * 64 + lane] = o[dt][i];
+      xm[qq * 64 + lane] = m_run;
+      xl[qq * 64 + lane] = l_run;
     }
-    if (p.sink.parts) {
-      out_max = wave_max(out_max);
-      if (lane == 0) amax_sink_update(p.sink, blockIdx.x * 4 + qq, out_max);
+    __syncthreads();
+    if (kp == 0) {
+      float out_max = 0.0f;
+      const float m1 = xm[qq * 64 + lane], l1 = xl[qq * 64 + lane];
+      const float m = fmaxf(m_run, m1);
+      const float a0 = __builtin_amdgcn_exp2f((m_run - m) * p.scale_log2);
+      const float a1 = (m1 == -INFINITY) ? 0.0f : __builtin_amdgcn_exp2f((m1 - m) * p.scale_log2);
+      const float inv_l = 1.0f / (l_run * a0 + l1 * a1);
+      const int64_t query = (int64_t)qtile * kQueries + qq * kWaveQueries + l32;
+      if (query < c.Lq) {
+        uint16_t* dst = c.out + (query * p.H + head) * kHeadDim;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg) {
+            float v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const float o1 = xo[(qq * 64 + dt * 16 + 4 * rg + i) * 64 + lane];
+              v[i] = (o[dt][4 * rg + i] * a0 + o1 * a1) * inv_l;
+            }
+            const int d = dt * 32 + 8 * rg + 4 * lh;
+            const uint2 packed = make_uint2(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]));
+            *reinterpret_cast<uint2*>(dst + d) = packed;
+            out_max = abs_max_bf16x8(make_uint4(packed.x, packed.y, 0u, 0u), out_max);
+          }
+      }
+      if (c.sink.parts) {
+        out_max = wave_max(out_max);
+        if (lane == 0) amax_sink_update(AmaxSink{c.sink.parts, c.sink.epoch}, (uint32_t)tile_id * 4 + qq, out_max);
+      }
     }
   }
+  }
+  __syncthreads();  // the stages (and the merge area) are free for the next segment
+  }  // segments
 }
 
+// Memory for the partial results of a launch that splits tiles between workgroups: one set per (device, stream),
+// created at the first such launch there, grown when a later launch needs more, never released.  Launches on one
+// stream run one after the other, so they can share a set; launches on different streams get different sets.
+struct SplitWorkspace {
+  float* partials = nullptr;
+  int* arrivals = nullptr;
+  uint32_t groups = 0;
+  int tiles = 0;
+};
+static std::mutex g_split_mutex;
+static std::map<std::pair<int, hipStream_t>, SplitWorkspace> g_split_workspaces;
+
+static int split_workspace(int dev, hipStream_t stream, uint32_t groups, int tiles, SplitWorkspace& out) {
+  std::lock_guard<std::mutex> lock(g_split_mutex);
+  SplitWorkspace& w = g_split_workspaces[{dev, stream}];
+  if (w.groups < groups || w.tiles < tiles) {
+    if (w.partials) (void)hipFree(w.partials);  // waits for the launches that still use it
+    if (w.arrivals) (void)hipFree(w.arrivals);
+    w = SplitWorkspace{};
+    const int want_tiles = tiles < 1024 ? 1024 : tiles;
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&w.partials), (size_t)2 * groups * kPartialFloats * sizeof(float));
+    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&w.arrivals), (size_t)want_tiles * sizeof(int));
+    if (e == hipSuccess) e = hipMemsetAsync(w.arrivals, 0, (size_t)want_tiles * sizeof(int), stream);
+    if (e != hipSuccess) {
+      set_error("ll_kv_attention: cannot set up %zu bytes for partial results: %s",
+                (size_t)2 * groups * kPartialFloats * sizeof(float), hipGetErrorString(e));
+      if (w.partials) (void)hipFree(w.partials);
+      if (w.arrivals) (void)hipFree(w.arrivals);
+      w = SplitWorkspace{};
+      return LL_ELAUNCH;
+    }
+    w.groups = groups;
+    w.tiles = want_tiles;
+  }
+  out = w;
+  return LL_OK;
+}
+
+static std::atomic<int> g_attention_policy{LL_ATTENTION_AUTO};
+
+static int compute_units_of(int dev, int& cus) {
+  static std::atomic<int> cached[64];
+  if (dev >= 0 && dev < 64 && (cus = cached[dev].load(std::memory_order_relaxed)) > 0) return LL_OK;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
+    set_error("ll_kv_attention: cannot read the number of compute units of device %d", dev);
+    return LL_ELAUNCH;
+  }
+  if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
+  return LL_OK;
+}
+
+// Three ways to run a launch, all one workgroup per compute unit at a time (LDS):
+//  * 128 queries per workgroup, the key range halved between two sets of waves; one workgroup per tile;
+//  * 256 queries per workgroup (every decoded K/V tile serves twice as many MFMAs: an iteration takes about 1.64
+//    times as long for twice the work), one workgroup per tile;
+//  * 256 queries per workgroup, the (tile, iteration) sequence cut into one equal share per compute unit, tiles
+//    that straddle two shares combined by the workgroup that finishes last.
+// The costs below are in iterations of the first kind; whole rounds of workgroups count in full.
 static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
   AttnParams p = p_in;
-  p.n_qtiles = (int)((p.Lq + kWgQueries - 1) / kWgQueries);
   const size_t smem = 2 * kStageBytes + sizeof(SlotTable);
-  static std::atomic<uint64_t> lds_allowed{0};
-  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&kv_attention_kernel), smem, lds_allowed, "ll_kv_attention")) return rc;
-  hipLaunchKernelGGL(kv_attention_kernel, dim3((unsigned)(p.H * p.n_qtiles)), dim3(kAttnThreads), smem, stream, p);
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    set_error("ll_kv_attention: hipGetDevice failed");
+    return LL_ELAUNCH;
+  }
+  if (int rc = compute_units_of(dev, cus)) return rc;
+  const int64_t n_iter = (p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys;
+  const int64_t tiles_narrow = p.H * ((p.Lq + kWgQueries - 1) / kWgQueries);
+  const int64_t tiles_wide = p.H * ((p.Lq + 2 * kWgQueries - 1) / (2 * kWgQueries));
+  constexpr double kWideIteration = 1.64, kCombine = 6.0;
+  const double cost_narrow = (double)((tiles_narrow + cus - 1) / cus * n_iter);
+  const double cost_wide = kWideIteration * (double)((tiles_wide + cus - 1) / cus * n_iter);
+  const double cost_split = kWideIteration * (double)((tiles_wide * n_iter + cus - 1) / cus) + kCombine;
+  int mode = cost_narrow <= cost_wide && cost_narrow <= cost_split ? 0 : (cost_wide <= cost_split ? 1 : 2);
+  LL_REQUIRE(tiles_narrow * n_iter < (1ll << 32), "ll_kv_attention: too many (tile, iteration) units");
+  if (tiles_wide * n_iter >= (1ll << 31)) mode = 0;
+  if (const int policy = g_attention_policy.load(std::memory_order_relaxed); policy != LL_ATTENTION_AUTO) {
+    LL_REQUIRE(policy == LL_ATTENTION_NARROW || tiles_wide * n_iter < (1ll << 31), "ll_kv_attention: too many tiles for the selected policy");
+    mode = policy;
+  }
+
+  if (mode == 0) {
+    p.n_qtiles = (int)((p.Lq + kWgQueries - 1) / kWgQueries);
+    p.units = (uint32_t)(tiles_narrow * n_iter);
+    static std::atomic<uint64_t> lds_allowed{0};
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&kv_attention_kernel<false>), smem, lds_allowed, "ll_kv_attention")) return rc;
+    p.groups = (uint32_t)tiles_narrow;
+    hipLaunchKernelGGL(kv_attention_kernel<false>, dim3(p.groups), dim3(kAttnThreads), smem, stream, p);
+  } else {
+    p.n_qtiles = (int)((p.Lq + 2 * kWgQueries - 1) / (2 * kWgQueries));
+    p.units = (uint32_t)(tiles_wide * n_iter);
+    unsigned groups = (unsigned)tiles_wide;
+    if (mode == 2) {
+      groups = (unsigned)(p.units < (uint32_t)cus ? p.units : (uint32_t)cus);  // no workgroup without a unit
+      SplitWorkspace w;
+      if (int rc = split_workspace(dev, stream, groups, (int)tiles_wide, w)) return rc;
+      p.partials = w.partials;
+      p.arrivals = w.arrivals;
+    }
+    static std::atomic<uint64_t> lds_allowed_w{0};
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&kv_attention_kernel<true>), smem, lds_allowed_w, "ll_kv_attention")) return rc;
+    p.groups = groups;
+    hipLaunchKernelGGL(kv_attention_kernel<true>, dim3(groups), dim3(kAttnThreads), smem, stream, p);
+  }
   LL_CHECK_LAUNCH("kv_attention_kernel");
   return LL_OK;
 }
 
 }  // namespace ll
+
+extern "C" int ll_kv_attention_set_policy(int policy) {
+  LL_REQUIRE(policy >= LL_ATTENTION_AUTO && policy <= LL_ATTENTION_SPLIT, "ll_kv_attention_set_policy: unknown policy %d", policy);
+  ll::g_attention_policy.store(policy);
+  return LL_OK;
+}
+
+extern "C" int ll_kv_attention_get_policy(void) { return ll::g_attention_policy.load(); }
 
 extern "C" int ll_kv_attention(const void* q, int64_t Lq, int num_heads, const uint64_t* k_values_ptrs,
                                const uint64_t* k_scales_ptrs, const uint64_t* k_amax_ptrs,

@@ -573,3 +573,59 @@ def test_kv_dequantize_blocks_every_code_and_scale(gpu):
     assert np.array_equal(bits_of(got16), o.f32_to_bf16(ref32))
     gotf16 = _native.kv_dequantize_blocks(t[0], t[1], t[2], 5, H, T, torch.float16, 6.0, 256.0)[0]
     assert torch.equal(gotf16.cpu(), torch.from_numpy(ref32).half())
+
+
+# --------------------------------------------------------------------------- division of a launch between workgroups
+POLICIES = ["narrow", "wide", "split"]
+
+
+@pytest.mark.parametrize("policy", POLICIES)
+def test_every_work_division_against_the_oracle(gpu, policy):
+    """The three ways a launch is divided between workgroups (one workgroup per 128 queries, per 256 queries, or
+    256-query tiles with the key range cut into one equal share per compute unit and the parts combined), forced
+    one by one.  Shapes: fewer tiles than compute units, so that under "split" every tile has many parts (a single
+    iteration each for Lk = 1500); 320 tiles of two iterations, where a share is the end of one tile, a whole
+    tile and the start of a third; a last tile with fewer than 32 queries; FP4 slots with a partly attended last
+    slot.  Each against the fp64 oracle, and twice for identical bits (the order in which parts arrive must not
+    show)."""
+    with _native.attention_policy(policy):
+        for Lq, Lk, H in [(257, 130, 2), (300, 1500, 3), (700, 900, 2), (2000, 200, 40), (5, 3000, 1)]:
+            q, k, v = _randn((Lq, H, 128), 11), _randn((Lk, H, 128), 12), _randn((Lk, H, 128), 13)
+            got = _native.attention_bf16(q.to(gpu), k.to(gpu), v.to(gpu), 128 ** -0.5)
+            again = _native.attention_bf16(q.to(gpu), k.to(gpu), v.to(gpu), 128 ** -0.5)
+            assert torch.equal(got, again), (policy, Lq, Lk, H)
+            ref = o.attention(q.float().numpy(), k.float().numpy(), v.float().numpy())
+            err = np.abs(got.float().cpu().numpy() - ref).max()
+            assert err <= 2e-2, (policy, Lq, Lk, H, err)
+        test_kernel_accepts_any_number_of_cached_tokens(gpu, 4, 96, 232, 77, 50)
+        test_kernel_accepts_any_number_of_cached_tokens(gpu, 2, 192, 200, 300, 333)
+        test_cache_streaming_against_oracle(gpu, 3, 128, 4, 1, 3)
+        test_attention_reads_cached_values_bit_for_bit(gpu, 384, 100)
+    assert _native.load().ll_kv_attention_get_policy() == -1
+
+
+def test_work_divisions_agree_at_the_benchmark_shape_and_leave_the_same_amax(gpu):
+    """configs[2] (24 heads, 2640 queries, 13200 keys): the automatic choice is the split of 256-query tiles; its
+    output differs from the one-workgroup-per-128-queries result only by the order of fp32 additions, and the
+    amax it leaves in the sink is the maximum of its own output."""
+    H, T = 24, 2640
+    g = torch.Generator().manual_seed(21)
+    cache = kvc.initialize_kv_cache(1, T, 5, H, 128, CFG, gpu)[0]
+    for c in range(4):
+        q, k, v = (torch.randn(1, T, H, 128, generator=g).bfloat16().to(gpu) for _ in range(3))
+        _, (ce, le, info) = kvc.kv_cache_attention(q, k, v, cache, c * T, sink_tokens=T)
+        kvc.apply_cache_update(cache, ce, le, info, CFG)
+    q, k, v = (torch.randn(1, T, H, 128, generator=g).bfloat16().to(gpu) for _ in range(3))
+    outs = {}
+    for policy in ["auto"] + POLICIES:
+        with _native.attention_policy(policy):
+            ticket = _native.amax_ticket(gpu)
+            outs[policy] = kvc.kv_cache_attention(q, k, v, cache, 4 * T, sink_tokens=T, amax_out=ticket)[0]
+            xq = quantize_to_fp4(outs[policy][0].flatten(1), CFG, amax=ticket)
+            assert float(xq.amax) == float(outs[policy].float().abs().max())
+    assert torch.equal(outs["auto"], outs["split"])
+    for policy in ("wide", "split"):
+        assert (outs[policy].float() - outs["narrow"].float()).abs().max().item() <= 4e-3
+    with pytest.raises(ValueError):
+        _native.attention_policy("fastest")
+    assert _native.load().ll_kv_attention_set_policy(7) == -1 and b"unknown policy" in _native.load().ll_last_error()
