@@ -10,8 +10,8 @@ restatement (tests/test_unipc.py): the closed-form schedule for given (steps, sh
 is reproduced exactly by every step; order 1 equals the exponential-integrator (DDIM) formula; the order-2
 corrector is exact for x0 predictions that are polynomials of degree <= 2 in lambda (checked against numerical
 quadrature of the exact solution), which fixes R, b and the phi recurrence; the last step returns the x0
-prediction.  Parity unpinned: the fixed weight 1/2 of the order-2 predictor and of the order-1 corrector
-(:461-463, :603-604) is taken from the reference's text; no independent property determines it.
+prediction; the fixed weight 1/2 of the order-2 predictor and of the order-1 corrector (:461-463, :603-604)
+is the only weight for which the local error of those steps falls like h^3 instead of h^2 (measured by halving h).
 
 The weights are built from closed-form phi functions here, not from the reference's recurrence, so that the
 two formulations check each other.

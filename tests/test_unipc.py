@@ -116,3 +116,36 @@ def test_flow_to_x0_conversion():
     flow = torch.tensor([[0.5, 0.25]], dtype=torch.bfloat16)
     out = convert_flow_pred_to_x0(flow, xt, 0.75)
     assert out.dtype == torch.bfloat16 and torch.equal(out, torch.tensor([[0.625, -2.1875]]).bfloat16())
+
+
+def _sigma_of(lmbda):
+    return 1.0 / (1.0 + math.exp(lmbda))
+
+
+@pytest.mark.parametrize("which", ["predictor_order_2", "corrector_order_1"])
+def test_the_fixed_weight_one_half_is_what_makes_the_step_second_order(which):
+    """The order-2 predictor and the order-1 corrector do not solve for their single weight; the reference
+    writes 1/2 (wan_5b/utils/fm_solvers_unipc.py:461-463, 603-604).  What determines that number: with a
+    difference of two x0 predictions as the only correction term, the local error of a step of size h in lambda
+    falls like h^3 for the weight 1/2 and only like h^2 for any other.  Measured on an x0 prediction that is
+    linear in lambda: halving h divides the error by ~8 for the oracle's step, and by ~4 when the correction
+    term is rescaled to a weight of 0.45 or 0.55."""
+    c0, c1, x_s, lam_s = 0.3, 0.9, 0.21, 0.4
+    m = lambda l: c0 + c1 * (l - lam_s)
+
+    def errors(h):
+        s_prev, s_s, s_t = _sigma_of(lam_s - h), _sigma_of(lam_s), _sigma_of(lam_s + h)
+        exact = _exact_solution(x_s, s_s, s_t, m)
+        first_order = uo.uni_p(x_s, [m(lam_s)], [s_s], s_t, 1)
+        if which == "predictor_order_2":
+            step = uo.uni_p(x_s, [m(lam_s - h), m(lam_s)], [s_prev, s_s], s_t, 2)
+        else:
+            step = uo.uni_c(x_s, [m(lam_s)], [s_s], s_t, m(lam_s + h), 1)
+        correction = step - first_order  # the term that carries the weight 1/2
+        return {w: first_order + correction * (w / 0.5) - exact for w in (0.5, 0.45, 0.55)}
+
+    coarse, fine = errors(0.2), errors(0.1)
+    assert 6.5 < coarse[0.5] / fine[0.5] < 9.5, coarse[0.5] / fine[0.5]
+    for w in (0.45, 0.55):
+        assert 2.8 < coarse[w] / fine[w] < 5.5, (w, coarse[w] / fine[w])
+        assert abs(fine[w]) > 5 * abs(fine[0.5])
