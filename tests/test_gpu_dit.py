@@ -27,14 +27,16 @@ def _rel(a, b):
     return float(np.linalg.norm(a.astype(np.float64) - b.astype(np.float64)) / np.linalg.norm(b.astype(np.float64)))
 
 
-def test_block_against_oracle_with_cache(gpu):
-    """Reduced Wan-shaped block (dim 256, 2 heads x 128, FFN 512; chunk = 2 frames x 64 tokens), two
-    chunks so that the second one attends an FP4 slot.  Tolerance: relative Frobenius 6e-2 on the bf16
+@pytest.mark.parametrize("dim,heads,ffn", [(256, 2, 512), (3072, 24, 14336)])
+def test_block_against_oracle_with_cache(gpu, dim, heads, ffn):
+    """Wan-shaped block, reduced (dim 256, 2 heads x 128, FFN 512) and at the full width of the benchmark model
+    (dim 3072, 24 heads, FFN 14336); chunk = 2 frames x 64 tokens, two chunks so that the second one attends an
+    FP4 slot.  Tolerance: relative Frobenius 6e-2 on the bf16
     block output: attention outputs that differ by ~1e-3 are re-quantized to FP4 three more times
     before the block output, which amplifies the difference (measured 3.4e-2); the stage-wise test
     below carries the tight bounds."""
     torch.manual_seed(0)
-    dim, heads, ffn, F, h, w, T = 256, 2, 512, 2, 8, 8, 16
+    F, h, w, T = 2, 8, 8, 16
     fs, L = h * w, 2 * 8 * 8
     block = DiTBlock(dim, ffn, heads).to(gpu)
     for m in block.modules():
@@ -67,17 +69,19 @@ def test_block_against_oracle_with_cache(gpu):
         cached_v = o.kv_dequantize(vals, sc, am).reshape(L, heads, 128)
 
 
-def test_block_stage_by_stage_against_oracle(gpu):
+@pytest.mark.parametrize("dim,heads,ffn", [(256, 2, 512), (3072, 24, 14336)])
+def test_block_stage_by_stage_against_oracle(gpu, dim, heads, ffn):
     """Every stage of the block forward on the GPU against the oracle's stage fed with the same
     (GPU-produced) input: elementwise stages bit-exact, W4A4 linears <= 1e-3 relative Frobenius,
-    attention <= 2e-2 max-abs."""
+    attention <= 2e-2 max-abs.  Once on a reduced block and once at the full width of the benchmark model
+    (dim 3072, 24 heads, FFN 14336) on 128 tokens."""
     from longlive_amd import _native
     from longlive_amd.utils.adaln import adaln_modulate
     from longlive_amd.utils.quant import k_smooth
     from longlive_amd.utils.rope import rope_apply
 
     torch.manual_seed(0)
-    dim, heads, ffn, F, h, w, T = 256, 2, 512, 2, 8, 8, 16
+    F, h, w, T = 2, 8, 8, 16
     fs, L = h * w, 128
     block = DiTBlock(dim, ffn, heads).to(gpu)
     for m in block.modules():
@@ -96,6 +100,18 @@ def test_block_stage_by_stage_against_oracle(gpu):
     def exact(name, got, ref):
         assert np.array_equal(_f(got).reshape(ref.shape), ref), name
 
+    def one_ulp(name, got, ref):
+        """Reductions over the channel dimension (layer norm, RMS norm) add 3072 terms in another order than
+        numpy does: the fp32 statistics can differ in the last bit, which now and then moves a bf16 result to the
+        neighbouring value.  Bit-exact at dim 256; at full width the bar of the adaLN parity test: <= 3.1e-2 (one
+        bf16 ulp at the largest magnitudes here) on fewer than 5 in 1000."""
+        g_, r_ = _f(got).reshape(ref.shape), ref
+        if dim <= 256:
+            assert np.array_equal(g_, r_), name
+            return
+        diff = np.abs(g_ - r_)
+        assert diff.max() <= 3.1e-2 and (diff > 0).mean() < 5e-3, (name, diff.max(), (diff > 0).mean())
+
     def close(name, got, ref, tol=1e-3):
         assert _rel(_f(got).reshape(ref.shape), ref) <= tol, name
 
@@ -109,12 +125,12 @@ def test_block_stage_by_stage_against_oracle(gpu):
         eo = o.round_bf16(p["modulation"][None] + _f(e0)[0])
         exact("modulation", torch.cat(e, 2), eo)
         y = adaln_modulate(xg, e[1], e[0], fs)
-        exact("adaln1", y, o.adaln_modulate(_f(x)[0], eo[:, 1], eo[:, 0], fs))
+        one_ulp("adaln1", y, o.adaln_modulate(_f(x)[0], eo[:, 1], eo[:, 0], fs))
         sa = block.self_attn
         ql = sa.q(y)
         close("q linear", ql, dit_oracle.linear_w4a4(_f(y)[0], p["self_attn.q.w"], p["self_attn.q.b"]))
         qn = sa.norm_q(ql)
-        exact("q rms", qn, o.rms_norm(_f(ql)[0], p["self_attn.norm_q"]))
+        one_ulp("q rms", qn, o.rms_norm(_f(ql)[0], p["self_attn.norm_q"]))
         kn, vv = sa.norm_k(sa.k(y)), sa.v(y)
         rq = rope_apply(qn.view(L, heads, 128), cos, sin)
         exact("rope q", rq, o.rope_apply(_f(qn).reshape(L, heads, 128), ocs, osn))
