@@ -81,11 +81,22 @@ int ll_nvfp4_quantize_noalloc(const void* x, int64_t M, int64_t K, int64_t ldx, 
  * than all earlier ones (1, 2, 3, ...; clear the buffer before wrapping around), and
  * ll_nvfp4_quantize_from_sink reads the slots of that epoch.  Calls that share a buffer must be ordered
  * (one stream).
+ * Launches recorded into a HIP graph run again with the arguments they were recorded with, the epoch among them,
+ * and would meet their own values of the previous replay.  For those, `epoch_offset` names a device word that
+ * every kernel adds to `epoch` when it runs; the graph starts with ll_amax_epoch_advance, which raises that word
+ * by a step larger than the number of epochs one replay uses, so every replay works with fresh epochs.  A buffer
+ * used this way belongs to the graph (eager launches between replays use another buffer).
  */
 typedef struct ll_amax_sink {
-  uint64_t* parts;   /* device memory, LL_AMAX_PARTS entries, 8-byte aligned */
-  uint32_t epoch;    /* > 0 */
+  uint64_t* parts;              /* device memory, LL_AMAX_PARTS entries, 8-byte aligned */
+  uint32_t epoch;               /* > 0 */
+  const uint32_t* epoch_offset; /* device word added to epoch at run time, or NULL */
 } ll_amax_sink;
+
+/* *epoch_offset += step on the stream (a kernel launch, recordable into a graph); when the sum would come near
+ * 2^32 the word restarts from 0 and the LL_AMAX_PARTS slots of `parts` are cleared.  No counterpart in the
+ * reference. */
+int ll_amax_epoch_advance(uint32_t* epoch_offset, uint32_t step, uint64_t* parts, void* stream);
 
 /* ll_nvfp4_quantize whose tensor amax comes from an amax sink that the producer of x has filled with the
  * same epoch; amax (f32[1]) is written.  The bytes equal those of ll_nvfp4_quantize with amax_given == 0. */

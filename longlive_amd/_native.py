@@ -51,6 +51,7 @@ _SIGNATURES = {
                                      c_void_p, c_int64, c_int, c_float, c_float, c_void_p, c_void_p, c_int64, c_float,
                                      c_void_p, c_void_p, c_void_p]),
     "ll_attention_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_float, c_void_p, c_void_p]),
+    "ll_amax_epoch_advance": (c_int, [c_void_p, ctypes.c_uint32, c_void_p, c_void_p]),
     "ll_kv_attention_set_policy": (c_int, [c_int]),
     "ll_kv_attention_get_policy": (c_int, []),
     "ll_rope_apply": (c_int, [c_void_p, c_int64, c_int, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int64,
@@ -143,24 +144,75 @@ AMAX_PARTS = 1024
 
 class AmaxSinkStruct(ctypes.Structure):
     """struct ll_amax_sink of include/ll_nvfp4.h."""
-    _fields_ = [("parts", c_void_p), ("epoch", ctypes.c_uint32)]
+    _fields_ = [("parts", c_void_p), ("epoch", ctypes.c_uint32), ("epoch_offset", c_void_p)]
 
 
 class AmaxTicket:
     """One use of a device's amax sink: handed to the kernel that writes a tensor (``amax_out=``) and then to
     the quantization of that tensor (``amax=``), which reads the maximum the producer left."""
 
-    __slots__ = ("parts", "epoch", "key")
+    __slots__ = ("parts", "epoch", "key", "offset")
 
-    def __init__(self, parts: torch.Tensor, epoch: int, key=None) -> None:
-        self.parts, self.epoch, self.key = parts, epoch, key
+    def __init__(self, parts: torch.Tensor, epoch: int, key=None, offset: torch.Tensor | None = None) -> None:
+        self.parts, self.epoch, self.key, self.offset = parts, epoch, key, offset
 
     def struct(self) -> AmaxSinkStruct:
-        return AmaxSinkStruct(self.parts.data_ptr(), self.epoch)
+        return AmaxSinkStruct(self.parts.data_ptr(), self.epoch, None if self.offset is None else self.offset.data_ptr())
 
 
-# per device: [sink buffer, last epoch issued, (epoch, stream) of the last producer launch]
+# per sink: [sink buffer, last epoch issued, (epoch, stream) of the last producer launch]; the key of a device's own
+# sink is (device type, index), that of a graph's sink ("graph", id)
 _sinks: dict = {}
+# device key -> the ReplayableAmaxSink whose tickets amax_ticket hands out at the moment
+_active_graph_sinks: dict = {}
+
+
+def _device_key(device: torch.device):
+    index = device.index if device.index is not None else (torch.cuda.current_device() if device.type == "cuda" else 0)
+    return (device.type, index)
+
+
+class ReplayableAmaxSink:
+    """An amax sink for launches that are recorded into a HIP graph and replayed.  A recorded launch runs again
+    with the epoch it was recorded with, so every kernel adds a device word to its epoch, and the first recorded
+    launch (``__enter__``) raises that word by more than the number of tickets one replay uses: every replay
+    works with fresh epochs on a buffer of its own.  Use: create it ahead of the capture (it allocates), then
+
+        with torch.cuda.graph(g, stream=s), sink:
+            y = block(...)
+
+    Inside the ``with`` every ``amax_ticket`` of the device comes from this sink."""
+
+    STEP = 1 << 16  # epochs per replay; a replay may use at most STEP - 1 tickets
+
+    def __init__(self, device) -> None:
+        self.device = torch.device(device)
+        self.parts = torch.zeros(AMAX_PARTS, dtype=torch.int64, device=self.device)
+        self.offset = torch.zeros(1, dtype=torch.int32, device=self.device)
+        self.key = ("graph", id(self))
+        self.entry = [self.parts, 0, None]
+
+    def __enter__(self):
+        dkey = _device_key(self.device)
+        if dkey in _active_graph_sinks:
+            raise RuntimeError("another replayable amax sink is active on this device")
+        self.entry[1], self.entry[2] = 0, None
+        _sinks[self.key] = self.entry
+        _active_graph_sinks[dkey] = self
+        with torch.cuda.device(self.device):
+            _check(load().ll_amax_epoch_advance(self.offset.data_ptr(), self.STEP, self.parts.data_ptr(), _stream()),
+                   "ll_amax_epoch_advance")
+        return self
+
+    def __exit__(self, *exc):
+        del _active_graph_sinks[_device_key(self.device)]
+        if self.entry[1] >= self.STEP:
+            raise RuntimeError(f"{self.entry[1]} amax tickets in one recording; at most {self.STEP - 1} are supported")
+        return False
+
+    def ticket(self) -> "AmaxTicket":
+        self.entry[1] += 1
+        return AmaxTicket(self.parts, self.entry[1], self.key, self.offset)
 
 
 def amax_ticket(device: torch.device) -> AmaxTicket:
@@ -169,8 +221,9 @@ def amax_ticket(device: torch.device) -> AmaxTicket:
     producer launch followed by the quantization(s) of its output, on one stream, with no other producer launch
     in between: a later producer overwrites the slots.  The host side checks this (see ``_check_consumer``)."""
     device = torch.device(device)
-    index = device.index if device.index is not None else (torch.cuda.current_device() if device.type == "cuda" else 0)
-    key = (device.type, index)
+    key = _device_key(device)
+    if key in _active_graph_sinks:
+        return _active_graph_sinks[key].ticket()
     entry = _sinks.get(key)
     if entry is None or entry[1] >= 0xFFFFFFFE:
         entry = [torch.zeros(AMAX_PARTS, dtype=torch.int64, device=device), 0, None]

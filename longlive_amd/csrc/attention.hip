@@ -671,7 +671,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       }
       if (c.sink.parts) {
         out_max = wave_max(out_max);
-        if (lane == 0) amax_sink_update(AmaxSink{c.sink.parts, c.sink.epoch}, (uint32_t)tile_id * 8 + wave, out_max);
+        if (lane == 0) amax_sink_update(AmaxSink{c.sink.parts, c.sink.epoch, c.sink.epoch_offset}, (uint32_t)tile_id * 8 + wave, out_max);
       }
     }
   } else {
@@ -716,7 +716,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       }
       if (c.sink.parts) {
         out_max = wave_max(out_max);
-        if (lane == 0) amax_sink_update(AmaxSink{c.sink.parts, c.sink.epoch}, (uint32_t)tile_id * 4 + qq, out_max);
+        if (lane == 0) amax_sink_update(AmaxSink{c.sink.parts, c.sink.epoch, c.sink.epoch_offset}, (uint32_t)tile_id * 4 + qq, out_max);
       }
     }
   }
@@ -899,10 +899,8 @@ extern "C" int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads, co
   p.v_new = static_cast<const uint16_t*>(v_new);
   p.scale_log2 = softmax_scale * 1.4426950408889634f;
   p.out = static_cast<uint16_t*>(out);
-  if (amax_sink && amax_sink->parts) {
-    p.sink.parts = reinterpret_cast<unsigned long long*>(amax_sink->parts);
-    p.sink.epoch = amax_sink->epoch;
-  }
+  LL_REQUIRE(sink_is_valid(amax_sink), "ll_kv_attention_amax: amax sink needs 8-byte alignment and a non-zero epoch");
+  p.sink = make_sink(amax_sink);
   return launch_attention(p, static_cast<hipStream_t>(stream));
 }
 

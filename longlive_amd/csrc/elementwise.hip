@@ -381,13 +381,8 @@ extern "C" int ll_adaln_modulate_amax(const void* x, int64_t B, int64_t L, int C
                                       int64_t shift_stride_b, int64_t shift_stride_f, int64_t frame_seqlen, float eps,
                                       int add_one_to_scale, void* out, const ll_amax_sink* amax_sink, void* stream) {
   using namespace ll;
-  AmaxSink sink{};
-  if (amax_sink && amax_sink->parts) {
-    LL_REQUIRE((reinterpret_cast<uintptr_t>(amax_sink->parts) & 7) == 0 && amax_sink->epoch != 0,
-               "ll_adaln_modulate_amax: amax sink needs 8-byte alignment and a non-zero epoch");
-    sink.parts = reinterpret_cast<unsigned long long*>(amax_sink->parts);
-    sink.epoch = amax_sink->epoch;
-  }
+  LL_REQUIRE(sink_is_valid(amax_sink), "ll_adaln_modulate_amax: amax sink needs 8-byte alignment and a non-zero epoch");
+  const AmaxSink sink = make_sink(amax_sink);
   LL_REQUIRE(x && scale && shift && out, "ll_adaln_modulate: null pointer");
   LL_REQUIRE(B > 0 && L > 0 && C > 0 && C % 8 == 0 && C <= kMaxRowLength && frame_seqlen > 0 &&
                  L % frame_seqlen == 0,
@@ -423,13 +418,8 @@ extern "C" int ll_layer_norm(const void* x, int64_t rows, int C, const void* wei
   LL_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(weight) | reinterpret_cast<uintptr_t>(bias) |
                reinterpret_cast<uintptr_t>(out)) & 15) == 0,
              "ll_layer_norm: pointers must be 16-byte aligned");
-  AmaxSink sink{};
-  if (amax_sink && amax_sink->parts) {
-    LL_REQUIRE((reinterpret_cast<uintptr_t>(amax_sink->parts) & 7) == 0 && amax_sink->epoch != 0,
-               "ll_layer_norm: amax sink needs 8-byte alignment and a non-zero epoch");
-    sink.parts = reinterpret_cast<unsigned long long*>(amax_sink->parts);
-    sink.epoch = amax_sink->epoch;
-  }
+  LL_REQUIRE(sink_is_valid(amax_sink), "ll_layer_norm: amax sink needs 8-byte alignment and a non-zero epoch");
+  const AmaxSink sink = make_sink(amax_sink);
   const dim3 grid((unsigned)((rows + kRowsPerWg - 1) / kRowsPerWg));
 #define LL_LAUNCH_LN(NCH)                                                                                        \
   hipLaunchKernelGGL(layernorm_kernel<NCH>, grid, dim3(kRowThreads), 0, static_cast<hipStream_t>(stream),        \

@@ -529,12 +529,8 @@ extern "C" int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A
   GemmEpilogue epi{};
   epi.bias = static_cast<const uint16_t*>(bias);
   epi.act = activation;
-  if (epilogue->amax_sink.parts) {
-    LL_REQUIRE((reinterpret_cast<uintptr_t>(epilogue->amax_sink.parts) & 7) == 0 && epilogue->amax_sink.epoch != 0,
-               "ll_nvfp4_gemm_tnt_fused: amax sink needs 8-byte alignment and a non-zero epoch");
-    epi.sink.parts = reinterpret_cast<unsigned long long*>(epilogue->amax_sink.parts);
-    epi.sink.epoch = epilogue->amax_sink.epoch;
-  }
+  LL_REQUIRE(sink_is_valid(&epilogue->amax_sink), "ll_nvfp4_gemm_tnt_fused: amax sink needs 8-byte alignment and a non-zero epoch");
+  epi.sink = make_sink(&epilogue->amax_sink);
   if (epilogue->residual) {
     LL_REQUIRE(N % 8 == 0 && epilogue->ldr % 8 == 0 && epilogue->ldr >= N &&
                    (reinterpret_cast<uintptr_t>(epilogue->residual) & 15) == 0,

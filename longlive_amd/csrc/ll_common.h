@@ -163,11 +163,30 @@ __device__ __forceinline__ float abs_max_bf16x8(const uint4& v, float m) {
 // (The bit patterns of non-negative floats order like unsigned integers.)
 constexpr int kAmaxParts = LL_AMAX_PARTS;
 struct AmaxSink {
-  unsigned long long* parts;  // null: no sink
+  unsigned long long* parts;     // null: no sink
   uint32_t epoch;
+  const uint32_t* epoch_offset;  // device word added to epoch when the kernel runs (launches replayed from a graph), or null
 };
+__device__ __forceinline__ uint32_t amax_sink_epoch(uint32_t epoch, const uint32_t* epoch_offset) {
+  return epoch + (epoch_offset ? *epoch_offset : 0u);
+}
 __device__ __forceinline__ void amax_sink_update(const AmaxSink& sink, uint32_t slot, float v) {
-  atomicMax(sink.parts + (slot & (kAmaxParts - 1)), ((unsigned long long)sink.epoch << 32) | __float_as_uint(v));
+  const uint32_t epoch = amax_sink_epoch(sink.epoch, sink.epoch_offset);
+  atomicMax(sink.parts + (slot & (kAmaxParts - 1)), ((unsigned long long)epoch << 32) | __float_as_uint(v));
+}
+// The kernel-side sink of a caller's ll_amax_sink (null or without a buffer: no sink).
+inline AmaxSink make_sink(const ll_amax_sink* s) {
+  AmaxSink k{};
+  if (s && s->parts) {
+    k.parts = reinterpret_cast<unsigned long long*>(s->parts);
+    k.epoch = s->epoch;
+    k.epoch_offset = s->epoch_offset;
+  }
+  return k;
+}
+inline bool sink_is_valid(const ll_amax_sink* s) {
+  return !s || !s->parts ||
+         ((reinterpret_cast<uintptr_t>(s->parts) & 7) == 0 && s->epoch != 0 && (reinterpret_cast<uintptr_t>(s->epoch_offset) & 3) == 0);
 }
 __device__ __forceinline__ float amax_sink_read(const unsigned long long* parts, uint32_t epoch, int slot) {
   const unsigned long long v = parts[slot];

@@ -366,7 +366,8 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
                                                             const float* __restrict__ parts, int amax_given,
                                                             int64_t total_tiles,
                                                             const unsigned long long* __restrict__ sink_parts,
-                                                            uint32_t sink_epoch) {
+                                                            uint32_t sink_epoch_base,
+                                                            const uint32_t* __restrict__ sink_epoch_offset) {
   __shared__ float s_red[kThreads / 64];
   __shared__ uint32_t s_scales[2][128];  // two staged 512-byte scale tiles in blocked order
   __shared__ ScaleEntry s_tab[128];
@@ -380,6 +381,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
   } else {
     float4 p;
     if (sink_parts) {
+      const uint32_t sink_epoch = amax_sink_epoch(sink_epoch_base, sink_epoch_offset);
       p = make_float4(amax_sink_read(sink_parts, sink_epoch, 4 * threadIdx.x),
                       amax_sink_read(sink_parts, sink_epoch, 4 * threadIdx.x + 1),
                       amax_sink_read(sink_parts, sink_epoch, 4 * threadIdx.x + 2),
@@ -570,7 +572,7 @@ static int quantize_impl(const void* x, int64_t M, int64_t K, int64_t ldx, int r
              (long long)K, (long long)ldx);
   LL_REQUIRE(rule >= 0 && rule <= 4, "ll_nvfp4_quantize: unknown scale rule %d", rule);
   LL_REQUIRE(amax_given || workspace || sink, "ll_nvfp4_quantize: workspace required to compute amax");
-  LL_REQUIRE(!sink || (sink->parts && (reinterpret_cast<uintptr_t>(sink->parts) & 7) == 0 && sink->epoch != 0),
+  LL_REQUIRE(!sink || (sink->parts && sink_is_valid(sink)),
              "ll_nvfp4_quantize_from_sink: amax sink needs an 8-byte aligned buffer and a non-zero epoch");
   LL_REQUIRE((reinterpret_cast<uintptr_t>(values) & 7) == 0 && (reinterpret_cast<uintptr_t>(scales) & 3) == 0,
              "ll_nvfp4_quantize: outputs must be 8-byte (values) / 4-byte (scales) aligned");
@@ -585,6 +587,7 @@ static int quantize_impl(const void* x, int64_t M, int64_t K, int64_t ldx, int r
   }
   const unsigned long long* sink_parts = sink ? reinterpret_cast<const unsigned long long*>(sink->parts) : nullptr;
   const uint32_t sink_epoch = sink ? sink->epoch : 0u;
+  const uint32_t* sink_epoch_offset = sink ? sink->epoch_offset : nullptr;
   const bool generic = (K % 64) != 0 || (ldx % 8) != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0;
   // One workgroup per tile up to what the chip holds at once (the launch is persistent: every workgroup has to be
   // resident from the start, or the ones that wait would run after the others have finished).
@@ -597,10 +600,10 @@ static int quantize_impl(const void* x, int64_t M, int64_t K, int64_t ldx, int r
   do {                                                                                                                  \
     if (generic)                                                                                                        \
       hipLaunchKernelGGL((quantize_kernel<R, true>), grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales,    \
-                         amax, workspace, amax_given, total_tiles, sink_parts, sink_epoch);                            \
+                         amax, workspace, amax_given, total_tiles, sink_parts, sink_epoch, sink_epoch_offset);                            \
     else                                                                                                                \
       hipLaunchKernelGGL((quantize_kernel<R, false>), grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales,   \
-                         amax, workspace, amax_given, total_tiles, sink_parts, sink_epoch);                            \
+                         amax, workspace, amax_given, total_tiles, sink_parts, sink_epoch, sink_epoch_offset);                            \
   } while (0)
   switch (rule) {
     case LL_RULE_STATIC_6: LL_LAUNCH_Q(LL_RULE_STATIC_6); break;
@@ -617,6 +620,28 @@ static int quantize_impl(const void* x, int64_t M, int64_t K, int64_t ldx, int r
 extern "C" int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ldx, int rule, uint8_t* values,
                                  uint8_t* scales, float* amax, int amax_given, float* workspace, void* stream) {
   return quantize_impl(x, M, K, ldx, rule, values, scales, amax, amax_given, workspace, nullptr, stream);
+}
+
+// One workgroup of kAmaxParts threads.  Every thread reads the word before anyone writes it, so all agree on
+// whether the slots have to be cleared.
+__global__ __launch_bounds__(ll::kAmaxParts) void amax_epoch_advance_kernel(uint32_t* epoch_offset, uint32_t step,
+                                                                            unsigned long long* parts) {
+  const uint32_t current = *epoch_offset;
+  __syncthreads();
+  const bool restart = current > 0xE0000000u - step;  // epochs stay clear of 2^32 whatever the base epochs are (< 2^28)
+  if (restart) parts[threadIdx.x] = 0ull;
+  if (threadIdx.x == 0) *epoch_offset = restart ? 0u : current + step;
+}
+
+extern "C" int ll_amax_epoch_advance(uint32_t* epoch_offset, uint32_t step, uint64_t* parts, void* stream) {
+  LL_REQUIRE(epoch_offset && parts && (reinterpret_cast<uintptr_t>(epoch_offset) & 3) == 0 &&
+                 (reinterpret_cast<uintptr_t>(parts) & 7) == 0,
+             "ll_amax_epoch_advance: epoch_offset (4-byte aligned) and parts (8-byte aligned) are required");
+  LL_REQUIRE(step > 0 && step <= (1u << 28), "ll_amax_epoch_advance: step %u outside 1..2^28", step);
+  hipLaunchKernelGGL(amax_epoch_advance_kernel, dim3(1), dim3(ll::kAmaxParts), 0, static_cast<hipStream_t>(stream),
+                     epoch_offset, step, reinterpret_cast<unsigned long long*>(parts));
+  LL_CHECK_LAUNCH("amax_epoch_advance_kernel");
+  return LL_OK;
 }
 
 extern "C" int ll_nvfp4_quantize_from_sink(const void* x, int64_t M, int64_t K, int64_t ldx, int rule,

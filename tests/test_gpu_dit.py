@@ -669,3 +669,57 @@ def test_head_modulation_through_the_adaln_kernel_matches_the_eager_graph(gpu):
         ref = head.head(ln.unflatten(1, (F, fs)) * (1 + em[1]) + em[0])
     assert got.shape == ref.shape == (1, F, fs, 32)
     assert (got.float() - ref.float()).abs().max() <= 2.0 ** -6 * ref.float().abs().max()
+
+
+def test_block_forward_recorded_into_a_graph_replays_bit_for_bit(gpu):
+    """One DiT block forward over an FP4 cache slot recorded into a HIP graph (27 kernels of the library, seven amax
+    tickets) and replayed with new inputs.  A recorded launch runs again with the epoch it was recorded with, so
+    the tickets of the recording come from a ReplayableAmaxSink, whose first recorded launch moves every epoch of
+    the replay past those of the previous one.  Each of four replays - with eager forwards of the same block,
+    which use the device's own sink, and synchronisations in between - must equal the eager result bit for bit;
+    a replay that met stale maxima of an earlier replay would quantize against too large an amax."""
+    from longlive_amd import _native
+
+    torch.manual_seed(0)
+    dim, heads, ffn, F, h, w, T = 256, 2, 512, 2, 8, 8, 16
+    L = F * h * w
+    block = DiTBlock(dim, ffn, heads).to(gpu)
+    block, _ = quantize_model_with_filter(block, ModelQuantizationConfig(), use_default_filtered_modules=True,
+                                          materialize_for_inference=True, verbose=False)
+    cache = kvc.initialize_kv_cache(1, L, 3, heads, 128, KV, gpu)[0]
+    cos0, sin0 = rope_cos_sin(build_rope_angles(128), F, h, w, 0, gpu)
+    cos1, sin1 = rope_cos_sin(build_rope_angles(128), F, h, w, F, gpu)
+    g = torch.Generator().manual_seed(3)
+
+    def inputs(scale):
+        return ((torch.randn(1, L, dim, generator=g) * scale).bfloat16().to(gpu),
+                torch.randn(1, F, 6, dim, generator=g).bfloat16().to(gpu),
+                torch.randn(1, T, dim, generator=g).bfloat16().to(gpu))
+
+    with torch.no_grad():
+        x, e0, ctx = inputs(1.0)  # chunk 0 fills slot 0
+        _, (ce, le, info) = block(x, e0, cos0, sin0, ctx, cache, 0, sink_tokens=L)
+        kvc.apply_cache_update(cache, ce, le, info, KV)
+        cases = [inputs(s) for s in (8.0, 1.0, 0.05, 3.0)]  # amax falls and rises between replays
+        eager = [block(x, e0, cos1, sin1, ctx, cache, L, sink_tokens=L)[0].clone() for x, e0, ctx in cases]
+
+        static = [t.clone() for t in cases[0]]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side), _native.attention_policy("narrow"):  # no allocation inside the recording
+            block(*static[:2], cos1, sin1, static[2], cache, L, sink_tokens=L)
+        torch.cuda.current_stream().wait_stream(side)
+        sink = _native.ReplayableAmaxSink(gpu)
+        graph = torch.cuda.CUDAGraph()
+        with _native.attention_policy("narrow"), torch.cuda.graph(graph, stream=side), sink:
+            y_static = block(*static[:2], cos1, sin1, static[2], cache, L, sink_tokens=L)[0]
+        assert sink.entry[1] >= 5  # the recording used the graph's sink
+        for i, case in enumerate(cases):
+            for dst, src in zip(static, case):
+                dst.copy_(src)
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y_static, eager[i]), i
+            other = block(*cases[(i + 1) % 4][:2], cos1, sin1, cases[(i + 1) % 4][2], cache, L, sink_tokens=L)[0]
+            assert torch.equal(other, eager[(i + 1) % 4])
+            torch.cuda.synchronize()

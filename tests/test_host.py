@@ -39,7 +39,8 @@ def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
     assert lib.ll_nvfp4_gemm_tnt_fused(None, None, None, None, None, None, None, 1.0, 1.0, 1, 1, 128, 128, 64, None,
                                        1, ctypes.byref(gated), None) == -1
     assert b"a gate needs a residual" in lib.ll_last_error()
-    assert ctypes.sizeof(_native.GemmEpilogue) == 72 and ctypes.sizeof(_native.AmaxSinkStruct) == 16
+    assert ctypes.sizeof(_native.GemmEpilogue) == 80 and ctypes.sizeof(_native.AmaxSinkStruct) == 24
+    assert lib.ll_amax_epoch_advance(None, 1, None, None) == -1 and b"epoch_offset" in lib.ll_last_error()
 
 
 def test_noalloc_quantize_refuses_inputs_beyond_its_limit_before_touching_the_gpu():
