@@ -55,9 +55,11 @@ struct AttnParams {
   uint16_t* out;
   AmaxSink sink;  // receives max |out| when sink.parts is not null
   int n_qtiles;
-  // Split of the key range between workgroups (256-query kernel only).  The launch covers `units` = tiles x
-  // iterations; workgroup g of G works through the units [g * units / G, (g + 1) * units / G).  With units =
-  // G * iterations every workgroup owns exactly one tile and `partials` / `arrivals` are not touched.
+  // Division of the launch between its G workgroups.  Workgroup g first runs `whole_rounds` whole tiles (tile
+  // j * G + g in round j).  The tiles behind those (256-query kernel only) are cut into `units` = tiles x
+  // iterations, of which workgroup g works through [g * units / G, (g + 1) * units / G); `partials` /
+  // `arrivals` serve those.  One workgroup per tile is whole_rounds = 1, units = 0.
+  uint32_t whole_rounds;
   uint32_t units;
   uint32_t groups;  // G, the number of workgroups of the launch
   float* partials;  // [2 G] records of kPartialFloats floats
@@ -231,6 +233,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   SlotTable& tab = *reinterpret_cast<SlotTable*>(smem + 2 * kStageBytes);
 
   const int n_iter = (int)((p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys);
+  uint32_t round = 0;  // whole-tile rounds done
   uint32_t share_end;  // end of what is left of this workgroup's share of the units
   {
     const auto& c = reread_params();
@@ -248,8 +251,9 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
 
   __syncthreads();
 
-  // A workgroup's share of the units is cut at tile boundaries into segments: iterations [seg_begin, seg_end) of
-  // one tile (head x group of queries).  A segment that is a whole tile ends with the normalised output; the
+  // After its whole tiles (workgroups that share an XCD run neighbouring tiles of a round side by side, in step
+  // through the key range), a workgroup's share of the units is cut at tile boundaries into segments: iterations
+  // [seg_begin, seg_end) of one tile (head x group of queries).  A segment that is a whole tile ends with the normalised output; the
   // others leave (O, reference point, row sum) in `partials`, and the workgroup that finishes a tile's last
   // segment combines them.  The segments are taken from the share's end backwards: a share is typically the
   // tail of one tile followed by the head of the next, and with the head (keys from 0) first and the tail
@@ -260,13 +264,21 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   bf16x8 qf[8];
   {
     const auto& c = reread_params();
-    const uint32_t share_begin = first_unit_of(group_number(c.groups), c.units, c.groups);
-    if (share_end <= share_begin) break;
-    tile_id = (int)((share_end - 1) / (uint32_t)n_iter);
-    const uint32_t tile_first_unit = (uint32_t)tile_id * (uint32_t)n_iter;
-    seg_begin = share_begin > tile_first_unit ? (int)(share_begin - tile_first_unit) : 0;
-    seg_end = (int)(share_end - tile_first_unit);
-    share_end = tile_first_unit + (uint32_t)seg_begin;
+    if (round < c.whole_rounds) {
+      tile_id = (int)(round * c.groups + group_number(c.groups));
+      seg_begin = 0;
+      seg_end = n_iter;
+      ++round;
+    } else {
+      const uint32_t share_begin = first_unit_of(group_number(c.groups), c.units, c.groups);
+      if (share_end <= share_begin) break;
+      const uint32_t split_tile = (share_end - 1) / (uint32_t)n_iter;
+      const uint32_t tile_first_unit = split_tile * (uint32_t)n_iter;
+      tile_id = (int)(c.whole_rounds * c.groups + split_tile);
+      seg_begin = share_begin > tile_first_unit ? (int)(share_begin - tile_first_unit) : 0;
+      seg_end = (int)(share_end - tile_first_unit);
+      share_end = tile_first_unit + (uint32_t)seg_begin;
+    }
   }
   const int head = tile_id / p.n_qtiles, qtile = tile_id - head * p.n_qtiles;
   // The thread's coordinates, derived anew in every segment (see fresh_thread_index).
@@ -600,16 +612,17 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       // normally also the last to arrive (the segments are walked backwards, see above): if a look at the
       // counter shows that, it goes on from its registers without writing a record.
       const uint32_t G = c.groups, units = c.units, wg = group_number(G);
+      const uint32_t split_tile = (uint32_t)tile_id - c.whole_rounds * G;  // the tile's number among the split ones
       auto record_of = [&](uint32_t g) {
-        const int first_tile = (int)(first_unit_of(g, units, G) / (uint32_t)n_iter);
-        return c.partials + (size_t)(2 * g + (first_tile == tile_id ? 0 : 1)) * kPartialFloats + wave * (66 * 64) + lane;
+        const uint32_t first_tile = first_unit_of(g, units, G) / (uint32_t)n_iter;
+        return c.partials + (size_t)(2 * g + (first_tile == split_tile ? 0 : 1)) * kPartialFloats + wave * (66 * 64) + lane;
       };
-      const uint32_t tile_first_unit = (uint32_t)tile_id * (uint32_t)n_iter;
+      const uint32_t tile_first_unit = split_tile * (uint32_t)n_iter;
       const uint32_t g_first = (uint32_t)((((uint64_t)tile_first_unit + 1) * G - 1) / units);
       const uint32_t g_last = (uint32_t)((((uint64_t)tile_first_unit + (uint32_t)n_iter) * G - 1) / units);
       const int others = (int)(g_last - g_first);
       if (tid == 0)
-        tab.last_arrival = wg == g_last && __hip_atomic_load(c.arrivals + tile_id, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
+        tab.last_arrival = wg == g_last && __hip_atomic_load(c.arrivals + split_tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
       __syncthreads();
       const bool from_registers = tab.last_arrival != 0;
       write_out = from_registers;
@@ -624,12 +637,12 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the stores have left before the arrival is counted
         __syncthreads();
         if (tid == 0)
-          tab.last_arrival = __hip_atomic_fetch_add(c.arrivals + tile_id, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
+          tab.last_arrival = __hip_atomic_fetch_add(c.arrivals + split_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
         __syncthreads();
         write_out = tab.last_arrival != 0;
       }
       if (write_out) {
-        if (tid == 0) __hip_atomic_store(c.arrivals + tile_id, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+        if (tid == 0) __hip_atomic_store(c.arrivals + split_tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
         if (!from_registers) {  // start from nothing; the first step below turns that into the last part exactly
           m_run = -INFINITY;
           l_run = 0.0f;
@@ -798,7 +811,14 @@ static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
   constexpr double kWideIteration = 1.64, kCombine = 6.0;
   const double cost_narrow = (double)((tiles_narrow + cus - 1) / cus * n_iter);
   const double cost_wide = kWideIteration * (double)((tiles_wide + cus - 1) / cus * n_iter);
-  const double cost_split = kWideIteration * (double)((tiles_wide * n_iter + cus - 1) / cus) + kCombine;
+  // Split: whole rounds first, the tiles behind them in equal shares.  A handful of left-over tiles would be cut
+  // into many thin parts each (and combined by a single workgroup): then one whole round joins the split part,
+  // whose shares are a little more than one tile.
+  int64_t whole_rounds = tiles_wide / cus;
+  if (const int64_t left = tiles_wide % cus; left > 0 && left * 4 < cus && whole_rounds > 0) --whole_rounds;
+  const int64_t split_tiles = tiles_wide - whole_rounds * cus;
+  const double cost_split =
+      kWideIteration * (double)(whole_rounds * n_iter + (split_tiles * n_iter + cus - 1) / cus) + kCombine;
   int mode = cost_narrow <= cost_wide && cost_narrow <= cost_split ? 0 : (cost_wide <= cost_split ? 1 : 2);
   LL_REQUIRE(tiles_narrow * n_iter < (1ll << 32), "ll_kv_attention: too many (tile, iteration) units");
   if (tiles_wide * n_iter >= (1ll << 31)) mode = 0;
@@ -807,21 +827,29 @@ static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
     mode = policy;
   }
 
+  // Every workgroup needs a unit of the split part when there are whole rounds too (the parts of a tile are
+  // counted by shares): otherwise run the tiles whole.
+  if (mode == 2 && (split_tiles == 0 || (whole_rounds > 0 && split_tiles * n_iter < cus))) mode = 1;
   if (mode == 0) {
     p.n_qtiles = (int)((p.Lq + kWgQueries - 1) / kWgQueries);
-    p.units = (uint32_t)(tiles_narrow * n_iter);
+    p.whole_rounds = 1;
+    p.units = 0;
     static std::atomic<uint64_t> lds_allowed{0};
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&kv_attention_kernel<false>), smem, lds_allowed, "ll_kv_attention")) return rc;
     p.groups = (uint32_t)tiles_narrow;
     hipLaunchKernelGGL(kv_attention_kernel<false>, dim3(p.groups), dim3(kAttnThreads), smem, stream, p);
   } else {
     p.n_qtiles = (int)((p.Lq + 2 * kWgQueries - 1) / (2 * kWgQueries));
-    p.units = (uint32_t)(tiles_wide * n_iter);
+    p.whole_rounds = 1;
+    p.units = 0;
     unsigned groups = (unsigned)tiles_wide;
-    if (mode == 2) {
-      groups = (unsigned)(p.units < (uint32_t)cus ? p.units : (uint32_t)cus);  // no workgroup without a unit
+    if (mode == 2 && split_tiles > 0) {
+      p.whole_rounds = (uint32_t)whole_rounds;
+      p.units = (uint32_t)(split_tiles * n_iter);
+      // without whole rounds no workgroup may be left without a unit (the parts of a tile are counted by shares)
+      groups = (unsigned)(whole_rounds == 0 && p.units < (uint32_t)cus ? p.units : (uint32_t)cus);
       SplitWorkspace w;
-      if (int rc = split_workspace(dev, stream, groups, (int)tiles_wide, w)) return rc;
+      if (int rc = split_workspace(dev, stream, groups, (int)split_tiles, w)) return rc;
       p.partials = w.partials;
       p.arrivals = w.arrivals;
     }

@@ -585,11 +585,12 @@ def test_every_work_division_against_the_oracle(gpu, policy):
     256-query tiles with the key range cut into one equal share per compute unit and the parts combined), forced
     one by one.  Shapes: fewer tiles than compute units, so that under "split" every tile has many parts (a single
     iteration each for Lk = 1500); 320 tiles of two iterations, where a share is the end of one tile, a whole
-    tile and the start of a third; a last tile with fewer than 32 queries; FP4 slots with a partly attended last
-    slot.  Each against the fp64 oracle, and twice for identical bits (the order in which parts arrive must not
+    tile and the start of a third; 432 tiles of six iterations, which "split" runs as one whole round of 256 and
+    the other 176 tiles in equal shares; a last tile with fewer than 32 queries; FP4 slots with a partly attended
+    last slot.  Each against the fp64 oracle, and twice for identical bits (the order in which parts arrive must not
     show)."""
     with _native.attention_policy(policy):
-        for Lq, Lk, H in [(257, 130, 2), (300, 1500, 3), (700, 900, 2), (2000, 200, 40), (5, 3000, 1)]:
+        for Lq, Lk, H in [(257, 130, 2), (300, 1500, 3), (700, 900, 2), (2000, 200, 40), (5, 3000, 1), (3000, 700, 36)]:
             q, k, v = _randn((Lq, H, 128), 11), _randn((Lk, H, 128), 12), _randn((Lk, H, 128), 13)
             got = _native.attention_bf16(q.to(gpu), k.to(gpu), v.to(gpu), 128 ** -0.5)
             again = _native.attention_bf16(q.to(gpu), k.to(gpu), v.to(gpu), 128 ** -0.5)
