@@ -227,6 +227,13 @@ int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads,
 #define LL_ATTENTION_SPLIT 2
 int ll_kv_attention_set_policy(int policy); /* LL_OK, or LL_EINVAL for an unknown policy */
 int ll_kv_attention_get_policy(void);
+/* What a launch of Lq queries x num_heads heads over n_keys keys would do on a device with `compute_units` CUs
+ * under `policy` (pure host arithmetic, no GPU needed): the division taken (an LL_ATTENTION_SPLIT request falls
+ * back to WIDE when there is nothing to split), the number of workgroups, the whole tiles each of them runs first
+ * and the number of tiles cut into shares behind those.  Lets a caller know ahead of a launch whether it will
+ * take the allocating division.  Output pointers may be NULL. */
+int ll_kv_attention_plan(int64_t Lq, int num_heads, int64_t n_keys, int compute_units, int policy,
+                         int* division, uint32_t* workgroups, uint32_t* whole_rounds, int64_t* split_tiles);
 
 /* Plain bf16 attention (cross-attention to the text context; wan_5b/modules/causal_model.py:197-262):
  * q [Lq,H,128], k/v [Lk,H,128], out [Lq,H,128], no mask. */

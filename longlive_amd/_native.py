@@ -54,6 +54,7 @@ _SIGNATURES = {
     "ll_amax_epoch_advance": (c_int, [c_void_p, ctypes.c_uint32, c_void_p, c_void_p]),
     "ll_kv_attention_set_policy": (c_int, [c_int]),
     "ll_kv_attention_get_policy": (c_int, []),
+    "ll_kv_attention_plan": (c_int, [c_int64, c_int, c_int64, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ll_rope_apply": (c_int, [c_void_p, c_int64, c_int, c_int, c_int64, c_int64, c_void_p, c_void_p, c_int64,
                               c_void_p, c_void_p]),
     "ll_adaln_modulate": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64,
@@ -416,6 +417,20 @@ def attention_bf16(q, k, v, softmax_scale, amax_out=None):
 
 
 ATTENTION_POLICIES = {"auto": -1, "narrow": 0, "wide": 1, "split": 2}
+
+
+def attention_plan(Lq: int, num_heads: int, n_keys: int, compute_units: int = 256, policy: str = "auto") -> dict:
+    """How an attention launch of these sizes would be divided between workgroups on a device with
+    ``compute_units`` CUs (host arithmetic only): division name, workgroups, whole tiles per workgroup and the
+    number of tiles cut into shares."""
+    division, groups, rounds = c_int(), ctypes.c_uint32(), ctypes.c_uint32()
+    split = c_int64()
+    _check(load().ll_kv_attention_plan(Lq, num_heads, n_keys, compute_units, ATTENTION_POLICIES[policy],
+                                       ctypes.byref(division), ctypes.byref(groups), ctypes.byref(rounds),
+                                       ctypes.byref(split)), "ll_kv_attention_plan")
+    names = {v: k for k, v in ATTENTION_POLICIES.items()}
+    return {"division": names[division.value], "workgroups": groups.value, "whole_rounds": rounds.value,
+            "split_tiles": split.value}
 
 
 class attention_policy:

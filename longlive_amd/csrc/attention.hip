@@ -17,6 +17,7 @@
 // a per-lane scalar.  The V^T operand (a lane needs eight consecutive keys of one head-dim column) comes out of
 // the row-major tile through ds_read_b64_tr_b16, the LDS read that transposes 16-bit elements across 16 lanes.
 #include "ll_common.h"
+#include "attention_split.h"
 
 #include <map>
 #include <mutex>
@@ -221,9 +222,6 @@ __device__ __forceinline__ uint32_t group_number(uint32_t G) {
   asm volatile("" : "+s"(b));
   return G % 8 == 0 ? (b & 7) * (G / 8) + (b >> 3) : b;
 }
-__device__ __forceinline__ uint32_t first_unit_of(uint32_t g, uint32_t units, uint32_t G) {
-  return (uint32_t)((uint64_t)g * units / G);
-}
 
 template <bool WIDE>
 __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p) {
@@ -233,11 +231,10 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   SlotTable& tab = *reinterpret_cast<SlotTable*>(smem + 2 * kStageBytes);
 
   const int n_iter = (int)((p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys);
-  uint32_t round = 0;  // whole-tile rounds done
-  uint32_t share_end;  // end of what is left of this workgroup's share of the units
+  WorkCursor at;  // where this workgroup is in its work (attention_split.h)
   {
     const auto& c = reread_params();
-    share_end = first_unit_of(group_number(c.groups) + 1, c.units, c.groups);
+    at = start_of_work(group_number(c.groups), c.groups, c.units);
   }
 
   if (const int tid = threadIdx.x; tid < p.n_slots) {
@@ -264,21 +261,11 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   bf16x8 qf[8];
   {
     const auto& c = reread_params();
-    if (round < c.whole_rounds) {
-      tile_id = (int)(round * c.groups + group_number(c.groups));
-      seg_begin = 0;
-      seg_end = n_iter;
-      ++round;
-    } else {
-      const uint32_t share_begin = first_unit_of(group_number(c.groups), c.units, c.groups);
-      if (share_end <= share_begin) break;
-      const uint32_t split_tile = (share_end - 1) / (uint32_t)n_iter;
-      const uint32_t tile_first_unit = split_tile * (uint32_t)n_iter;
-      tile_id = (int)(c.whole_rounds * c.groups + split_tile);
-      seg_begin = share_begin > tile_first_unit ? (int)(share_begin - tile_first_unit) : 0;
-      seg_end = (int)(share_end - tile_first_unit);
-      share_end = tile_first_unit + (uint32_t)seg_begin;
-    }
+    Segment seg;
+    if (!next_segment(at, group_number(c.groups), c.groups, c.units, c.whole_rounds, (uint32_t)n_iter, seg)) break;
+    tile_id = (int)seg.tile;
+    seg_begin = seg.begin;
+    seg_end = seg.end;
   }
   const int head = tile_id / p.n_qtiles, qtile = tile_id - head * p.n_qtiles;
   // The thread's coordinates, derived anew in every segment (see fresh_thread_index).
@@ -614,12 +601,10 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       const uint32_t G = c.groups, units = c.units, wg = group_number(G);
       const uint32_t split_tile = (uint32_t)tile_id - c.whole_rounds * G;  // the tile's number among the split ones
       auto record_of = [&](uint32_t g) {
-        const uint32_t first_tile = first_unit_of(g, units, G) / (uint32_t)n_iter;
-        return c.partials + (size_t)(2 * g + (first_tile == split_tile ? 0 : 1)) * kPartialFloats + wave * (66 * 64) + lane;
+        return c.partials + (size_t)record_of_part(g, split_tile, G, units, (uint32_t)n_iter) * kPartialFloats + wave * (66 * 64) + lane;
       };
-      const uint32_t tile_first_unit = split_tile * (uint32_t)n_iter;
-      const uint32_t g_first = (uint32_t)((((uint64_t)tile_first_unit + 1) * G - 1) / units);
-      const uint32_t g_last = (uint32_t)((((uint64_t)tile_first_unit + (uint32_t)n_iter) * G - 1) / units);
+      uint32_t g_first, g_last;
+      parts_of_tile(split_tile, G, units, (uint32_t)n_iter, g_first, g_last);
       const int others = (int)(g_last - g_first);
       if (tid == 0)
         tab.last_arrival = wg == g_last && __hip_atomic_load(c.arrivals + split_tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
@@ -793,9 +778,10 @@ static int compute_units_of(int dev, int& cus) {
 //  * 128 queries per workgroup, the key range halved between two sets of waves; one workgroup per tile;
 //  * 256 queries per workgroup (every decoded K/V tile serves twice as many MFMAs: an iteration takes about 1.64
 //    times as long for twice the work), one workgroup per tile;
-//  * 256 queries per workgroup, the (tile, iteration) sequence cut into one equal share per compute unit, tiles
-//    that straddle two shares combined by the workgroup that finishes last.
-// The costs below are in iterations of the first kind; whole rounds of workgroups count in full.
+//  * 256 queries per workgroup, whole rounds of tiles first and the (tile, iteration) sequence of the tiles behind
+//    them cut into one equal share per compute unit; tiles that straddle two shares are combined by the workgroup
+//    that finishes last.
+// plan_attention (attention_split.h) chooses.
 static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
   AttnParams p = p_in;
   const size_t smem = 2 * kStageBytes + sizeof(SlotTable);
@@ -806,57 +792,26 @@ static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
   }
   if (int rc = compute_units_of(dev, cus)) return rc;
   const int64_t n_iter = (p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys;
-  const int64_t tiles_narrow = p.H * ((p.Lq + kWgQueries - 1) / kWgQueries);
-  const int64_t tiles_wide = p.H * ((p.Lq + 2 * kWgQueries - 1) / (2 * kWgQueries));
-  constexpr double kWideIteration = 1.64, kCombine = 6.0;
-  const double cost_narrow = (double)((tiles_narrow + cus - 1) / cus * n_iter);
-  const double cost_wide = kWideIteration * (double)((tiles_wide + cus - 1) / cus * n_iter);
-  // Split: whole rounds first, the tiles behind them in equal shares.  A handful of left-over tiles would be cut
-  // into many thin parts each (and combined by a single workgroup): then one whole round joins the split part,
-  // whose shares are a little more than one tile.
-  int64_t whole_rounds = tiles_wide / cus;
-  if (const int64_t left = tiles_wide % cus; left > 0 && left * 4 < cus && whole_rounds > 0) --whole_rounds;
-  const int64_t split_tiles = tiles_wide - whole_rounds * cus;
-  const double cost_split =
-      kWideIteration * (double)(whole_rounds * n_iter + (split_tiles * n_iter + cus - 1) / cus) + kCombine;
-  int mode = cost_narrow <= cost_wide && cost_narrow <= cost_split ? 0 : (cost_wide <= cost_split ? 1 : 2);
-  LL_REQUIRE(tiles_narrow * n_iter < (1ll << 32), "ll_kv_attention: too many (tile, iteration) units");
-  if (tiles_wide * n_iter >= (1ll << 31)) mode = 0;
-  if (const int policy = g_attention_policy.load(std::memory_order_relaxed); policy != LL_ATTENTION_AUTO) {
-    LL_REQUIRE(policy == LL_ATTENTION_NARROW || tiles_wide * n_iter < (1ll << 31), "ll_kv_attention: too many tiles for the selected policy");
-    mode = policy;
-  }
-
-  // Every workgroup needs a unit of the split part when there are whole rounds too (the parts of a tile are
-  // counted by shares): otherwise run the tiles whole.
-  if (mode == 2 && (split_tiles == 0 || (whole_rounds > 0 && split_tiles * n_iter < cus))) mode = 1;
-  if (mode == 0) {
-    p.n_qtiles = (int)((p.Lq + kWgQueries - 1) / kWgQueries);
-    p.whole_rounds = 1;
-    p.units = 0;
+  LL_REQUIRE(p.H * ((p.Lq + kWgQueries - 1) / kWgQueries) * n_iter < (1ll << 32), "ll_kv_attention: too many (tile, iteration) units");
+  const AttentionPlan plan = plan_attention(p.Lq, p.H, p.n_cached + p.n_new, cus, g_attention_policy.load(std::memory_order_relaxed));
+  p.n_qtiles = plan.n_qtiles;
+  p.groups = plan.groups;
+  p.whole_rounds = plan.whole_rounds;
+  p.units = plan.units;
+  if (plan.mode == LL_ATTENTION_NARROW) {
     static std::atomic<uint64_t> lds_allowed{0};
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&kv_attention_kernel<false>), smem, lds_allowed, "ll_kv_attention")) return rc;
-    p.groups = (uint32_t)tiles_narrow;
     hipLaunchKernelGGL(kv_attention_kernel<false>, dim3(p.groups), dim3(kAttnThreads), smem, stream, p);
   } else {
-    p.n_qtiles = (int)((p.Lq + 2 * kWgQueries - 1) / (2 * kWgQueries));
-    p.whole_rounds = 1;
-    p.units = 0;
-    unsigned groups = (unsigned)tiles_wide;
-    if (mode == 2 && split_tiles > 0) {
-      p.whole_rounds = (uint32_t)whole_rounds;
-      p.units = (uint32_t)(split_tiles * n_iter);
-      // without whole rounds no workgroup may be left without a unit (the parts of a tile are counted by shares)
-      groups = (unsigned)(whole_rounds == 0 && p.units < (uint32_t)cus ? p.units : (uint32_t)cus);
+    if (plan.mode == LL_ATTENTION_SPLIT) {
       SplitWorkspace w;
-      if (int rc = split_workspace(dev, stream, groups, (int)split_tiles, w)) return rc;
+      if (int rc = split_workspace(dev, stream, plan.groups, (int)plan.split_tiles, w)) return rc;
       p.partials = w.partials;
       p.arrivals = w.arrivals;
     }
     static std::atomic<uint64_t> lds_allowed_w{0};
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&kv_attention_kernel<true>), smem, lds_allowed_w, "ll_kv_attention")) return rc;
-    p.groups = groups;
-    hipLaunchKernelGGL(kv_attention_kernel<true>, dim3(groups), dim3(kAttnThreads), smem, stream, p);
+    hipLaunchKernelGGL(kv_attention_kernel<true>, dim3(p.groups), dim3(kAttnThreads), smem, stream, p);
   }
   LL_CHECK_LAUNCH("kv_attention_kernel");
   return LL_OK;
@@ -871,6 +826,19 @@ extern "C" int ll_kv_attention_set_policy(int policy) {
 }
 
 extern "C" int ll_kv_attention_get_policy(void) { return ll::g_attention_policy.load(); }
+
+extern "C" int ll_kv_attention_plan(int64_t Lq, int num_heads, int64_t n_keys, int compute_units, int policy,
+                                    int* division, uint32_t* workgroups, uint32_t* whole_rounds, int64_t* split_tiles) {
+  LL_REQUIRE(Lq > 0 && num_heads > 0 && n_keys > 0 && compute_units > 0 && Lq < (1ll << 30) && n_keys < (1ll << 30),
+             "ll_kv_attention_plan: bad sizes");
+  LL_REQUIRE(policy >= LL_ATTENTION_AUTO && policy <= LL_ATTENTION_SPLIT, "ll_kv_attention_plan: unknown policy %d", policy);
+  const ll::AttentionPlan plan = ll::plan_attention(Lq, num_heads, n_keys, compute_units, policy);
+  if (division) *division = plan.mode;
+  if (workgroups) *workgroups = plan.groups;
+  if (whole_rounds) *whole_rounds = plan.whole_rounds;
+  if (split_tiles) *split_tiles = plan.split_tiles;
+  return LL_OK;
+}
 
 extern "C" int ll_kv_attention(const void* q, int64_t Lq, int num_heads, const uint64_t* k_values_ptrs,
                                const uint64_t* k_scales_ptrs, const uint64_t* k_amax_ptrs,

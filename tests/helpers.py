@@ -87,3 +87,49 @@ def generator_oracle_params(model) -> dict:
             P[f"{name}.{i}.weight"], P[f"{name}.{i}.bias"] = c(seq[i].weight), c(seq[i].bias)
     P["blocks"] = [block_oracle_params(b) for b in model.blocks]
     return P
+
+
+def _test_hooks():
+    import ctypes
+    import os
+
+    from longlive_amd import _native
+
+    path = os.path.join(os.path.dirname(_native.LIB_PATH), "libll_nvfp4_testhooks.so")
+    if not os.path.exists(path):
+        raise RuntimeError(f"{path} is missing: run `make -C longlive_amd/csrc`")
+    return ctypes.CDLL(path)
+
+
+def attention_segments(G: int, units: int, whole_rounds: int, n_iter: int, g: int):
+    """The (tile, begin, end) segments workgroup g of G walks, in order, from the attention kernel's own division
+    arithmetic compiled for the host (longlive_amd/csrc/attention_split.h through the test-only library)."""
+    import ctypes
+
+    lib = _test_hooks()
+    lib.ll_test_attention_segments.restype = ctypes.c_int
+    lib.ll_test_attention_segments.argtypes = [ctypes.c_uint32] * 5 + [ctypes.c_void_p, ctypes.c_int]
+    buf = (ctypes.c_int32 * (3 * 64))()
+    n = lib.ll_test_attention_segments(G, units, whole_rounds, n_iter, g, buf, 64)
+    assert n <= 64
+    return [(buf[3 * i], buf[3 * i + 1], buf[3 * i + 2]) for i in range(n)]
+
+
+def attention_parts(split_tile: int, G: int, units: int, n_iter: int):
+    import ctypes
+
+    lib = _test_hooks()
+    lib.ll_test_attention_parts.restype = None
+    lib.ll_test_attention_parts.argtypes = [ctypes.c_uint32] * 4 + [ctypes.c_void_p, ctypes.c_void_p]
+    first, last = ctypes.c_uint32(), ctypes.c_uint32()
+    lib.ll_test_attention_parts(split_tile, G, units, n_iter, ctypes.byref(first), ctypes.byref(last))
+    return first.value, last.value
+
+
+def attention_record(g: int, split_tile: int, G: int, units: int, n_iter: int) -> int:
+    import ctypes
+
+    lib = _test_hooks()
+    lib.ll_test_attention_record.restype = ctypes.c_uint32
+    lib.ll_test_attention_record.argtypes = [ctypes.c_uint32] * 5
+    return lib.ll_test_attention_record(g, split_tile, G, units, n_iter)

@@ -1,5 +1,6 @@
 """CPU tests of the host side: the C-ABI library loads and exports every declared symbol, the
 configuration / front-end error behaviour mirrors the reference, module swap and cache policy."""
+import numpy as np
 import pytest
 import torch
 import torch.nn as nn
@@ -230,3 +231,66 @@ def test_nvfp4_checkpoint_helpers_on_plain_dictionaries():
     cfg = ck.build_model_quantization_config(SimpleNamespace(model_quant_scale_rule="mse"))
     assert cfg.scale_rule.value == "mse" and cfg.activation_scale_rule.value == "mse" and not cfg.keep_master_weights
     assert ck.build_model_quantization_config(None).scale_rule.value == "static_6"
+
+
+# --------------------------------------------------------------------------- attention: division of a launch
+def test_attention_plan_for_the_benchmark_shapes():
+    """The launcher's choice, as pure host arithmetic: configs[2] (24 x 11 = 264 tiles of 256 queries on 256 CUs) is
+    cut into 256 equal shares with no whole round; the released shape (672 tiles) runs two whole rounds and cuts
+    the other 160 tiles; cross-attention over 512 text keys keeps one workgroup per 128 queries; a forced split
+    with nothing to split falls back to whole tiles."""
+    plan = _native.attention_plan
+    assert plan(2640, 24, 13200) == {"division": "split", "workgroups": 256, "whole_rounds": 0, "split_tiles": 264}
+    assert plan(7040, 24, 28160) == {"division": "split", "workgroups": 256, "whole_rounds": 2, "split_tiles": 160}
+    assert plan(2640, 24, 512)["division"] == "narrow" and plan(2640, 24, 512)["workgroups"] == 24 * 21
+    assert plan(2560, 24, 4096) == {"division": "wide", "workgroups": 240, "whole_rounds": 1, "split_tiles": 0}
+    assert plan(2048, 32, 4096, policy="split")["division"] == "wide"   # 256 tiles: nothing is left to split
+    assert plan(5, 1, 3000, policy="split") == {"division": "split", "workgroups": 24, "whole_rounds": 0, "split_tiles": 1}
+    assert plan(2640, 24, 13200, compute_units=304)["division"] == "split"
+    with pytest.raises(ValueError):
+        plan(0, 24, 100)
+
+
+def test_attention_work_division_covers_every_iteration_exactly_once():
+    """The kernel's own division arithmetic (csrc/attention_split.h, compiled for the host by the test-only library),
+    for the plans of a spread of launch sizes: every (tile, iteration) is in exactly one segment; a workgroup's
+    whole tiles come first; the parts of a split tile are held by exactly the workgroups parts_of_tile names, one
+    part each, in records that no two parts share; and a share touches at most two tiles partially."""
+    from helpers import attention_parts, attention_record, attention_segments
+
+    cases = [(2640, 24, 13200, 256), (7040, 24, 28160, 256), (300, 3, 1500, 256), (2000, 40, 200, 256),
+             (5, 1, 3000, 256), (3000, 36, 700, 256), (1320, 24, 13200, 256), (2640, 24, 13200, 304),
+             (2640, 24, 13200, 80), (777, 5, 999, 7)]
+    for Lq, H, n_keys, cus in cases:
+        plan = _native.attention_plan(Lq, H, n_keys, cus, policy="split")
+        n_iter = -(-n_keys // 128)
+        tiles = H * -(-Lq // 256)
+        G, rounds, split_tiles = plan["workgroups"], plan["whole_rounds"], plan["split_tiles"]
+        if plan["division"] != "split":
+            assert G == tiles and rounds == 1 and split_tiles == 0
+            continue
+        units = split_tiles * n_iter
+        assert rounds * G + split_tiles == tiles and units >= G
+        covered = np.zeros((tiles, n_iter), dtype=np.int32)
+        holders = {}   # split tile -> workgroups with a part of it
+        records = set()
+        for g in range(G):
+            segs = attention_segments(G, units, rounds, n_iter, g)
+            assert [s[0] for s in segs[:rounds]] == [j * G + g for j in range(rounds)]
+            assert all(s[1] == 0 and s[2] == n_iter for s in segs[:rounds])
+            partial = 0
+            for tile, begin, end in segs:
+                assert 0 <= begin < end <= n_iter
+                covered[tile, begin:end] += 1
+                if (begin, end) != (0, n_iter):
+                    partial += 1
+                    split_tile = tile - rounds * G
+                    holders.setdefault(split_tile, []).append(g)
+                    rec = attention_record(g, split_tile, G, units, n_iter)
+                    assert rec in (2 * g, 2 * g + 1) and rec not in records
+                    records.add(rec)
+            assert partial <= 2
+        assert (covered == 1).all(), (Lq, H, n_keys, cus)
+        for split_tile, gs in holders.items():
+            first, last = attention_parts(split_tile, G, units, n_iter)
+            assert gs == list(range(first, last + 1)), (split_tile, gs, first, last)
