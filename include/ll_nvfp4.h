@@ -298,6 +298,14 @@ int ll_qk_norm_rope_pair(const void* q, const void* k, int64_t rows, int num_hea
                          const void* k_weight, float eps, const float* cos, const float* sin, int64_t seq_len,
                          void* q_out, void* k_out, void* k_out_smooth, void* stream);
 
+/* ll_qk_norm_rope_pair that also leaves max |k_out| in k_amax_sink (may be NULL): k_out is what the cache
+ * quantizes when the chunk is written (wan_5b/modules/causal_model.py:1406-1429), and with the maximum at hand
+ * that quantization needs no pass of its own over the tensor to find it. */
+int ll_qk_norm_rope_pair_amax(const void* q, const void* k, int64_t rows, int num_heads, const void* q_weight,
+                              const void* k_weight, float eps, const float* cos, const float* sin, int64_t seq_len,
+                              void* q_out, void* k_out, void* k_out_smooth, const ll_amax_sink* k_amax_sink,
+                              void* stream);
+
 #ifdef __cplusplus
 }
 #endif

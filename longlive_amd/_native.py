@@ -65,6 +65,8 @@ _SIGNATURES = {
                                 c_void_p, c_void_p]),
     "ll_qk_norm_rope_pair": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_float, c_void_p,
                                      c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ll_qk_norm_rope_pair_amax": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p, c_void_p, c_float, c_void_p,
+                                     c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ll_gate_residual": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_int64, c_int64,
                                  c_void_p, c_void_p]),
     "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
@@ -171,6 +173,28 @@ _active_graph_sinks: dict = {}
 def _device_key(device: torch.device):
     index = device.index if device.index is not None else (torch.cuda.current_device() if device.type == "cuda" else 0)
     return (device.type, index)
+
+
+class PrivateAmaxSink:
+    """An amax sink buffer of its own for one producer / consumer pair whose two ends lie far apart in the launch
+    sequence (the K and V of a chunk are produced early in a forward and quantized into the cache after it): the
+    tickets of the device's shared sink are good only until the next producer launch."""
+
+    def __init__(self, device) -> None:
+        self.parts = torch.zeros(AMAX_PARTS, dtype=torch.int64, device=torch.device(device))
+        self.key = ("private", id(self))
+        self.entry = [self.parts, 0, None]
+        _sinks[self.key] = self.entry
+
+    def ticket(self) -> "AmaxTicket":
+        key = _device_key(self.parts.device)
+        if key in _active_graph_sinks:  # a recording: epochs have to move with the replays
+            return _active_graph_sinks[key].ticket()
+        if self.entry[1] >= 0xFFFFFFFE:
+            self.parts.zero_()
+            self.entry[1] = 0
+        self.entry[1] += 1
+        return AmaxTicket(self.parts, self.entry[1], self.key)
 
 
 class ReplayableAmaxSink:
@@ -494,10 +518,12 @@ def qk_norm_rope(x, weight, eps, cos, sin, num_heads, seq_len=None, smooth=False
     return (out, out_s) if smooth else out
 
 
-def qk_norm_rope_pair(q, k, q_weight, k_weight, eps, cos, sin, num_heads, seq_len=None):
+def qk_norm_rope_pair(q, k, q_weight, k_weight, eps, cos, sin, num_heads, seq_len=None, k_amax_out=None):
     """:func:`qk_norm_rope` of q and of k (with the smoothed second output) in one launch:
-    returns (roped_q, roped_k, smoothed_k), each bf16 [S, num_heads, 128]."""
+    returns (roped_q, roped_k, smoothed_k), each bf16 [S, num_heads, 128].  ``k_amax_out`` (an
+    :class:`AmaxTicket`) receives the absolute maximum of roped_k."""
     _require_cuda(q, k, q_weight, k_weight, cos, sin)
+    sink = _sink_struct(k_amax_out)
     for x in (q, k):
         if x.ndim != 2 or x.dtype != torch.bfloat16 or not x.is_contiguous() or x.shape[1] != num_heads * 128:
             raise ValueError("q and k must be contiguous bfloat16 [S, num_heads * 128] tensors")
@@ -515,10 +541,11 @@ def qk_norm_rope_pair(q, k, q_weight, k_weight, eps, cos, sin, num_heads, seq_le
     out_q = torch.empty((S, num_heads, 128), dtype=q.dtype, device=q.device)
     out_k, out_s = torch.empty_like(out_q), torch.empty_like(out_q)
     with torch.cuda.device(q.device):
-        code = load().ll_qk_norm_rope_pair(q.data_ptr(), k.data_ptr(), S, num_heads, q_weight.contiguous().data_ptr(),
-                                           k_weight.contiguous().data_ptr(), float(eps), cos.data_ptr(),
-                                           sin.data_ptr(), seq_len, out_q.data_ptr(), out_k.data_ptr(),
-                                           out_s.data_ptr(), _stream())
+        code = load().ll_qk_norm_rope_pair_amax(q.data_ptr(), k.data_ptr(), S, num_heads,
+                                                q_weight.contiguous().data_ptr(), k_weight.contiguous().data_ptr(),
+                                                float(eps), cos.data_ptr(), sin.data_ptr(), seq_len,
+                                                out_q.data_ptr(), out_k.data_ptr(), out_s.data_ptr(),
+                                                ctypes.byref(sink), _stream())
     _check(code, "ll_qk_norm_rope_pair")
     return out_q, out_k, out_s
 

@@ -249,6 +249,7 @@ struct QkProblem {  // one tensor of the q / k pair
   const uint16_t* w;
   uint16_t* out;
   uint16_t* out_smooth;  // or null
+  AmaxSink sink;         // receives max |out| when sink.parts is not null
 };
 struct QkProblems {
   QkProblem p[2];
@@ -282,6 +283,7 @@ __global__ __launch_bounds__(kRowThreads) void qk_norm_rope_kernel(QkProblems pr
   const float ms = wave_sum_dpp(sq) / (float)C;
   const float r = 1.0f / sqrtf(ms + eps);
   const bool rotate = row < seq_len;
+  float out_max = 0.0f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = lane + i * 64;  // uniform over each group of 16 threads: c < nchunks or not
@@ -305,7 +307,9 @@ __global__ __launch_bounds__(kRowThreads) void qk_norm_rope_kernel(QkProblems pr
 #pragma unroll
         for (int j = 0; j < 8; ++j) o8[j] = y[j];
       }
-      *reinterpret_cast<uint4*>(out + row * (int64_t)C + c * 8) = pack8(o8);
+      const uint4 packed = pack8(o8);
+      *reinterpret_cast<uint4*>(out + row * (int64_t)C + c * 8) = packed;
+      out_max = abs_max_bf16x8(packed, out_max);
       if (out_smooth) {
         float part = 0.0f;
 #pragma unroll
@@ -319,6 +323,10 @@ __global__ __launch_bounds__(kRowThreads) void qk_norm_rope_kernel(QkProblems pr
         *reinterpret_cast<uint4*>(out_smooth + row * (int64_t)C + c * 8) = pack8(s8);
       }
     }
+  }
+  if (pr.sink.parts) {
+    out_max = wave_max(out_max);
+    if (lane == 0) amax_sink_update(pr.sink, (uint32_t)row, out_max);
   }
 }
 
@@ -514,17 +522,26 @@ extern "C" int ll_qk_norm_rope(const void* x, int64_t rows, int num_heads, const
                                void* stream) {
   ll::QkProblems problems{};
   problems.p[0] = {static_cast<const uint16_t*>(x), static_cast<const uint16_t*>(weight), static_cast<uint16_t*>(out),
-                   static_cast<uint16_t*>(out_smooth)};
+                   static_cast<uint16_t*>(out_smooth), ll::AmaxSink{}};
   return launch_qk_norm_rope(problems, 1, rows, num_heads, eps, cos, sin, seq_len, stream);
 }
 
 extern "C" int ll_qk_norm_rope_pair(const void* q, const void* k, int64_t rows, int num_heads, const void* q_weight,
                                     const void* k_weight, float eps, const float* cos, const float* sin,
                                     int64_t seq_len, void* q_out, void* k_out, void* k_out_smooth, void* stream) {
+  return ll_qk_norm_rope_pair_amax(q, k, rows, num_heads, q_weight, k_weight, eps, cos, sin, seq_len, q_out, k_out,
+                                   k_out_smooth, nullptr, stream);
+}
+
+extern "C" int ll_qk_norm_rope_pair_amax(const void* q, const void* k, int64_t rows, int num_heads,
+                                         const void* q_weight, const void* k_weight, float eps, const float* cos,
+                                         const float* sin, int64_t seq_len, void* q_out, void* k_out,
+                                         void* k_out_smooth, const ll_amax_sink* k_amax_sink, void* stream) {
+  LL_REQUIRE(ll::sink_is_valid(k_amax_sink), "ll_qk_norm_rope_pair_amax: amax sink needs 8-byte alignment and a non-zero epoch");
   ll::QkProblems problems{};
   problems.p[0] = {static_cast<const uint16_t*>(q), static_cast<const uint16_t*>(q_weight),
-                   static_cast<uint16_t*>(q_out), nullptr};
+                   static_cast<uint16_t*>(q_out), nullptr, ll::AmaxSink{}};
   problems.p[1] = {static_cast<const uint16_t*>(k), static_cast<const uint16_t*>(k_weight),
-                   static_cast<uint16_t*>(k_out), static_cast<uint16_t*>(k_out_smooth)};
+                   static_cast<uint16_t*>(k_out), static_cast<uint16_t*>(k_out_smooth), ll::make_sink(k_amax_sink)};
   return launch_qk_norm_rope(problems, 2, rows, num_heads, eps, cos, sin, seq_len, stream);
 }

@@ -70,16 +70,19 @@ class WanLayerNorm(nn.LayerNorm):
         return super().forward(x).type_as(x)
 
 
-def _project_shared(x: torch.Tensor, layers, amax: torch.Tensor | None = None) -> list[torch.Tensor]:
+def _project_shared(x: torch.Tensor, layers, amax: torch.Tensor | None = None, amax_outs=None) -> list[torch.Tensor]:
     """Apply several linear layers to the same input.  Quantized layers with the same activation config
     share one quantized operand (bit-identical to quantizing per layer, as the reference does).  ``amax`` is
-    the amax ticket that the kernel which produced ``x`` was given."""
+    the amax ticket that the kernel which produced ``x`` was given; ``amax_outs`` (one entry per layer, ``None``
+    for none) are tickets that receive the absolute maximum of a layer's output, which only the quantized path
+    can deliver: the return value says whether it did."""
     first = layers[0]
     if all(isinstance(m, FourOverSixLinear) for m in layers) and all(
             m.config.get_activation_config() == first.config.get_activation_config() for m in layers):
         xq = first.quantize_input(x.reshape(-1, x.shape[-1]), amax=amax)
-        return [m.forward_quantized(xq).reshape(*x.shape[:-1], -1) for m in layers]
-    return [m(x) for m in layers]
+        outs = amax_outs or [None] * len(layers)
+        return [m.forward_quantized(xq, amax_out=t).reshape(*x.shape[:-1], -1) for m, t in zip(layers, outs)], True
+    return [m(x) for m in layers], False
 
 
 def _fused_linear(layer, x: torch.Tensor, *, amax: torch.Tensor | None = None, activation: str | None = None,
@@ -136,7 +139,18 @@ class CausalSelfAttention(nn.Module):
         ``residual + out * gate``, folded into the output projection."""
         b, s = x.shape[:2]
         n, d = self.num_heads, self.head_dim
-        q, k, v = _project_shared(x, [self.q, self.k, self.v], amax=input_amax)
+        # The chunk's K (after norm and RoPE) and V are what the cache quantizes when the chunk is written, after
+        # the forward; their producers leave the tensor maxima in two sinks that belong to this layer's cache, so
+        # that quantization needs no pass of its own to find them.
+        fused_path = b == 1 and d == 128 and not self.use_relative_rope and self.norm_q.eps == self.norm_k.eps
+        k_amax = v_amax = None
+        if fused_path and isinstance(kv_cache, dict):
+            sinks = kv_cache.get("_amax_sinks")
+            if sinks is None:
+                sinks = kv_cache["_amax_sinks"] = (_native.PrivateAmaxSink(x.device), _native.PrivateAmaxSink(x.device))
+            k_amax, v_amax = sinks[0].ticket(), sinks[1].ticket()
+        (q, k, v), v_amax_written = _project_shared(x, [self.q, self.k, self.v], amax=input_amax,
+                                                    amax_outs=[None, None, v_amax])
         v = v.view(b, s, n, d)
         if self.use_relative_rope:
             if rope_fn is None:
@@ -152,7 +166,8 @@ class CausalSelfAttention(nn.Module):
             # RMSNorm -> RoPE (-> K smoothing) of the reference in one pass over q and k
             if self.norm_q.eps == self.norm_k.eps:
                 roped_q, roped_k, smooth_k = _native.qk_norm_rope_pair(
-                    q[0], k[0], self.norm_q.weight.data, self.norm_k.weight.data, self.norm_q.eps, cos, sin, n)
+                    q[0], k[0], self.norm_q.weight.data, self.norm_k.weight.data, self.norm_q.eps, cos, sin, n,
+                    k_amax_out=k_amax)
             else:
                 roped_q = _native.qk_norm_rope(q[0], self.norm_q.weight.data, self.norm_q.eps, cos, sin, n)
                 roped_k, smooth_k = _native.qk_norm_rope(k[0], self.norm_k.weight.data, self.norm_k.eps, cos, sin, n,
@@ -168,6 +183,9 @@ class CausalSelfAttention(nn.Module):
         out, update = kvc.kv_cache_attention(roped_q, roped_k, v, kv_cache, current_start, sink_tokens,
                                              max_attention_size=max_attention_size, smoothed_key=smooth_k,
                                              amax_out=out_amax, global_sink_tokens=global_sink_tokens)
+        if update[2] is not None:
+            update[2]["new_k_amax"] = k_amax
+            update[2]["new_v_amax"] = v_amax if v_amax_written else None
         return _project_out(self.o, out.flatten(2), out_amax, residual, gate, gate_rows), update
 
 
@@ -186,11 +204,11 @@ class CrossAttention(nn.Module):
         calls; the reference has the argument but recomputes on every call (:229-235), which gives the same
         tensors.  Without a cache K / V are recomputed here too."""
         b, n, d = x.shape[0], self.num_heads, self.head_dim
-        q = self.norm_q(_project_shared(x, [self.q], amax=input_amax)[0]).view(b, -1, n, d)
+        q = self.norm_q(_project_shared(x, [self.q], amax=input_amax)[0][0]).view(b, -1, n, d)
         if crossattn_cache is not None and crossattn_cache.get("is_init"):
             k, v = crossattn_cache["k"], crossattn_cache["v"]
         else:
-            k, v = _project_shared(context, [self.k, self.v])
+            k, v = _project_shared(context, [self.k, self.v])[0]
             k = self.norm_k(k).view(b, -1, n, d)
             v = v.view(b, -1, n, d)
             if crossattn_cache is not None:

@@ -228,7 +228,10 @@ def apply_cache_update(cache: dict, current_end: int, local_end_index: int, info
             for name, new in (("k", info["new_k"]), ("v", info["new_v"])):
                 slot: QuantizedTensor = cache[name][start_blk + bi]
                 block = new[0, bi * blk:(bi + 1) * blk].reshape(-1, new.shape[-1])
-                _native.quantize(block, rule, out=(slot.values, slot.scale_factors, slot.amax))
+                # A chunk of one block is quantized as a whole: if its producer left the tensor maximum behind
+                # (an amax ticket of the layer's own sink), the quantization takes it from there.
+                ticket = info.get(f"new_{name}_amax") if n_insert == 1 and new.shape[1] == blk else None
+                _native.quantize(block, rule, amax=ticket, out=(slot.values, slot.scale_factors, slot.amax))
     cache["global_end_index"].fill_(current_end)
     cache["local_end_index"].fill_(local_end_index)
     cache["_global_end"] = current_end

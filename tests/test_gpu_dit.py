@@ -723,3 +723,38 @@ def test_block_forward_recorded_into_a_graph_replays_bit_for_bit(gpu):
             other = block(*cases[(i + 1) % 4][:2], cos1, sin1, cases[(i + 1) % 4][2], cache, L, sink_tokens=L)[0]
             assert torch.equal(other, eager[(i + 1) % 4])
             torch.cuda.synchronize()
+
+
+def test_cache_write_takes_the_k_and_v_maxima_from_their_producers(gpu):
+    """The chunk's roped K and its V are quantized into the cache after the forward.  Their producers (the norm +
+    RoPE kernel, the V projection's epilogue) leave the tensor maxima in the layer's own amax sinks, and the cache
+    write reads them instead of reducing the tensors again: the slot bytes and the slot amax equal those of a write
+    that computes the maxima itself, and a second forward's tickets replace the first's."""
+    from longlive_amd import _native
+
+    torch.manual_seed(0)
+    dim, heads, ffn, F, h, w, T = 256, 2, 512, 2, 8, 8, 16
+    L = F * h * w
+    block = DiTBlock(dim, ffn, heads).to(gpu)
+    block, _ = quantize_model_with_filter(block, ModelQuantizationConfig(), use_default_filtered_modules=True,
+                                          materialize_for_inference=True, verbose=False)
+    cos, sin = rope_cos_sin(build_rope_angles(128), F, h, w, 0, gpu)
+    g = torch.Generator().manual_seed(4)
+    cache = kvc.initialize_kv_cache(1, L, 2, heads, 128, KV, gpu)[0]
+    plain = kvc.initialize_kv_cache(1, L, 2, heads, 128, KV, gpu)[0]
+    with torch.no_grad():
+        for scale in (4.0, 0.25):  # the second forward writes the same slot again, with smaller maxima
+            x = (torch.randn(1, L, dim, generator=g) * scale).bfloat16().to(gpu)
+            e0 = torch.randn(1, F, 6, dim, generator=g).bfloat16().to(gpu)
+            ctx = torch.randn(1, T, dim, generator=g).bfloat16().to(gpu)
+            _, (ce, le, info) = block(x, e0, cos, sin, ctx, cache, 0, sink_tokens=L)
+            assert isinstance(info["new_k_amax"], _native.AmaxTicket) and isinstance(info["new_v_amax"], _native.AmaxTicket)
+            assert info["new_k_amax"].parts is not info["new_v_amax"].parts
+            without = {k: v for k, v in info.items() if not k.endswith("_amax")}
+            kvc.apply_cache_update(plain, ce, le, without, KV)
+            kvc.apply_cache_update(cache, ce, le, info, KV)
+            for name, new in (("k", info["new_k"]), ("v", info["new_v"])):
+                a, b = cache[name][0], plain[name][0]
+                assert float(a.amax) == float(b.amax) == float(new.float().abs().max())
+                assert torch.equal(a.values, b.values) and np.array_equal(u8(a.scale_factors), u8(b.scale_factors))
+            cache["_global_end"] = cache["_local_end"] = plain["_global_end"] = plain["_local_end"] = 0  # write slot 0 again
