@@ -130,8 +130,10 @@ class CausalSelfAttention(nn.Module):
         self.use_relative_rope = False  # set on the module by the pipeline (pipeline/causal_diffusion_inference.py:316)
 
     def forward(self, x, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size, *, input_amax=None,
-                residual=None, gate=None, gate_rows=0, global_sink_tokens=0, rope_fn=None):
+                residual=None, gate=None, gate_rows=0, global_sink_tokens=0, rope_fn=None, collect_kv_amax=True):
         """``input_amax``: the amax ticket the producer of ``x`` was given, if any.
+        ``collect_kv_amax``: leave the maxima of the chunk's K and V behind for the cache write (a forward whose
+        cache update will not be applied has no use for them, and they cost ~3 us).
         ``global_sink_tokens``: leading tokens of the stream that stay in the cache for good (multi-shot mode).
         ``rope_fn(frames, start_frame) -> (cos, sin)``: needed when ``use_relative_rope`` is set; the positions
         then count frames of the attended window instead of frames of the stream.
@@ -144,7 +146,7 @@ class CausalSelfAttention(nn.Module):
         # that quantization needs no pass of its own to find them.
         fused_path = b == 1 and d == 128 and not self.use_relative_rope and self.norm_q.eps == self.norm_k.eps
         k_amax = v_amax = None
-        if fused_path and isinstance(kv_cache, dict):
+        if fused_path and collect_kv_amax and isinstance(kv_cache, dict):
             sinks = kv_cache.get("_amax_sinks")
             if sinks is None:
                 sinks = kv_cache["_amax_sinks"] = (_native.PrivateAmaxSink(x.device), _native.PrivateAmaxSink(x.device))
@@ -245,7 +247,7 @@ class DiTBlock(nn.Module):
         return _project_out(down, h, h_amax, residual, gate, gate_rows)
 
     def forward(self, x, e, cos, sin, context, kv_cache, current_start, sink_tokens, max_attention_size=None,
-                crossattn_cache=None, global_sink_tokens=0, rope_fn=None):
+                crossattn_cache=None, global_sink_tokens=0, rope_fn=None, collect_kv_amax=True):
         """x [1, L, C]; e [1, F, 6, C]; returns (x, (current_end, local_end_index, cache_update_info)).
         The tensor amax that each activation quantization needs is produced by the kernel that writes the
         activation wherever that kernel is one of this package's."""
@@ -256,7 +258,8 @@ class DiTBlock(nn.Module):
         y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.eps, amax_out=y_amax)
         x, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size,
                                    input_amax=y_amax, residual=x, gate=gates[0], gate_rows=frame_seqlen,
-                                   global_sink_tokens=global_sink_tokens, rope_fn=rope_fn)
+                                   global_sink_tokens=global_sink_tokens, rope_fn=rope_fn,
+                                   collect_kv_amax=collect_kv_amax)
         y_amax = _native.amax_ticket(x.device) if isinstance(self.cross_attn.q, FourOverSixLinear) else None
         x = self.cross_attn(self.norm3(x, amax_out=y_amax), context, crossattn_cache, residual=x, input_amax=y_amax)
         y_amax = _native.amax_ticket(x.device) if isinstance(self.ffn[0], FourOverSixLinear) else None
@@ -377,7 +380,8 @@ class CausalDiT(nn.Module):
             x, upd = block(x, e0, cos, sin, ctx, kv_cache[i], current_start, sink_tokens, max_attn,
                            None if crossattn_cache is None else crossattn_cache[i],
                            global_sink_tokens=self.global_sink_size * frame_seqlen,
-                           rope_fn=lambda frames, first: self._rope(frames, h, w, first, x.device))
+                           rope_fn=lambda frames, first: self._rope(frames, h, w, first, x.device),
+                           collect_kv_amax=apply_cache_updates)
             updates.append(upd)
         if apply_cache_updates:
             for i, (cur_end, loc_end, info) in enumerate(updates):
