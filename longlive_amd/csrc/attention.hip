@@ -4,11 +4,15 @@
 // Replaces "dequantize the whole cache to bf16, copy the chunk in, call flash attention"
 // (wan_5b/modules/causal_model.py:557-567, 628-671, 781; utils/quant.py:731-768).
 //
-// Workgroup = one head x 128 queries, 8 waves = two per SIMD.  Wave w owns 32 queries (w & 3) and every
-// second 64-key tile (w >> 2); the two halves of the key range are merged at the end.  A wave needs at most
-// 256 registers (64 for O^T, 32 for S^T, 32 for its Q fragments, the rest for tile fragments, raw FP4 data
-// and addressing), which is what lets two waves share a SIMD: while one wave converts FP4 data or evaluates
-// exponentials, the other one's MFMAs run.  Per iteration all 512 threads decode 128 keys of K and V
+// A workgroup is 8 waves = two per SIMD, in one of two shapes (template parameter WIDE):
+//   * one head x 128 queries: wave w owns 32 queries (w & 3) and every second 64-key tile (w >> 2); the two
+//     halves of the key range are merged at the end;
+//   * one head x 256 queries: wave w owns 32 queries and walks both 64-key tiles of an iteration, so a decoded
+//     tile serves twice as many MFMAs.  A launch of this shape may hand a workgroup whole tiles, parts of the
+//     key range of tiles (combined through device memory), or both: attention_split.h.
+// A wave needs at most 256 registers (64 for O^T, 32 for S^T, 32 for its Q fragments, the rest for tile
+// fragments, raw FP4 data and addressing), which is what lets two waves share a SIMD: while one wave converts
+// FP4 data or evaluates exponentials, the other one's MFMAs run.  Per iteration all 512 threads decode 128 keys of K and V
 // ((e2m1 x e4m3) x slot scale -> bf16: bit for bit the values the reference's fused cache dequantization and
 // ll_kv_dequantize_blocks produce, utils/kernel/kv_dequant_cuda.cu:95-106) into LDS, both
 // row-major (one row per key), with the same thread layout and the same byte offsets for K and V.  The MFMAs
