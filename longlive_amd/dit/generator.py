@@ -82,7 +82,8 @@ class StreamingGenerator:
     @torch.no_grad()
     def generate(self, noise: torch.Tensor, context, on_chunk=None, scene_cuts=(),
                  negative_context: torch.Tensor | None = None,
-                 initial_latent: torch.Tensor | None = None) -> torch.Tensor:
+                 initial_latent: torch.Tensor | None = None, decode_chunk=None,
+                 decode_stream: "torch.cuda.Stream | None" = None):
         """noise [1, F, C, H, W] bf16 latents, context [L, text_dim] bf16 (or one such tensor per chunk) ->
         denoised latents of the same shape.  ``on_chunk(index)`` is called after each chunk (timing hooks).
         ``scene_cuts``: indices of the chunks that open a new scene (the reference recognises them by a prefix
@@ -91,7 +92,14 @@ class StreamingGenerator:
         latents of frames that precede the generated ones (image / video continuation, :375-432): they are run
         through the model at timestep 0 block by block to fill the cache and are returned in front of the generated
         frames; F0 must be a whole number of blocks (the reference's single independent first frame is not
-        supported by the block-wise FP4 cache)."""
+        supported by the block-wise FP4 cache).
+        ``decode_chunk(latents [1, C, f, H, W]) -> tensor``: streaming decode (:443-456, 666-683).  Every finished
+        chunk is handed to it on ``decode_stream`` (a side stream of default priority, created here when none is
+        given) behind an event recorded after the chunk's last denoising step, so that decoding chunk i overlaps the
+        clean-context pass of chunk i and the forwards of chunk i + 1; chunks are decoded in order, and the decode
+        of chunk i - 1 is waited for before that of chunk i is issued, as the reference's asynchronous VAE path does
+        (a decoder that caches features between chunks relies on it).  The return value is then
+        ``(latents, [decoded chunks])``; the caller's stream has waited for the last decode."""
         cfg = self.cfg
         _, F, C, H, W = noise.shape
         fs = (H // cfg.patch_size[1]) * (W // cfg.patch_size[2])
@@ -120,6 +128,9 @@ class StreamingGenerator:
         shot_index = 0
         self.model.rope_temporal_offset = 0.0
         sigmas = [t / 1000.0 for t in self.timesteps] + [0.0]
+        decoded, previous_decode = [], None
+        if decode_chunk is not None and decode_stream is None:
+            decode_stream = torch.cuda.Stream(device=self.device)
         for ci, src in enumerate(range(0, F, nb)):
             start = f0 + src                                              # position of the chunk in the stream
             x = noise[0, src:src + nb].transpose(0, 1).contiguous()      # [C, f, H, W]
@@ -154,6 +165,18 @@ class StreamingGenerator:
                 else:
                     x = (x.float() + (sigmas[si + 1] - sigmas[si]) * flow.float()).to(noise.dtype)
             out[0, start:start + f] = x.transpose(0, 1)
+            if decode_chunk is not None:
+                chunk_done = torch.cuda.Event()
+                chunk_done.record()
+                if previous_decode is not None:
+                    previous_decode.synchronize()
+                with torch.cuda.stream(decode_stream):
+                    decode_stream.wait_event(chunk_done)
+                    latents = x.unsqueeze(0)
+                    latents.record_stream(decode_stream)
+                    decoded.append(decode_chunk(latents))
+                previous_decode = torch.cuda.Event()
+                previous_decode.record(decode_stream)
             # clean-context pass: rewrites this chunk's K / V in the cache
             for cache, text, xc in zip(caches, (context, negative_context), (xcache, xcache_neg)):
                 if is_scene_cut and self.shot_clean_recache:
@@ -163,4 +186,7 @@ class StreamingGenerator:
                     kvc.pin_current_chunk(cache, f * fs, cfg.sink_size * fs)
             if on_chunk is not None:
                 on_chunk(ci)
+        if decode_chunk is not None:
+            torch.cuda.current_stream(self.device).wait_stream(decode_stream)
+            return out, decoded
         return out

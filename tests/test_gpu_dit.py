@@ -758,3 +758,46 @@ def test_cache_write_takes_the_k_and_v_maxima_from_their_producers(gpu):
                 assert float(a.amax) == float(b.amax) == float(new.float().abs().max())
                 assert torch.equal(a.values, b.values) and np.array_equal(u8(a.scale_factors), u8(b.scale_factors))
             cache["_global_end"] = cache["_local_end"] = plain["_global_end"] = plain["_local_end"] = 0  # write slot 0 again
+
+
+def test_streaming_decode_hook_decodes_every_chunk_in_order_on_a_side_stream(gpu):
+    """Streaming decode (pipeline/causal_diffusion_inference.py:443-456, 666-683): each finished chunk goes to a
+    decoder on a side stream while the generator carries on.  The decoder here keeps state between chunks like
+    the reference's cached VAE decode (a running sum of everything seen so far enters each output), so a chunk
+    decoded out of order, twice, or before its latents are final would show.  The decoded chunks must equal the
+    same decoder run over the finished latents afterwards, and the latents those of a run without the hook."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+
+    def build():
+        return StreamingGenerator(cfg, gpu, seed=11)
+
+    gen = build()
+    g = torch.Generator().manual_seed(12)
+    noise = torch.randn(1, 10, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    context = torch.randn(6, 64, generator=g).bfloat16().to(gpu)
+    plain = gen.generate(noise, context)
+
+    class Decoder:
+        def __init__(self):
+            self.seen = torch.zeros((), device=gpu, dtype=torch.float32)
+            self.calls = 0
+
+        def __call__(self, latents):
+            assert latents.shape[0] == 1 and latents.shape[1] == gen.cfg.in_dim
+            self.calls += 1
+            self.seen = self.seen + latents.float().sum()
+            up = torch.nn.functional.interpolate(latents[0].float(), scale_factor=2.0, mode="nearest")
+            return (up + self.seen).clamp_(-50, 50)
+
+    gen2 = build()
+    streamed = Decoder()
+    latents, chunks = gen2.generate(noise, context, decode_chunk=streamed)
+    torch.cuda.synchronize()
+    assert torch.equal(latents, plain)
+    nb = gen.cfg.num_frame_per_block
+    assert streamed.calls == len(chunks) == noise.shape[1] // nb
+    offline = Decoder()
+    for i, chunk in enumerate(chunks):
+        want = offline(plain[:, i * nb:(i + 1) * nb].transpose(1, 2).contiguous())
+        assert torch.equal(chunk, want), i
