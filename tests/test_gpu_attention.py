@@ -630,3 +630,18 @@ def test_work_divisions_agree_at_the_benchmark_shape_and_leave_the_same_amax(gpu
     with pytest.raises(ValueError):
         _native.attention_policy("fastest")
     assert _native.load().ll_kv_attention_set_policy(7) == -1 and b"unknown policy" in _native.load().ll_last_error()
+
+
+@pytest.mark.parametrize("policy", POLICIES)
+def test_random_shapes_under_every_division(gpu, policy):
+    """Twelve random (heads, slot size, cached tokens, new tokens, queries) combinations per division against the
+    oracle: partly attended last slots, no new tokens, no cached tokens, fewer queries than a wave holds."""
+    rng = np.random.default_rng(20240607)
+    with _native.attention_policy(policy):
+        for _ in range(12):
+            H = int(rng.choice([1, 2, 4, 8]))
+            bts = (128 // H) * int(rng.integers(1, 4))
+            n_cached = int(rng.integers(0, 3 * bts + 1))
+            n_new = int(rng.integers(0 if n_cached else 1, 300))
+            Lq = int(rng.integers(1, 700))
+            test_kernel_accepts_any_number_of_cached_tokens(gpu, H, bts, n_cached, n_new, Lq)
