@@ -2,8 +2,9 @@
  * ll_nvfp4.h — C ABI of the MI355X (gfx950) NVFP4 inference hot path.
  *
  * Every entry point takes raw device pointers, sizes and a HIP stream (as void*),
- * launches on that stream, allocates nothing and returns 0 on success or a negative
- * LL_E* code; ll_last_error() gives the message for the calling thread.  All tensors
+ * launches on that stream and returns 0 on success or a negative LL_E* code;
+ * ll_last_error() gives the message for the calling thread.  Nothing is allocated, with
+ * one exception that a caller can switch off (ll_kv_attention_set_policy).  All tensors
  * are row-major.  "bf16" means the 16-bit bit pattern.  Pointers must be valid on
  * the current HIP device.
  *
