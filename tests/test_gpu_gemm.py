@@ -78,6 +78,50 @@ def test_mixed_scale_rules_and_explicit_alpha(gpu):
     assert _rel(y.float().cpu().numpy(), ref) <= TOL
 
 
+def _exact_product(xq, wq):
+    """The product of the two quantized operands in float64 (no rounding that matters: every factor has at most
+    6 significant bits times an fp32 tensor scale), and sum |a||b| for the accumulation bound."""
+    def operand(q):
+        d = _as_oracle(q)
+        Mp, Kp = d["padded"]
+        v = o.unpack_e2m1(d["values"]).astype(np.float64)
+        s = o.e4m3_decode(o.from_blocked(d["scales"], (Mp, Kp // 16))).astype(np.float64)
+        e2, e4 = o.rule_limits(d["rule"])
+        return (v * np.repeat(s, 16, axis=1) * float(d["amax"]) / (e2 * e4))[: d["orig"][0], : d["orig"][1]]
+    a, b = operand(xq), operand(wq)
+    return a @ b.T, np.abs(a) @ np.abs(b).T
+
+
+@pytest.mark.parametrize("M,N,K,kind,seed", [(130, 1, 16, "tie", 0), (64, 128, 64, "tie", 1), (100, 72, 16, "lattice", 2),
+                                             (513, 200, 2048, "tie", 3), (257, 129, 320, "lattice", 4),
+                                             (300, 256, 1024, "gauss", 5)])
+def test_every_output_is_the_exact_product_rounded_once(gpu, M, N, K, kind, seed):
+    """Element-wise bar, tighter than the relative Frobenius norm: each bf16 output lies within half a bf16 ulp of
+    the exact product of the quantized operands, plus the fp32 accumulation error (K * 2^-23 * sum |a||b|).  The
+    "tie" inputs make one product dominate whose exact value (3 * bf16(0.06)) is a bf16 rounding tie, and the
+    lattice inputs produce many such ties: there the fp32 dequantize-then-matmul of the reference may round the
+    other way and differ by a whole ulp, so agreement with it in the norm alone would say nothing."""
+    g = torch.Generator().manual_seed(seed)
+    def make(rows, cols):
+        if kind == "tie":
+            t = torch.randn(rows, cols, generator=g) * 1e-4
+            t[0, 0] = 3.0
+        elif kind == "lattice":
+            t = torch.randint(-12, 13, (rows, cols), generator=g).float() * 0.25
+        else:
+            t = torch.randn(rows, cols, generator=g)
+        return t
+    x, w = make(M, K).bfloat16(), (make(N, K) * 0.02).bfloat16()
+    xq, wq = quantize_to_fp4(x.to(gpu)), quantize_to_fp4(w.to(gpu))
+    y = fp4_matmul(xq, wq).float().cpu().numpy().astype(np.float64)
+    exact, mass = _exact_product(xq, wq)
+    top = np.maximum(np.abs(y), np.abs(exact))
+    ulp = 2.0 ** (np.floor(np.log2(np.maximum(top, 2.0 ** -126))) - 7)
+    bound = 0.5 * ulp + K * 2.0 ** -23 * mass + 2.0 ** -133
+    worst = ((np.abs(y - exact) - bound) / ulp).max()
+    assert worst <= 0, f"an output is {worst:.3f} bf16 ulp beyond the bound"
+
+
 def test_high_precision_operands_are_quantized_on_the_fly(gpu):
     x, w = activations((128, 128), 8).to(gpu), weights((128, 128), 9).to(gpu)
     y1 = fp4_matmul(x, w)
