@@ -9,7 +9,9 @@
 //     halves of the key range are merged at the end;
 //   * one head x 256 queries: wave w owns 32 queries and walks both 64-key tiles of an iteration, so a decoded
 //     tile serves twice as many MFMAs.  A launch of this shape may hand a workgroup whole tiles, parts of the
-//     key range of tiles (combined through device memory), or both: attention_split.h.
+//     key range of tiles (combined through device memory), or both: attention_split.h.  Where a head's last
+//     group of queries fills at most four of the eight waves, the waves without queries do no matrix work and
+//     the division counts such a tile as the lighter load it is.
 // A wave needs at most 256 registers (64 for O^T, 32 for S^T, 32 for its Q fragments, the rest for tile
 // fragments, raw FP4 data and addressing), which is what lets two waves share a SIMD: while one wave converts
 // FP4 data or evaluates exponentials, the other one's MFMAs run.  Per iteration all 512 threads decode 128 keys of K and V
@@ -59,14 +61,12 @@ struct AttnParams {
   float scale_log2;  // softmax scale * log2(e)
   uint16_t* out;
   AmaxSink sink;  // receives max |out| when sink.parts is not null
-  int n_qtiles;
-  // Division of the launch between its G workgroups.  Workgroup g first runs `whole_rounds` whole tiles (tile
-  // j * G + g in round j).  The tiles behind those (256-query kernel only) are cut into `units` = tiles x
-  // iterations, of which workgroup g works through [g * units / G, (g + 1) * units / G); `partials` /
-  // `arrivals` serve those.  One workgroup per tile is whole_rounds = 1, units = 0.
-  uint32_t whole_rounds;
-  uint32_t units;
-  uint32_t groups;  // G, the number of workgroups of the launch
+  int n_qtiles;     // groups of queries per head
+  int full_qtiles;  // tile t < H * full_qtiles is (head t / full_qtiles, group t % full_qtiles); the tiles behind are
+                    // the heads' last groups, (head t - H * full_qtiles, group full_qtiles)
+  // Division of the launch between its d.G workgroups (attention_split.h).  One workgroup per tile is
+  // whole_rounds = 1, extra = 0, units = 0; `partials` / `arrivals` serve the split part (256-query kernel only).
+  Division d;
   float* partials;  // [2 G] records of kPartialFloats floats
   int* arrivals;    // [tiles] counters, zero between launches
 };
@@ -200,6 +200,10 @@ __device__ __forceinline__ const __attribute__((address_space(4))) AttnParams& r
   asm volatile("" : "+s"(a));
   return *a;
 }
+// The launch's division as an ordinary value (seven scalar loads from the argument segment).
+__device__ __forceinline__ Division division_of(const __attribute__((address_space(4))) AttnParams& c) {
+  return Division{c.d.G, c.d.whole_rounds, c.d.extra, c.d.n_iter, c.d.units, c.d.full_units, c.d.light};
+}
 // threadIdx.x as a value the compiler knows nothing about: what is derived from it inside a segment's prologue or
 // epilogue is then computed there, and not ahead of the loop over segments, where it would occupy registers
 // throughout the main loops.
@@ -238,7 +242,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   WorkCursor at;  // where this workgroup is in its work (attention_split.h)
   {
     const auto& c = reread_params();
-    at = start_of_work(group_number(c.groups), c.groups, c.units);
+    at = start_of_work(group_number(c.d.G), division_of(c));
   }
 
   if (const int tid = threadIdx.x; tid < p.n_slots) {
@@ -266,16 +270,35 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   {
     const auto& c = reread_params();
     Segment seg;
-    if (!next_segment(at, group_number(c.groups), c.groups, c.units, c.whole_rounds, (uint32_t)n_iter, seg)) break;
+    if (!next_segment(at, group_number(c.d.G), division_of(c), seg)) break;
     tile_id = (int)seg.tile;
     seg_begin = seg.begin;
     seg_end = seg.end;
   }
-  const int head = tile_id / p.n_qtiles, qtile = tile_id - head * p.n_qtiles;
+  int head, qtile;
+  if (const int n_full = p.H * p.full_qtiles; tile_id < n_full) {
+    head = tile_id / p.full_qtiles;
+    qtile = tile_id - head * p.full_qtiles;
+  } else {
+    head = tile_id - n_full;
+    qtile = p.full_qtiles;
+  }
   // The thread's coordinates, derived anew in every segment (see fresh_thread_index).
   const int tid = fresh_thread_index(), lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, lh = lane >> 5;
   const int qq = WIDE ? wave : (wave & 3), kp = WIDE ? 0 : (wave >> 2);  // group of 32 queries, key parity
+  // 256-query kernel: when the tile holds at most 128 queries (the last group of queries of a head is rarely
+  // full), its waves 4..7 have none, and each wave that has some then has its SIMD to itself (waves w and w + 4
+  // share one).  The waves without queries take their part in bringing K and V into LDS and in every barrier, and
+  // nothing else: no MFMAs, no exponentials, no fragment reads.  With more than 128 queries some SIMD carries two
+  // busy waves whatever the others do, and nothing would be gained (in the 128-query kernel, where the two waves
+  // of a SIMD serve the same queries, never).
+  bool wave_idle = false;
+  if constexpr (WIDE) {
+    const auto& c = reread_params();
+    const int64_t first = (int64_t)qtile * kQueries;
+    wave_idle = __builtin_amdgcn_readfirstlane((int)(c.Lq - first <= 128 && first + qq * kWaveQueries >= c.Lq)) != 0;
+  }
   {
     const auto& c = reread_params();
     int64_t query = (int64_t)qtile * kQueries + qq * kWaveQueries + l32;
@@ -457,6 +480,32 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   // body in a loop of its own.
   const int n_fast = min(n_cached / kIterKeys, seg_end) - 1;
   int it = seg_begin;
+  if (wave_idle) {
+    // A wave without queries: the conversion of its rows, the same number of barriers, nothing else.
+    for (; it < n_fast; ++it) {
+      uint8_t* nxt = smem + ((it + 1) & 1) * kStageBytes;
+      const bool has_next2 = it + 2 < seg_end;
+      const uint32_t wk[4] = {kf.v.x, kf.v.y, kf.v.z, kf.v.w}, wv[4] = {vf.v.x, vf.v.y, vf.v.z, vf.v.w};
+      half2v ks2[2], vs2[2];
+      block_scales_f16(kf.scales, ks2);
+      block_scales_f16(vf.scales, vs2);
+      uint8_t* kdst = nxt + k_dst_off;
+      uint8_t* vdst = nxt + v_dst_off;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float v8[8];
+        fp4x8_to_f32(wk[j], ks2[j >> 1], k_gs, v8);
+        reinterpret_cast<uint4*>(kdst)[j] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
+                                                       pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
+        fp4x8_to_f32(wv[j], vs2[j >> 1], v_gs, v8);
+        reinterpret_cast<uint4*>(vdst)[j] = make_uint4(pack_bf16(v8[0], v8[1]), pack_bf16(v8[2], v8[3]),
+                                                       pack_bf16(v8[4], v8[5]), pack_bf16(v8[6], v8[7]));
+      }
+      advance();
+      if (has_next2) fetch_next();
+      __syncthreads();
+    }
+  }
   for (; it < n_fast; ++it) {
     const uint8_t* cur = smem + (it & 1) * kStageBytes;
     uint8_t* nxt = smem + ((it + 1) & 1) * kStageBytes;
@@ -540,7 +589,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     for (int h = 0; h < kHalves; ++h) {
       const int tile = WIDE ? h : kp;
       const int tile_base = it * kIterKeys + tile * kTileKeys;
-      if (tile_base >= Lk_i) break;
+      if (tile_base >= Lk_i || wave_idle) break;
       float16v sc[2];
       const uint8_t* krow0 = cur + tile * kKTileBytes + l32 * kKPitch + lh * 16;
       const uint8_t* krow1 = krow0 + 32 * kKPitch;
@@ -602,13 +651,13 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       // the result does not depend on the order of arrival.  The workgroup that holds the last part is
       // normally also the last to arrive (the segments are walked backwards, see above): if a look at the
       // counter shows that, it goes on from its registers without writing a record.
-      const uint32_t G = c.groups, units = c.units, wg = group_number(G);
-      const uint32_t split_tile = (uint32_t)tile_id - c.whole_rounds * G;  // the tile's number among the split ones
+      const uint32_t wg = group_number(c.d.G);
+      const uint32_t split_tile = (uint32_t)tile_id - c.d.whole_rounds * c.d.G - c.d.extra;  // the tile's number among the split ones
       auto record_of = [&](uint32_t g) {
-        return c.partials + (size_t)record_of_part(g, split_tile, G, units, (uint32_t)n_iter) * kPartialFloats + wave * (66 * 64) + lane;
+        return c.partials + (size_t)record_of_part(g, split_tile, division_of(c)) * kPartialFloats + wave * (66 * 64) + lane;
       };
       uint32_t g_first, g_last;
-      parts_of_tile(split_tile, G, units, (uint32_t)n_iter, g_first, g_last);
+      parts_of_tile(split_tile, division_of(c), g_first, g_last);
       const int others = (int)(g_last - g_first);
       if (tid == 0)
         tab.last_arrival = wg == g_last && __hip_atomic_load(c.arrivals + split_tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
@@ -616,13 +665,15 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       const bool from_registers = tab.last_arrival != 0;
       write_out = from_registers;
       if (!from_registers) {
-        float* mine = record_of(wg);
+        if (!wave_idle) {
+          float* mine = record_of(wg);
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+          for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-          for (int i = 0; i < 16; ++i) store_shared_f32(mine + (dt * 16 + i) * 64, o[dt][i]);
-        store_shared_f32(mine + 64 * 64, m_run);
-        store_shared_f32(mine + 65 * 64, l_run);
+            for (int i = 0; i < 16; ++i) store_shared_f32(mine + (dt * 16 + i) * 64, o[dt][i]);
+          store_shared_f32(mine + 64 * 64, m_run);
+          store_shared_f32(mine + 65 * 64, l_run);
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the stores have left before the arrival is counted
         __syncthreads();
         if (tid == 0)
@@ -640,7 +691,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
 #pragma unroll
             for (int i = 0; i < 16; ++i) o[dt][i] = 0.0f;
         }
-        for (int g = (int)g_last - (from_registers ? 1 : 0); g >= (int)g_first; --g) {
+        for (int g = (int)g_last - (from_registers ? 1 : 0); g >= (int)g_first && !wave_idle; --g) {
           const float* theirs = record_of((uint32_t)g);
           const float m1 = load_shared_f32(theirs + 64 * 64), l1 = load_shared_f32(theirs + 65 * 64);
           const float m = fmaxf(m_run, m1);
@@ -681,7 +732,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
     float* xo = reinterpret_cast<float*>(smem);   // [qq][64 regs][64 lanes]
     float* xm = xo + 4 * 64 * 64;                  // [qq][64]
     float* xl = xm + 4 * 64;
-    if (kp == 1) {
+    if (kp == 1 && !wave_idle) {
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
@@ -690,7 +741,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
       xl[qq * 64 + lane] = l_run;
     }
     __syncthreads();
-    if (kp == 0) {
+    if (kp == 0 && !wave_idle) {
       float out_max = 0.0f;
       const float m1 = xm[qq * 64 + lane], l1 = xl[qq * 64 + lane];
       const float m = fmaxf(m_run, m1);
@@ -799,23 +850,22 @@ static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
   LL_REQUIRE(p.H * ((p.Lq + kWgQueries - 1) / kWgQueries) * n_iter < (1ll << 32), "ll_kv_attention: too many (tile, iteration) units");
   const AttentionPlan plan = plan_attention(p.Lq, p.H, p.n_cached + p.n_new, cus, g_attention_policy.load(std::memory_order_relaxed));
   p.n_qtiles = plan.n_qtiles;
-  p.groups = plan.groups;
-  p.whole_rounds = plan.whole_rounds;
-  p.units = plan.units;
+  p.full_qtiles = plan.full_qtiles;
+  p.d = plan.d;
   if (plan.mode == LL_ATTENTION_NARROW) {
     static std::atomic<uint64_t> lds_allowed{0};
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&kv_attention_kernel<false>), smem, lds_allowed, "ll_kv_attention")) return rc;
-    hipLaunchKernelGGL(kv_attention_kernel<false>, dim3(p.groups), dim3(kAttnThreads), smem, stream, p);
+    hipLaunchKernelGGL(kv_attention_kernel<false>, dim3(p.d.G), dim3(kAttnThreads), smem, stream, p);
   } else {
     if (plan.mode == LL_ATTENTION_SPLIT) {
       SplitWorkspace w;
-      if (int rc = split_workspace(dev, stream, plan.groups, (int)plan.split_tiles, w)) return rc;
+      if (int rc = split_workspace(dev, stream, plan.d.G, (int)plan.split_tiles, w)) return rc;
       p.partials = w.partials;
       p.arrivals = w.arrivals;
     }
     static std::atomic<uint64_t> lds_allowed_w{0};
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&kv_attention_kernel<true>), smem, lds_allowed_w, "ll_kv_attention")) return rc;
-    hipLaunchKernelGGL(kv_attention_kernel<true>, dim3(p.groups), dim3(kAttnThreads), smem, stream, p);
+    hipLaunchKernelGGL(kv_attention_kernel<true>, dim3(p.d.G), dim3(kAttnThreads), smem, stream, p);
   }
   LL_CHECK_LAUNCH("kv_attention_kernel");
   return LL_OK;
@@ -838,8 +888,8 @@ extern "C" int ll_kv_attention_plan(int64_t Lq, int num_heads, int64_t n_keys, i
   LL_REQUIRE(policy >= LL_ATTENTION_AUTO && policy <= LL_ATTENTION_SPLIT, "ll_kv_attention_plan: unknown policy %d", policy);
   const ll::AttentionPlan plan = ll::plan_attention(Lq, num_heads, n_keys, compute_units, policy);
   if (division) *division = plan.mode;
-  if (workgroups) *workgroups = plan.groups;
-  if (whole_rounds) *whole_rounds = plan.whole_rounds;
+  if (workgroups) *workgroups = plan.d.G;
+  if (whole_rounds) *whole_rounds = plan.d.whole_rounds;
   if (split_tiles) *split_tiles = plan.split_tiles;
   return LL_OK;
 }

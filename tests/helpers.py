@@ -101,35 +101,85 @@ def _test_hooks():
     return ctypes.CDLL(path)
 
 
-def attention_segments(G: int, units: int, whole_rounds: int, n_iter: int, g: int):
-    """The (tile, begin, end) segments workgroup g of G walks, in order, from the attention kernel's own division
-    arithmetic compiled for the host (longlive_amd/csrc/attention_split.h through the test-only library)."""
+DIVISION_FIELDS = ("G", "whole_rounds", "extra", "n_iter", "units", "full_units", "light")
+
+
+def _division_array(division: dict):
+    import ctypes
+
+    return (ctypes.c_uint32 * 7)(*[int(division[k]) for k in DIVISION_FIELDS])
+
+
+def attention_segments(division: dict, g: int):
+    """The (tile, begin, end) segments workgroup g walks, in order, from the attention kernel's own division
+    arithmetic compiled for the host (longlive_amd/csrc/attention_split.h through the test-only library).
+    ``division`` has the keys of DIVISION_FIELDS."""
     import ctypes
 
     lib = _test_hooks()
     lib.ll_test_attention_segments.restype = ctypes.c_int
-    lib.ll_test_attention_segments.argtypes = [ctypes.c_uint32] * 5 + [ctypes.c_void_p, ctypes.c_int]
-    buf = (ctypes.c_int32 * (3 * 64))()
-    n = lib.ll_test_attention_segments(G, units, whole_rounds, n_iter, g, buf, 64)
-    assert n <= 64
+    lib.ll_test_attention_segments.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_int]
+    buf = (ctypes.c_int32 * (3 * 4096))()
+    n = lib.ll_test_attention_segments(_division_array(division), g, buf, 4096)
+    assert n <= 4096
     return [(buf[3 * i], buf[3 * i + 1], buf[3 * i + 2]) for i in range(n)]
 
 
-def attention_parts(split_tile: int, G: int, units: int, n_iter: int):
+def attention_parts(split_tile: int, division: dict):
     import ctypes
 
     lib = _test_hooks()
     lib.ll_test_attention_parts.restype = None
-    lib.ll_test_attention_parts.argtypes = [ctypes.c_uint32] * 4 + [ctypes.c_void_p, ctypes.c_void_p]
+    lib.ll_test_attention_parts.argtypes = [ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     first, last = ctypes.c_uint32(), ctypes.c_uint32()
-    lib.ll_test_attention_parts(split_tile, G, units, n_iter, ctypes.byref(first), ctypes.byref(last))
+    lib.ll_test_attention_parts(split_tile, _division_array(division), ctypes.byref(first), ctypes.byref(last))
     return first.value, last.value
 
 
-def attention_record(g: int, split_tile: int, G: int, units: int, n_iter: int) -> int:
+def attention_record(g: int, split_tile: int, division: dict) -> int:
     import ctypes
 
     lib = _test_hooks()
     lib.ll_test_attention_record.restype = ctypes.c_uint32
-    lib.ll_test_attention_record.argtypes = [ctypes.c_uint32] * 5
-    return lib.ll_test_attention_record(g, split_tile, G, units, n_iter)
+    lib.ll_test_attention_record.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p]
+    return lib.ll_test_attention_record(g, split_tile, _division_array(division))
+
+
+def attention_full_plan(Lq: int, H: int, n_keys: int, cus: int = 256, policy: int = -1) -> dict:
+    """The launcher's choice for a shape, division included: mode (0 narrow, 1 wide, 2 split), n_qtiles,
+    full_qtiles, split_tiles and the keys of DIVISION_FIELDS."""
+    import ctypes
+
+    lib = _test_hooks()
+    lib.ll_test_attention_full_plan.restype = None
+    lib.ll_test_attention_full_plan.argtypes = [ctypes.c_int64, ctypes.c_int, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+                                                ctypes.c_void_p]
+    out = (ctypes.c_uint32 * 11)()
+    lib.ll_test_attention_full_plan(Lq, H, n_keys, cus, policy, out)
+    plan = dict(mode=out[0], n_qtiles=out[1], full_qtiles=out[2], split_tiles=out[3])
+    plan.update({k: out[4 + i] for i, k in enumerate(DIVISION_FIELDS)})
+    return plan
+
+
+def attention_division_on_device(division: dict, split_tiles: int, device):
+    """first_unit_of(g) for g = 0 .. G and (first, last) holder of every split tile, computed by a kernel that calls the
+    same functions as the attention kernel; and the host's values for the same division."""
+    import ctypes
+
+    import torch
+
+    lib = _test_hooks()
+    lib.ll_test_attention_division_on_device.restype = ctypes.c_int
+    lib.ll_test_attention_division_on_device.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p]
+    lib.ll_test_attention_first_unit.restype = ctypes.c_uint32
+    lib.ll_test_attention_first_unit.argtypes = [ctypes.c_uint32, ctypes.c_void_p]
+    arr = _division_array(division)
+    G = int(division["G"])
+    out = torch.zeros(G + 1 + 2 * split_tiles, dtype=torch.int32, device=device)
+    rc = lib.ll_test_attention_division_on_device(arr, split_tiles, out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    got = out.cpu().numpy().astype(np.uint32)
+    host = [lib.ll_test_attention_first_unit(g, arr) for g in range(G + 1)]
+    host += [x for t in range(split_tiles) for x in attention_parts(t, division)]
+    return got, np.array(host, dtype=np.uint32)

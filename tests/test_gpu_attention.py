@@ -674,6 +674,23 @@ def test_work_divisions_agree_at_the_benchmark_shape_and_leave_the_same_amax(gpu
     assert _native.load().ll_kv_attention_set_policy(7) == -1 and b"unknown policy" in _native.load().ll_last_error()
 
 
+def test_division_arithmetic_is_the_same_on_device_and_host(gpu):
+    """The launcher plans on the host, the kernel walks the plan on the device, the CPU tests check the host side:
+    the share boundaries and the holders of every split tile must come out the same on both (64-bit integer
+    arithmetic throughout), for the launcher's plans of the benchmark shapes and for a division beyond 32 bits."""
+    from helpers import DIVISION_FIELDS, attention_division_on_device, attention_full_plan
+
+    for shape in [(2640, 24, 13200), (7040, 24, 28160), (880, 24, 13200), (3000, 24, 9000), (5, 1, 3000), (1320, 24, 2640)]:
+        plan = attention_full_plan(*shape)
+        if plan["mode"] != 2:
+            continue
+        got, host = attention_division_on_device({k: plan[k] for k in DIVISION_FIELDS}, plan["split_tiles"], gpu)
+        assert np.array_equal(got, host), shape
+    big = dict(G=256, whole_rounds=1, extra=200, n_iter=300001, units=9 * 300001, full_units=2 * 300001, light=12)
+    got, host = attention_division_on_device(big, 9, gpu)
+    assert np.array_equal(got, host)
+
+
 @pytest.mark.parametrize("policy", POLICIES)
 def test_random_shapes_under_every_division(gpu, policy):
     """Twelve random (heads, slot size, cached tokens, new tokens, queries) combinations per division against the

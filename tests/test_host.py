@@ -235,62 +235,107 @@ def test_nvfp4_checkpoint_helpers_on_plain_dictionaries():
 
 # --------------------------------------------------------------------------- attention: division of a launch
 def test_attention_plan_for_the_benchmark_shapes():
-    """The launcher's choice, as pure host arithmetic: configs[2] (24 x 11 = 264 tiles of 256 queries on 256 CUs) is
-    cut into 256 equal shares with no whole round; the released shape (672 tiles) runs two whole rounds and cuts
-    the other 160 tiles; cross-attention over 512 text keys keeps one workgroup per 128 queries; a forced split
-    with nothing to split falls back to whole tiles."""
+    """The launcher's choice, as pure host arithmetic.  configs[2] has 24 x 10 full tiles of 256 queries and 24
+    tiles of 80 queries (three of eight waves busy: 11 sixteenths of the cost) on 256 CUs: the full tiles run whole
+    on 240 workgroups and the other 16 share the light ones.  The released shape (27 full groups of queries and
+    one of 128 per head) runs two whole rounds; whole left-over tiles would make that three, so the 136 full and
+    24 light tiles behind the rounds are shared by all workgroups, by cost.  Cross-attention over 512 text keys
+    keeps one workgroup per 128 queries; a forced split with nothing to split falls back to whole tiles."""
+    from helpers import attention_full_plan
+
     plan = _native.attention_plan
-    assert plan(2640, 24, 13200) == {"division": "split", "workgroups": 256, "whole_rounds": 0, "split_tiles": 264}
+    assert plan(2640, 24, 13200) == {"division": "split", "workgroups": 256, "whole_rounds": 0, "split_tiles": 24}
+    full = attention_full_plan(2640, 24, 13200)
+    assert (full["extra"], full["full_units"], full["units"], full["light"], full["full_qtiles"]) == (240, 0, 24 * 104, 11, 10)
     assert plan(7040, 24, 28160) == {"division": "split", "workgroups": 256, "whole_rounds": 2, "split_tiles": 160}
+    full = attention_full_plan(7040, 24, 28160)
+    assert (full["extra"], full["full_units"], full["light"], full["full_qtiles"], full["n_qtiles"]) == (0, 136 * 220, 12, 27, 28)
     assert plan(2640, 24, 512)["division"] == "narrow" and plan(2640, 24, 512)["workgroups"] == 24 * 21
     assert plan(2560, 24, 4096) == {"division": "wide", "workgroups": 240, "whole_rounds": 1, "split_tiles": 0}
     assert plan(2048, 32, 4096, policy="split")["division"] == "wide"   # 256 tiles: nothing is left to split
-    assert plan(5, 1, 3000, policy="split") == {"division": "split", "workgroups": 24, "whole_rounds": 0, "split_tiles": 1}
+    assert plan(5, 1, 3000, policy="split") == {"division": "split", "workgroups": 13, "whole_rounds": 0, "split_tiles": 1}
     assert plan(2640, 24, 13200, compute_units=304)["division"] == "split"
     with pytest.raises(ValueError):
         plan(0, 24, 100)
 
 
+def _check_division(plan, tiles):
+    """Every (tile, iteration) in exactly one segment; whole tiles first; the parts of a split tile held by exactly
+    the workgroups parts_of_tile names, one part each, in records no two parts share; at most two partial tiles
+    per share; shares of equal cost to within one unit."""
+    from helpers import DIVISION_FIELDS, attention_parts, attention_record, attention_segments
+
+    d = {k: plan[k] for k in DIVISION_FIELDS}
+    G, rounds, extra, n_iter = d["G"], d["whole_rounds"], d["extra"], d["n_iter"]
+    assert rounds * G + extra + plan["split_tiles"] == tiles and d["units"] == plan["split_tiles"] * n_iter
+    assert d["full_units"] <= d["units"] and d["full_units"] % n_iter == 0 and 9 <= d["light"] <= 16
+    covered = np.zeros((tiles, n_iter), dtype=np.int32)
+    holders, records, costs = {}, set(), []
+    for g in range(G):
+        segs = attention_segments(d, g)
+        whole = rounds + (1 if g < extra else 0)
+        assert [s[0] for s in segs[:whole]] == [j * G + g for j in range(whole)]
+        assert all(s[1] == 0 and s[2] == n_iter for s in segs[:whole])
+        assert g >= extra or len(segs) == whole          # a workgroup with an extra tile takes no share
+        partial, cost = 0, 0
+        for tile, begin, end in segs[whole:]:
+            split_tile = tile - rounds * G - extra
+            cost += (end - begin) * (16 if split_tile * n_iter < d["full_units"] else d["light"])
+        for tile, begin, end in segs:
+            assert 0 <= begin < end <= n_iter
+            covered[tile, begin:end] += 1
+            if (begin, end) != (0, n_iter):
+                partial += 1
+                split_tile = tile - rounds * G - extra
+                holders.setdefault(split_tile, []).append(g)
+                rec = attention_record(g, split_tile, d)
+                assert rec in (2 * g, 2 * g + 1) and rec not in records
+                records.add(rec)
+        assert partial <= 2
+        if g >= extra and d["units"]:
+            assert cost > 0
+            costs.append(cost)
+    assert (covered == 1).all()
+    if costs:
+        assert max(costs) - min(costs) <= 2 * 16
+    for split_tile, gs in holders.items():
+        first, last = attention_parts(split_tile, d)
+        assert gs == list(range(first, last + 1)), (split_tile, gs, first, last)
+
+
 def test_attention_work_division_covers_every_iteration_exactly_once():
-    """The kernel's own division arithmetic (csrc/attention_split.h, compiled for the host by the test-only library),
-    for the plans of a spread of launch sizes: every (tile, iteration) is in exactly one segment; a workgroup's
-    whole tiles come first; the parts of a split tile are held by exactly the workgroups parts_of_tile names, one
-    part each, in records that no two parts share; and a share touches at most two tiles partially."""
-    from helpers import attention_parts, attention_record, attention_segments
+    """The kernel's own division arithmetic (csrc/attention_split.h, compiled for the host by the test-only
+    library) for the launcher's plans of a spread of shapes - light last tiles, none, only light tiles, more and
+    fewer tiles than compute units - and for hand-made divisions the launcher would not choose."""
+    from helpers import attention_full_plan
 
     cases = [(2640, 24, 13200, 256), (7040, 24, 28160, 256), (300, 3, 1500, 256), (2000, 40, 200, 256),
              (5, 1, 3000, 256), (3000, 36, 700, 256), (1320, 24, 13200, 256), (2640, 24, 13200, 304),
-             (2640, 24, 13200, 80), (777, 5, 999, 7)]
+             (2640, 24, 13200, 80), (777, 5, 999, 7), (2560, 30, 5000, 256), (100, 300, 640, 256),
+             (2640, 24, 2640, 256), (2640, 24, 5280, 256), (2640, 24, 7920, 256), (2640, 24, 10560, 256)]
+    rng = np.random.default_rng(11)
+    cases += [(int(rng.integers(1, 9000)), int(rng.integers(1, 48)), int(rng.integers(1, 40000)), int(rng.choice([8, 64, 256, 304])))
+              for _ in range(60)]
+    split_seen = 0
     for Lq, H, n_keys, cus in cases:
-        plan = _native.attention_plan(Lq, H, n_keys, cus, policy="split")
-        n_iter = -(-n_keys // 128)
+        plan = attention_full_plan(Lq, H, n_keys, cus, policy=2)
         tiles = H * -(-Lq // 256)
-        G, rounds, split_tiles = plan["workgroups"], plan["whole_rounds"], plan["split_tiles"]
-        if plan["division"] != "split":
-            assert G == tiles and rounds == 1 and split_tiles == 0
+        assert plan["n_iter"] == -(-n_keys // 128) and plan["n_qtiles"] == -(-Lq // 256)
+        if plan["mode"] != 2:
+            assert plan["G"] == tiles and plan["whole_rounds"] == 1 and plan["units"] == 0 and plan["extra"] == 0
+            assert plan["full_qtiles"] == plan["n_qtiles"]
             continue
-        units = split_tiles * n_iter
-        assert rounds * G + split_tiles == tiles and units >= G
-        covered = np.zeros((tiles, n_iter), dtype=np.int32)
-        holders = {}   # split tile -> workgroups with a part of it
-        records = set()
-        for g in range(G):
-            segs = attention_segments(G, units, rounds, n_iter, g)
-            assert [s[0] for s in segs[:rounds]] == [j * G + g for j in range(rounds)]
-            assert all(s[1] == 0 and s[2] == n_iter for s in segs[:rounds])
-            partial = 0
-            for tile, begin, end in segs:
-                assert 0 <= begin < end <= n_iter
-                covered[tile, begin:end] += 1
-                if (begin, end) != (0, n_iter):
-                    partial += 1
-                    split_tile = tile - rounds * G
-                    holders.setdefault(split_tile, []).append(g)
-                    rec = attention_record(g, split_tile, G, units, n_iter)
-                    assert rec in (2 * g, 2 * g + 1) and rec not in records
-                    records.add(rec)
-            assert partial <= 2
-        assert (covered == 1).all(), (Lq, H, n_keys, cus)
-        for split_tile, gs in holders.items():
-            first, last = attention_parts(split_tile, G, units, n_iter)
-            assert gs == list(range(first, last + 1)), (split_tile, gs, first, last)
+        split_seen += 1
+        # the tile numbering: full groups of queries first, head by head, the light last groups behind them
+        light_tiles = H if 1 <= Lq % 256 <= 128 else 0   # busy waves with a SIMD each
+        assert plan["full_qtiles"] == plan["n_qtiles"] - (1 if light_tiles else 0)
+        assert plan["units"] - plan["full_units"] == light_tiles * plan["n_iter"]
+        _check_division(plan, tiles)
+    assert split_seen > 40
+    # hand-made divisions, the last two large enough to leave the 32-bit arithmetic
+    for G, rounds, extra, full_split, light_split, light, n_iter in [
+            (16, 0, 0, 20, 0, 16, 50), (16, 1, 5, 0, 7, 11, 50), (16, 2, 15, 3, 9, 9, 50), (7, 0, 3, 2, 2, 13, 50),
+            (32, 0, 0, 0, 5, 10, 50), (8, 3, 0, 9, 1, 15, 50), (256, 0, 0, 3, 5, 11, 400000), (256, 1, 200, 2, 7, 12, 300001)]:
+        plan = dict(mode=2, n_iter=n_iter, G=G, whole_rounds=rounds, extra=extra, units=(full_split + light_split) * n_iter,
+                    full_units=full_split * n_iter, light=light, split_tiles=full_split + light_split)
+        _check_division(plan, rounds * G + extra + full_split + light_split)
