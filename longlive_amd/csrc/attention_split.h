@@ -185,7 +185,8 @@ inline AttentionPlan plan_attention(int64_t Lq, int H, int64_t n_keys, int cus, 
       plan.d.full_units = (uint32_t)(split_full * n_iter);
       plan.d.light = light_tiles ? light : kFullUnitCost;
       // without whole tiles no workgroup may be left without a unit either
-      const uint64_t shares = split_cost(plan.d) / kFullUnitCost;
+      const uint64_t cost = split_cost(plan.d);
+      const uint64_t shares = cost < kFullUnitCost ? 1 : cost / kFullUnitCost;  // a single light unit costs less than 16
       plan.d.G = (uint32_t)(best.rounds == 0 && best.extra == 0 && shares < (uint64_t)cus ? shares : (uint64_t)cus);
     }
   }

@@ -674,6 +674,18 @@ def test_work_divisions_agree_at_the_benchmark_shape_and_leave_the_same_amax(gpu
     assert _native.load().ll_kv_attention_set_policy(7) == -1 and b"unknown policy" in _native.load().ll_last_error()
 
 
+@pytest.mark.parametrize("policy", POLICIES)
+@pytest.mark.parametrize("H,n_new,Lq", [(1, 14, 64), (1, 1, 1), (2, 130, 5), (3, 64, 129)])
+def test_smallest_launches_under_every_division(gpu, policy, H, n_new, Lq):
+    """One tile of one iteration, a single key, a single query: the split division then has a single light unit
+    (a plan with no workgroup at all once came out of that) or falls back to whole tiles."""
+    q, k, v = _randn((Lq, H, 128), 71), _randn((n_new, H, 128), 72), _randn((n_new, H, 128), 73)
+    with _native.attention_policy(policy):
+        out = _native.attention_bf16(q.to(gpu), k.to(gpu), v.to(gpu), 128 ** -0.5)
+    ref = o.attention(q.float().numpy(), k.float().numpy(), v.float().numpy())
+    assert np.abs(out.float().cpu().numpy() - ref).max() <= 2e-2
+
+
 def test_division_arithmetic_is_the_same_on_device_and_host(gpu):
     """The launcher plans on the host, the kernel walks the plan on the device, the CPU tests check the host side:
     the share boundaries and the holders of every split tile must come out the same on both (64-bit integer

@@ -312,7 +312,8 @@ def test_attention_work_division_covers_every_iteration_exactly_once():
     cases = [(2640, 24, 13200, 256), (7040, 24, 28160, 256), (300, 3, 1500, 256), (2000, 40, 200, 256),
              (5, 1, 3000, 256), (3000, 36, 700, 256), (1320, 24, 13200, 256), (2640, 24, 13200, 304),
              (2640, 24, 13200, 80), (777, 5, 999, 7), (2560, 30, 5000, 256), (100, 300, 640, 256),
-             (2640, 24, 2640, 256), (2640, 24, 5280, 256), (2640, 24, 7920, 256), (2640, 24, 10560, 256)]
+             (2640, 24, 2640, 256), (2640, 24, 5280, 256), (2640, 24, 7920, 256), (2640, 24, 10560, 256),
+             (64, 1, 14, 256), (1, 1, 1, 256), (200, 2, 100, 256), (129, 3, 128, 4)]
     rng = np.random.default_rng(11)
     cases += [(int(rng.integers(1, 9000)), int(rng.integers(1, 48)), int(rng.integers(1, 40000)), int(rng.choice([8, 64, 256, 304])))
               for _ in range(60)]
