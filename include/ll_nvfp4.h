@@ -214,8 +214,9 @@ int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads,
  * launch the cheapest of the three by a cost estimate:
  *   LL_ATTENTION_NARROW  one workgroup per (head, 128 queries);
  *   LL_ATTENTION_WIDE    one workgroup per (head, 256 queries): every decoded K/V tile serves twice as many MFMAs;
- *   LL_ATTENTION_SPLIT   256-query tiles, the (tile, key range) sequence cut into one equal share per compute
- *                        unit, so that the last round of workgroups is as full as the others.  Tiles shared by two
+ *   LL_ATTENTION_SPLIT   256-query tiles; what does not fill whole rounds of one tile per compute unit is cut
+ *                        along the key range into shares of equal cost (a head's last, partly filled group of
+ *                        queries counts for less), so that no compute unit waits for another.  Tiles shared by two
  *                        workgroups pass through device memory that the library allocates on the first such
  *                        launch on a (device, stream) pair and keeps (69 MB on a 256-CU device); launches that
  *                        use it must not overlap on one stream's memory, which same-stream order guarantees.
@@ -230,8 +231,9 @@ int ll_kv_attention_set_policy(int policy); /* LL_OK, or LL_EINVAL for an unknow
 int ll_kv_attention_get_policy(void);
 /* What a launch of Lq queries x num_heads heads over n_keys keys would do on a device with `compute_units` CUs
  * under `policy` (pure host arithmetic, no GPU needed): the division taken (an LL_ATTENTION_SPLIT request falls
- * back to WIDE when there is nothing to split), the number of workgroups, the whole tiles each of them runs first
- * and the number of tiles cut into shares behind those.  Lets a caller know ahead of a launch whether it will
+ * back to WIDE when there is nothing to split), the number of workgroups, the whole rounds of tiles all of them
+ * run first and the number of tiles cut into shares (tiles behind the whole rounds that are not counted here run
+ * whole on workgroups that take no share).  Lets a caller know ahead of a launch whether it will
  * take the allocating division.  Output pointers may be NULL. */
 int ll_kv_attention_plan(int64_t Lq, int num_heads, int64_t n_keys, int compute_units, int policy,
                          int* division, uint32_t* workgroups, uint32_t* whole_rounds, int64_t* split_tiles);
