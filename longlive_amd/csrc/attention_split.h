@@ -115,7 +115,10 @@ struct AttentionPlan {
 
 inline AttentionPlan plan_attention(int64_t Lq, int H, int64_t n_keys, int cus, int policy) {
   constexpr double kWideIteration = 1.64;  // an iteration of the 256-query kernel takes this much longer for twice the work
-  constexpr double kCombine = 6.0;         // partial results: writing, counting, combining
+  constexpr double kCombine = 6.0;         // partial results when every workgroup shares: writing, counting, combining
+  constexpr double kCombineFew = 1.5;      // the same when only the workgroups without a whole extra tile share
+  constexpr double kRound = 4.0;           // what a workgroup spends per tile outside the iterations (Q, first K/V
+                                           // tile, output); fitted on 256 .. 2640 keys, where it decides
   const int64_t n_iter = (n_keys + 127) / 128;
   const int64_t tiles_narrow = H * ((Lq + 127) / 128);
   const int64_t nq = (Lq + 255) / 256;
@@ -146,7 +149,8 @@ inline AttentionPlan plan_attention(int64_t Lq, int H, int64_t n_keys, int cus, 
     // every sharing workgroup needs a unit when others run whole tiles too (the parts of a tile are counted by shares)
     if ((rounds > 0 || extra > 0) && cost < (int64_t)kFullUnitCost * servers) return sh;
     const double share = (double)((cost + servers - 1) / servers) / kFullUnitCost;
-    sh.cost = kWideIteration * ((double)(rounds * n_iter) + (extra > 0 && share < (double)n_iter ? (double)n_iter : share)) + kCombine;
+    sh.cost = kWideIteration * ((double)(rounds * n_iter) + (extra > 0 && share < (double)n_iter ? (double)n_iter : share)) +
+              kRound * (double)(rounds + 1) + (extra > 0 ? kCombineFew : kCombine);
     return sh;
   };
   int64_t rounds_b = full_tiles / cus;
@@ -158,8 +162,8 @@ inline AttentionPlan plan_attention(int64_t Lq, int H, int64_t n_keys, int cus, 
     const Shape a = weigh(full_tiles / cus, full_tiles % cus);
     if (a.cost <= best.cost * 1.04) best = a;
   }
-  const double cost_narrow = (double)((tiles_narrow + cus - 1) / cus * n_iter);
-  const double cost_wide = kWideIteration * (double)((tiles_wide + cus - 1) / cus * n_iter);
+  const double cost_narrow = (double)((tiles_narrow + cus - 1) / cus) * ((double)n_iter + kRound);
+  const double cost_wide = (double)((tiles_wide + cus - 1) / cus) * (kWideIteration * (double)n_iter + kRound);
   int mode = cost_narrow <= cost_wide && cost_narrow <= best.cost ? 0 : (cost_wide <= best.cost ? 1 : 2);
   if (policy >= 0) mode = policy;
   if (tiles_wide * n_iter >= (1ll << 31)) mode = 0;  // units are counted in 32 bits (costs in 64)

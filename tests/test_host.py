@@ -239,8 +239,10 @@ def test_attention_plan_for_the_benchmark_shapes():
     tiles of 80 queries (three of eight waves busy: 11 sixteenths of the cost) on 256 CUs: the full tiles run whole
     on 240 workgroups and the other 16 share the light ones.  The released shape (27 full groups of queries and
     one of 128 per head) runs two whole rounds; whole left-over tiles would make that three, so the 136 full and
-    24 light tiles behind the rounds are shared by all workgroups, by cost.  Cross-attention over 512 text keys
-    keeps one workgroup per 128 queries; a forced split with nothing to split falls back to whole tiles."""
+    24 light tiles behind the rounds are shared by all workgroups, by cost.  Cross-attention of the same 2640
+    queries over 512 text keys takes the first shape too (two rounds of 128-query tiles cost more outside their
+    four iterations than inside); with 880 queries one round of 128-query tiles is best, with 7040 three rounds
+    of 256-query tiles.  A forced split with nothing to split falls back to whole tiles."""
     from helpers import attention_full_plan
 
     plan = _native.attention_plan
@@ -250,7 +252,9 @@ def test_attention_plan_for_the_benchmark_shapes():
     assert plan(7040, 24, 28160) == {"division": "split", "workgroups": 256, "whole_rounds": 2, "split_tiles": 160}
     full = attention_full_plan(7040, 24, 28160)
     assert (full["extra"], full["full_units"], full["light"], full["full_qtiles"], full["n_qtiles"]) == (0, 136 * 220, 12, 27, 28)
-    assert plan(2640, 24, 512)["division"] == "narrow" and plan(2640, 24, 512)["workgroups"] == 24 * 21
+    assert plan(2640, 24, 512) == {"division": "split", "workgroups": 256, "whole_rounds": 0, "split_tiles": 24}
+    assert plan(880, 24, 512)["division"] == "narrow" and plan(880, 24, 512)["workgroups"] == 24 * 7
+    assert plan(7040, 24, 512) == {"division": "wide", "workgroups": 672, "whole_rounds": 1, "split_tiles": 0}
     assert plan(2560, 24, 4096) == {"division": "wide", "workgroups": 240, "whole_rounds": 1, "split_tiles": 0}
     assert plan(2048, 32, 4096, policy="split")["division"] == "wide"   # 256 tiles: nothing is left to split
     assert plan(5, 1, 3000, policy="split") == {"division": "split", "workgroups": 13, "whole_rounds": 0, "split_tiles": 1}
