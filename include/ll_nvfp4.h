@@ -166,6 +166,28 @@ int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A_scales, co
                             void* D, int64_t ldd, const ll_gemm_epilogue* epilogue, void* stream);
 
 /*
+ * Several ll_nvfp4_gemm_tnt products with the same A operand and the same N and Kp in one launch: the q, k and v
+ * projections of one activation (wan_5b/modules/causal_model.py:363-365) and the k, v projections of the text
+ * (:234-235), three resp. two fp4_matmul calls in the reference.  Each product has its own weight, scales, tensor
+ * scale, bias, output and amax sink (bias and sink optional, as in ll_gemm_epilogue); product i computes exactly
+ * what ll_nvfp4_gemm_tnt_fused computes for it alone, bit for bit.  1 <= n_products <= 4.
+ */
+typedef struct ll_gemm_product {
+  const uint8_t* B_values;
+  const uint8_t* B_scales;
+  const float* alpha;     /* f32[1] or NULL: then amax_a * amax_b / (denom_a * denom_b) */
+  const float* amax_b;
+  float denom_b;
+  void* D;                /* bf16 [M, ldd] */
+  int64_t ldd;
+  const void* bias;       /* bf16 [N] or NULL */
+  ll_amax_sink amax_sink; /* parts == NULL: none */
+} ll_gemm_product;
+int ll_nvfp4_gemm_tnt_grouped(const uint8_t* A_values, const uint8_t* A_scales, const float* amax_a, float denom_a,
+                              int64_t M, int64_t N, int64_t Mp, int64_t Np, int64_t Kp, int n_products,
+                              const ll_gemm_product* products, void* stream);
+
+/*
  * Replaces torch.ops.longlive_kernels.dequantize_kv_cache_fp4 (utils/kernel/kv_dequant.cpp:14,
  * utils/kernel/kv_dequant_cuda.cu:59-239): n_blocks cache slots, each NVFP4 [rows_padded, 128] holding
  * block_token_size*num_heads logical rows, are dequantized to out[1, n_blocks*block_token_size, num_heads, 128]

@@ -42,6 +42,8 @@ _SIGNATURES = {
     "ll_nvfp4_gemm_tnt_fused": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
                                         c_float, c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64,
                                         c_void_p, c_void_p]),
+    "ll_nvfp4_gemm_tnt_grouped": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int64, c_int64, c_int64,
+                                          c_int64, c_int, c_void_p, c_void_p]),
     "ll_kv_dequantize_blocks": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_float, c_float,
                                         c_void_p, c_void_p]),
     "ll_kv_attention": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
@@ -396,6 +398,44 @@ def gemm(a_values, a_scales, b_values, b_scales, M: int, N: int, *, alpha=None, 
             ctypes.byref(epi), _stream())
     _check(code, "ll_nvfp4_gemm_tnt")
     return out
+
+
+class GemmProduct(ctypes.Structure):
+    """struct ll_gemm_product of include/ll_nvfp4.h."""
+    _fields_ = [("B_values", c_void_p), ("B_scales", c_void_p), ("alpha", c_void_p), ("amax_b", c_void_p),
+                ("denom_b", ctypes.c_float), ("D", c_void_p), ("ldd", c_int64), ("bias", c_void_p),
+                ("amax_sink", AmaxSinkStruct)]
+
+
+def gemm_grouped(a_values, a_scales, amax_a, denom_a: float, M: int, N: int, products) -> list[torch.Tensor]:
+    """Several products ``A @ B_i^T`` with the same A operand and the same N and K in one launch
+    (ll_nvfp4_gemm_tnt_grouped).  ``products``: one dict per product with ``values``, ``scales``, ``amax``,
+    ``denom`` and optionally ``bias`` and ``amax_out`` (an :class:`AmaxTicket`).  Each output equals what
+    :func:`gemm` returns for that product alone, bit for bit."""
+    Mp, Kb = a_values.shape
+    sinks = [pr["amax_out"].parts.data_ptr() for pr in products if pr.get("amax_out") is not None]
+    if len(set(sinks)) != len(sinks):
+        raise ValueError("the products of one launch need amax sinks with buffers of their own (a later epoch hides an "
+                         "earlier one on a shared buffer)")
+    outs, structs = [], (GemmProduct * len(products))()
+    for i, pr in enumerate(products):
+        bias = pr.get("bias")
+        _require_cuda(pr["values"], pr["scales"], pr["amax"], bias)
+        if pr["values"].shape[1] != Kb or pr["values"].shape[0] != products[0]["values"].shape[0]:
+            raise ValueError("the products of one launch must have the same N and K")
+        if bias is not None and (bias.dtype != torch.bfloat16 or bias.numel() != N or not bias.is_contiguous()):
+            raise ValueError("bias must be a contiguous bfloat16 vector of length N")
+        out = torch.empty((M, N), dtype=torch.bfloat16, device=a_values.device)
+        outs.append(out)
+        structs[i] = GemmProduct(pr["values"].data_ptr(), pr["scales"].data_ptr(), None, pr["amax"].data_ptr(),
+                                 float(pr["denom"]), out.data_ptr(), out.stride(0), _ptr(bias),
+                                 _sink_struct(pr.get("amax_out")))
+    with torch.cuda.device(a_values.device):
+        code = load().ll_nvfp4_gemm_tnt_grouped(a_values.data_ptr(), a_scales.data_ptr(), amax_a.data_ptr(), float(denom_a),
+                                                M, N, Mp, products[0]["values"].shape[0], Kb * 2, len(products),
+                                                ctypes.cast(structs, c_void_p), _stream())
+    _check(code, "ll_nvfp4_gemm_tnt_grouped")
+    return outs
 
 
 # --------------------------------------------------------------------------- KV cache

@@ -92,13 +92,41 @@ struct GemmEpilogue {
   AmaxSink sink;
 };
 
+// Several products with the same A operand and the same N and K in one launch (the q / k / v projections of one
+// activation): the weight, its scales and tensor scale, the bias, the output and the amax sink of the products
+// behind the first one.  The column tiles of all products form one row of tiles_n tiles, tiles_n_each per product.
+constexpr int kMaxGemmGroups = 4;
+struct GemmGroup {
+  const uint8_t* Bv;
+  const uint8_t* Bs;
+  const float* alpha;
+  const float* amax_b;
+  float inv_denom_b;
+  uint16_t* D;
+  int64_t ldd;
+  const uint16_t* bias;
+  AmaxSink sink;
+};
+struct GemmGroups {
+  int n;             // number of products (1: the plain call, `more` unused)
+  int tiles_n_each;  // column tiles per product
+  GemmGroup more[kMaxGemmGroups - 1];
+};
+
 template <int FA, int FB>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
-    const uint8_t* __restrict__ Av, const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bv,
-    const uint8_t* __restrict__ Bs, const float* __restrict__ alpha_ptr, const float* __restrict__ amax_a,
-    const float* __restrict__ amax_b, float inv_denom_a, float inv_denom_b, int M, int N, int Mp, int Np, int Kp,
-    uint16_t* __restrict__ D, int64_t ldd, int tiles_m, int tiles_n, GemmEpilogue epi) {
+    const uint8_t* __restrict__ Av, const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bv0,
+    const uint8_t* __restrict__ Bs0, const float* __restrict__ alpha_ptr0, const float* __restrict__ amax_a,
+    const float* __restrict__ amax_b0, float inv_denom_a, float inv_denom_b0, int M, int N, int Mp, int Np, int Kp,
+    uint16_t* __restrict__ D0, int64_t ldd0, int tiles_m, int tiles_n, GemmEpilogue epi, GemmGroups groups) {
   using S = GemmSmem<FA, FB>;
+  const uint8_t* __restrict__ Bv = Bv0;
+  const uint8_t* __restrict__ Bs = Bs0;
+  const float* __restrict__ alpha_ptr = alpha_ptr0;
+  const float* __restrict__ amax_b = amax_b0;
+  float inv_denom_b = inv_denom_b0;
+  uint16_t* __restrict__ D = D0;
+  int64_t ldd = ldd0;
   const uint16_t* __restrict__ bias = epi.bias;
   const int act = epi.act;
   constexpr int BM = S::BM, BN = S::BN;
@@ -130,6 +158,22 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
       const int c = in_band / rows_in_band;
       tile_m = band * kBandRows + (in_band - c * rows_in_band);
       tile_n = xcd * panels + c;
+    }
+  }
+  if (groups.n > 1) {  // which product this column tile belongs to (uniform over the workgroup)
+    const int g = tile_n / groups.tiles_n_each;
+    tile_n -= g * groups.tiles_n_each;
+    if (g > 0) {
+      const GemmGroup& gg = groups.more[g - 1];
+      Bv = gg.Bv;
+      Bs = gg.Bs;
+      alpha_ptr = gg.alpha;
+      amax_b = gg.amax_b;
+      inv_denom_b = gg.inv_denom_b;
+      D = gg.D;
+      ldd = gg.ldd;
+      bias = gg.bias;
+      epi.sink = gg.sink;
     }
   }
   const int row0 = tile_m * BM;  // first row of A (output row)
@@ -480,18 +524,24 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
 template <int FA, int FB>
 int launch_gemm(const uint8_t* Av, const uint8_t* As, const uint8_t* Bv, const uint8_t* Bs, const float* alpha,
                 const float* amax_a, const float* amax_b, float denom_a, float denom_b, int M, int N, int Mp, int Np,
-                int Kp, void* D, int64_t ldd, const GemmEpilogue& epi, hipStream_t stream) {
+                int Kp, void* D, int64_t ldd, const GemmEpilogue& epi, GemmGroups groups, hipStream_t stream) {
   using S = GemmSmem<FA, FB>;
-  const int tiles_m = (M + S::BM - 1) / S::BM, tiles_n = (N + S::BN - 1) / S::BN;
+  groups.tiles_n_each = (N + S::BN - 1) / S::BN;
+  const int tiles_m = (M + S::BM - 1) / S::BM, tiles_n = groups.tiles_n_each * groups.n;
   const size_t smem = 2 * S::kStage;
   static std::atomic<uint64_t> lds_allowed{0};  // one per tile configuration
   if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_w4a4_kernel<FA, FB>), smem, lds_allowed, "ll_nvfp4_gemm_tnt")) return rc;
   hipLaunchKernelGGL((gemm_w4a4_kernel<FA, FB>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kGemmThreads), smem, stream,
                      Av, As, Bv, Bs, alpha, amax_a, amax_b, 1.0f / denom_a, 1.0f / denom_b, M, N, Mp, Np, Kp,
-                     static_cast<uint16_t*>(D), ldd, tiles_m, tiles_n, epi);
+                     static_cast<uint16_t*>(D), ldd, tiles_m, tiles_n, epi, groups);
   LL_CHECK_LAUNCH("gemm_w4a4_kernel");
   return LL_OK;
 }
+
+int dispatch_gemm(const uint8_t* A_values, const uint8_t* A_scales, const uint8_t* B_values, const uint8_t* B_scales,
+                  const float* alpha, const float* amax_a, const float* amax_b, float denom_a, float denom_b, int64_t M,
+                  int64_t N, int64_t Mp, int64_t Np, int64_t Kp, void* D, int64_t ldd, const GemmEpilogue& epi,
+                  const GemmGroups& groups, hipStream_t s);
 
 }  // namespace ll
 
@@ -561,12 +611,24 @@ extern "C" int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A
              "ll_nvfp4_gemm_tnt: operands must be 16-byte aligned");
   LL_REQUIRE((reinterpret_cast<uintptr_t>(D) & 1) == 0 && (!bias || (reinterpret_cast<uintptr_t>(bias) & 1) == 0),
              "ll_nvfp4_gemm_tnt: D and bias must be 2-byte aligned");
-  hipStream_t s = static_cast<hipStream_t>(stream);
+  GemmGroups groups{};
+  groups.n = 1;
+  return dispatch_gemm(A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, M, N, Mp, Np, Kp,
+                       D, ldd, epi, groups, static_cast<hipStream_t>(stream));
+}
+
+namespace ll {
+// Tile choice and launch; `groups.n` products side by side count as one product of groups.n * N columns.
+int dispatch_gemm(const uint8_t* A_values, const uint8_t* A_scales, const uint8_t* B_values, const uint8_t* B_scales,
+                  const float* alpha, const float* amax_a, const float* amax_b, float denom_a, float denom_b, int64_t M,
+                  int64_t N, int64_t Mp, int64_t Np, int64_t Kp, void* D, int64_t ldd, const GemmEpilogue& epi,
+                  const GemmGroups& groups, hipStream_t s) {
+  const int64_t n_all = N * groups.n;
   // Tile choice.  Two workgroups are resident per CU (512 slots on 256 CUs).  The 256x128 / 128x256
   // tiles need 6 decode instructions per MFMA, the 128x128 tile 8, so the larger tiles win unless
   // they fill the slots in whole rounds much worse.
   auto rounds_eff = [&](int bm, int bn) {
-    const double tiles = (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn);
+    const double tiles = (double)((M + bm - 1) / bm) * (double)((N + bn - 1) / bn) * groups.n;
     const double rounds = (double)(int64_t)((tiles + 511.0) / 512.0);
     return tiles / (512.0 * rounds);
   };
@@ -584,7 +646,7 @@ extern "C" int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A
   // Small problems: when even 128x128 tiles would occupy at most half of the CUs, 64x64 tiles (more decode
   // work per MFMA, but four times the workgroups) finish sooner.  Configuration 3 (64x128) is only reachable
   // through the override below.
-  if (((M + 127) / 128) * ((N + 127) / 128) <= 128) best = 4;
+  if (((M + 127) / 128) * ((n_all + 127) / 128) <= 128) best = 4;
   // Tuning aid: LL_GEMM_TILE=0..4 in the environment when the library is first used pins one tile configuration.
   static const int forced_tile = [] {
     const char* force = getenv("LL_GEMM_TILE");
@@ -593,7 +655,7 @@ extern "C" int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A
   }();
   if (forced_tile >= 0) best = forced_tile;
 #define LL_GEMM_ARGS A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, (int)M, (int)N, \
-                     (int)Mp, (int)Np, (int)Kp, D, ldd, epi, s
+                     (int)Mp, (int)Np, (int)Kp, D, ldd, epi, groups, s
   switch (best) {
     case 0: return launch_gemm<4, 2>(LL_GEMM_ARGS);
     case 1: return launch_gemm<2, 4>(LL_GEMM_ARGS);
@@ -602,4 +664,53 @@ extern "C" int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A
     default: return launch_gemm<1, 1>(LL_GEMM_ARGS);
   }
 #undef LL_GEMM_ARGS
+}
+}  // namespace ll
+
+extern "C" int ll_nvfp4_gemm_tnt_grouped(const uint8_t* A_values, const uint8_t* A_scales, const float* amax_a,
+                                         float denom_a, int64_t M, int64_t N, int64_t Mp, int64_t Np, int64_t Kp,
+                                         int n_products, const ll_gemm_product* products, void* stream) {
+  using namespace ll;
+  LL_REQUIRE(products && n_products >= 1 && n_products <= kMaxGemmGroups,
+             "ll_nvfp4_gemm_tnt_grouped: 1 to %d products, got %d", kMaxGemmGroups, n_products);
+  LL_REQUIRE(A_values && A_scales, "ll_nvfp4_gemm_tnt_grouped: null pointer");
+  LL_REQUIRE(M > 0 && N > 0 && Mp % 128 == 0 && Np % 128 == 0 && Kp % 64 == 0 && Kp > 0 && M <= Mp && N <= Np,
+             "ll_nvfp4_gemm_tnt_grouped: bad shape M=%lld N=%lld Mp=%lld Np=%lld Kp=%lld", (long long)M, (long long)N,
+             (long long)Mp, (long long)Np, (long long)Kp);
+  LL_REQUIRE(Mp < (1 << 30) && Np * n_products < (1 << 30) && Kp < (1 << 30), "ll_nvfp4_gemm_tnt_grouped: dimension too large");
+  LL_REQUIRE(((reinterpret_cast<uintptr_t>(A_values) | reinterpret_cast<uintptr_t>(A_scales)) & 15) == 0,
+             "ll_nvfp4_gemm_tnt_grouped: operands must be 16-byte aligned");
+  GemmGroups groups{};
+  groups.n = n_products;
+  GemmEpilogue epi{};
+  for (int i = 0; i < n_products; ++i) {
+    const ll_gemm_product& pr = products[i];
+    LL_REQUIRE(pr.B_values && pr.B_scales && pr.D && pr.ldd >= N, "ll_nvfp4_gemm_tnt_grouped: product %d: null pointer or ldd < N", i);
+    LL_REQUIRE(pr.alpha || (amax_a && pr.amax_b && denom_a > 0.f && pr.denom_b > 0.f),
+               "ll_nvfp4_gemm_tnt_grouped: product %d: pass alpha, or both amax pointers with positive denominators", i);
+    LL_REQUIRE(((reinterpret_cast<uintptr_t>(pr.B_values) | reinterpret_cast<uintptr_t>(pr.B_scales)) & 15) == 0,
+               "ll_nvfp4_gemm_tnt_grouped: product %d: operands must be 16-byte aligned", i);
+    LL_REQUIRE((reinterpret_cast<uintptr_t>(pr.D) & 1) == 0 && (!pr.bias || (reinterpret_cast<uintptr_t>(pr.bias) & 1) == 0),
+               "ll_nvfp4_gemm_tnt_grouped: product %d: D and bias must be 2-byte aligned", i);
+    LL_REQUIRE(sink_is_valid(&pr.amax_sink), "ll_nvfp4_gemm_tnt_grouped: product %d: amax sink needs 8-byte alignment and a non-zero epoch", i);
+    if (i == 0) {
+      epi.bias = static_cast<const uint16_t*>(pr.bias);
+      epi.sink = make_sink(&pr.amax_sink);
+    } else {
+      GemmGroup& g = groups.more[i - 1];
+      g.Bv = pr.B_values;
+      g.Bs = pr.B_scales;
+      g.alpha = pr.alpha;
+      g.amax_b = pr.amax_b;
+      g.inv_denom_b = pr.denom_b > 0.f ? 1.0f / pr.denom_b : 0.f;
+      g.D = static_cast<uint16_t*>(pr.D);
+      g.ldd = pr.ldd;
+      g.bias = static_cast<const uint16_t*>(pr.bias);
+      g.sink = make_sink(&pr.amax_sink);
+    }
+  }
+  const ll_gemm_product& p0 = products[0];
+  return dispatch_gemm(A_values, A_scales, p0.B_values, p0.B_scales, p0.alpha, amax_a, p0.amax_b, denom_a,
+                       p0.denom_b > 0.f ? p0.denom_b : 1.f, M, N, Mp, Np, Kp, p0.D, p0.ldd, epi, groups,
+                       static_cast<hipStream_t>(stream));
 }

@@ -80,8 +80,8 @@ def _project_shared(x: torch.Tensor, layers, amax: torch.Tensor | None = None, a
     if all(isinstance(m, FourOverSixLinear) for m in layers) and all(
             m.config.get_activation_config() == first.config.get_activation_config() for m in layers):
         xq = first.quantize_input(x.reshape(-1, x.shape[-1]), amax=amax)
-        outs = amax_outs or [None] * len(layers)
-        return [m.forward_quantized(xq, amax_out=t).reshape(*x.shape[:-1], -1) for m, t in zip(layers, outs)], True
+        outs = FourOverSixLinear.forward_quantized_together(layers, xq, amax_outs)
+        return [y.reshape(*x.shape[:-1], -1) for y in outs], True
     return [m(x) for m in layers], False
 
 

@@ -129,6 +129,31 @@ class FourOverSixLinear(nn.Linear):
         the amax ticket of the kernel that produced ``x2d``, if it was given one."""
         return quantize_to_fp4(x2d, self.config.get_activation_config(), amax=amax)
 
+    @staticmethod
+    def forward_quantized_together(layers, xq: QuantizedTensor, amax_outs=None) -> list[torch.Tensor]:
+        """``[m.forward_quantized(xq) for m in layers]`` as one GEMM launch when the layers have the same shape
+        (the q / k / v projections of an attention layer): the products are computed exactly as they would be
+        alone, only the cost of two launches and of two half-empty rounds of workgroups is saved.  ``amax_outs``:
+        one amax ticket or ``None`` per layer."""
+        from .... import _native
+
+        amax_outs = amax_outs or [None] * len(layers)
+        weights = [m.quantized_weight() for m in layers]
+        same = (1 < len(layers) <= 4 and all(isinstance(w, QuantizedTensor) for w in weights)
+                and all(w.values.shape == weights[0].values.shape and w.original_shape == weights[0].original_shape
+                        and w.dtype == xq.dtype for w in weights)
+                and weights[0].original_shape[1] == xq.original_shape[1]
+                and all(m.bias is None or m.bias.dtype == torch.bfloat16 for m in layers)
+                # two tickets of one sink buffer cannot be served by one launch: the later epoch would hide the earlier
+                and len({t.parts.data_ptr() for t in amax_outs if t is not None}) == sum(t is not None for t in amax_outs))
+        if not same:
+            return [m.forward_quantized(xq, amax_out=t) for m, t in zip(layers, amax_outs)]
+        denom = lambda q: float(q.scale_rule.max_allowed_e2m1_value() * q.scale_rule.max_allowed_e4m3_value())
+        products = [dict(values=w.values, scales=w.scale_factors, amax=w.amax, denom=denom(w), bias=m.bias, amax_out=t)
+                    for m, w, t in zip(layers, weights, amax_outs)]
+        return _native.gemm_grouped(xq.values, xq.scale_factors, xq.amax, denom(xq), xq.original_shape[0],
+                                    weights[0].original_shape[0], products)
+
     def forward_quantized(self, xq: QuantizedTensor, activation: str | None = None, *,
                           residual: torch.Tensor | None = None, gate: torch.Tensor | None = None,
                           gate_rows: int = 0, amax_out=None) -> torch.Tensor:

@@ -277,6 +277,53 @@ def test_amax_sink_of_the_epilogue_feeds_the_next_quantization(gpu):
             assert torch.equal(via_sink.scale_factors.view(torch.uint8), direct.scale_factors.view(torch.uint8))
 
 
+@pytest.mark.parametrize("M,N,K,n", [(264, 384, 256, 3), (300, 200, 192, 2), (64, 128, 64, 4), (2640, 3072, 3072, 3),
+                                     (512, 3072, 3072, 2)])
+def test_products_that_share_their_input_in_one_launch_equal_the_separate_launches(gpu, M, N, K, n):
+    """ll_nvfp4_gemm_tnt_grouped (the q / k / v projections of one activation): every product - own weight, tensor
+    scale, bias and amax sink - is bit for bit what the single call computes, at ragged and at full sizes; the
+    quantized linear layers take that path through forward_quantized_together."""
+    from longlive_amd import _native
+    cfg = QuantizationConfig(scale_rule="mse")
+    xq = quantize_to_fp4(activations((M, K), 61).to(gpu), cfg)
+    ws = [quantize_to_fp4((weights((N, K), 62 + i) * (1 + i)).to(gpu), cfg) for i in range(n)]
+    biases = [None if i == 1 else (torch.randn(N, generator=torch.Generator().manual_seed(70 + i)) * 0.1).bfloat16().to(gpu)
+              for i in range(n)]
+    alone, alone_tickets = [], []
+    for w, b in zip(ws, biases):
+        t = _native.amax_ticket(gpu)
+        y = fp4_matmul(xq, w, bias=b, amax_out=t)
+        alone.append(y)
+        alone_tickets.append(float(quantize_to_fp4(y, cfg, amax=t).amax))
+    tickets = [_native.PrivateAmaxSink(gpu) for _ in range(n)]   # each product needs a sink of its own here: one launch
+    products = [dict(values=w.values, scales=w.scale_factors, amax=w.amax, denom=1536.0, bias=b, amax_out=s.ticket())
+                for w, b, s in zip(ws, biases, tickets)]
+    together = _native.gemm_grouped(xq.values, xq.scale_factors, xq.amax, 1536.0, M, N, products)
+    for i in range(n):
+        assert torch.equal(together[i], alone[i]), i
+        got = float(quantize_to_fp4(together[i], cfg, amax=products[i]["amax_out"]).amax)
+        assert got == alone_tickets[i] == float(alone[i].abs().max())
+    with pytest.raises(ValueError):     # more than four products
+        _native.gemm_grouped(xq.values, xq.scale_factors, xq.amax, 1536.0, M, N, [dict(p, amax_out=None) for p in products] * 3)
+    with pytest.raises(ValueError):     # two products on one sink buffer
+        _native.gemm_grouped(xq.values, xq.scale_factors, xq.amax, 1536.0, M, N,
+                             [dict(p, amax_out=tickets[0].ticket()) for p in products[:2]])
+
+
+def test_quantized_layers_with_one_input_run_as_one_launch(gpu):
+    lin = [nn.Linear(256, 384).to(gpu).bfloat16() for _ in range(3)]
+    holder = nn.Sequential(*lin)
+    holder, _ = quantize_model_with_filter(holder, ModelQuantizationConfig(), use_default_filtered_modules=False,
+                                           materialize_for_inference=True, verbose=False)
+    layers = list(holder)
+    assert all(isinstance(m, FourOverSixLinear) for m in layers)
+    x = activations((130, 256), 81).to(gpu)
+    xq = layers[0].quantize_input(x)
+    together = FourOverSixLinear.forward_quantized_together(layers, xq)
+    for m, y in zip(layers, together):
+        assert torch.equal(y, m.forward_quantized(xq)) and torch.equal(y, m(x))
+
+
 @pytest.mark.gpu
 def test_ffn_down_full_size_fused_epilogue_and_sink(gpu):
     """The FFN pair at the benchmark size: GELU + amax sink in the up projection, gated residual in the down

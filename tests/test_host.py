@@ -41,6 +41,7 @@ def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
                                        1, ctypes.byref(gated), None) == -1
     assert b"a gate needs a residual" in lib.ll_last_error()
     assert ctypes.sizeof(_native.GemmEpilogue) == 80 and ctypes.sizeof(_native.AmaxSinkStruct) == 24
+    assert ctypes.sizeof(_native.GemmProduct) == 88
     assert lib.ll_amax_epoch_advance(None, 1, None, None) == -1 and b"epoch_offset" in lib.ll_last_error()
 
 
