@@ -247,12 +247,13 @@ class DiTBlock(nn.Module):
         return _project_out(down, h, h_amax, residual, gate, gate_rows)
 
     def forward(self, x, e, cos, sin, context, kv_cache, current_start, sink_tokens, max_attention_size=None,
-                crossattn_cache=None, global_sink_tokens=0, rope_fn=None, collect_kv_amax=True):
+                crossattn_cache=None, global_sink_tokens=0, rope_fn=None, collect_kv_amax=True, modulated=None):
         """x [1, L, C]; e [1, F, 6, C]; returns (x, (current_end, local_end_index, cache_update_info)).
         The tensor amax that each activation quantization needs is produced by the kernel that writes the
-        activation wherever that kernel is one of this package's."""
+        activation wherever that kernel is one of this package's.  ``modulated`` is ``self.modulation.unsqueeze(1)
+        + e`` when the caller has already formed it (the model does so for all its blocks in one operation)."""
         num_frames, frame_seqlen = e.shape[1], x.shape[1] // e.shape[1]
-        e = (self.modulation.unsqueeze(1) + e).chunk(6, dim=2)
+        e = (self.modulation.unsqueeze(1) + e if modulated is None else modulated).chunk(6, dim=2)
         gates = [g.reshape(-1, g.shape[-1]) for g in (e[2], e[5])]  # [B*F, C] views, one row per frame
         y_amax = _native.amax_ticket(x.device) if isinstance(self.self_attn.q, FourOverSixLinear) else None
         y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.eps, amax_out=y_amax)
@@ -355,6 +356,16 @@ class CausalDiT(nn.Module):
         u = torch.einsum("fhwpqrc->cfphqwr", u)
         return u.reshape(c, *[i * j for i, j in zip(grid, self.cfg.patch_size)])
 
+    def _stacked_modulation(self) -> torch.Tensor:
+        """The blocks' modulation parameters as one [blocks, 1, 6, C] tensor, rebuilt when a parameter has been
+        replaced or written (inference keeps it)."""
+        key = tuple((b.modulation.data_ptr(), b.modulation._version) for b in self.blocks)
+        cached = getattr(self, "_modulation_stack", None)
+        if cached is None or cached[0] != key:
+            cached = (key, torch.stack([b.modulation.detach() for b in self.blocks]))
+            self._modulation_stack = cached
+        return cached[1]
+
     @torch.no_grad()
     def forward(self, x: torch.Tensor, t: torch.Tensor, context: torch.Tensor, kv_cache: list[dict],
                 current_start: int, apply_cache_updates: bool = True,
@@ -376,12 +387,14 @@ class CausalDiT(nn.Module):
         sink_tokens = cfg.sink_size * frame_seqlen
         max_attn = cfg.local_attn_size * frame_seqlen
         updates = []
+        # modulation + e0 of every block in one operation (the same additions and roundings as block by block)
+        modulated = self._stacked_modulation().unsqueeze(2) + e0.unsqueeze(0)   # [blocks, 1, F, 6, C]
         for i, block in enumerate(self.blocks):
             x, upd = block(x, e0, cos, sin, ctx, kv_cache[i], current_start, sink_tokens, max_attn,
                            None if crossattn_cache is None else crossattn_cache[i],
                            global_sink_tokens=self.global_sink_size * frame_seqlen,
                            rope_fn=lambda frames, first: self._rope(frames, h, w, first, x.device),
-                           collect_kv_amax=apply_cache_updates)
+                           collect_kv_amax=apply_cache_updates, modulated=modulated[i])
             updates.append(upd)
         if apply_cache_updates:
             for i, (cur_end, loc_end, info) in enumerate(updates):

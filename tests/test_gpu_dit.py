@@ -671,6 +671,39 @@ def test_head_modulation_through_the_adaln_kernel_matches_the_eager_graph(gpu):
     assert (got.float() - ref.float()).abs().max() <= 2.0 ** -6 * ref.float().abs().max()
 
 
+def test_modulation_of_all_blocks_in_one_operation_is_what_each_block_would_form(gpu):
+    """The model adds its blocks' modulation parameters to the time projection in one operation per forward; each
+    slice is bit for bit the block's own ``modulation.unsqueeze(1) + e``, follows a parameter that is written in
+    place, and the generated latents are those of the block-by-block path."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=3, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    gen = StreamingGenerator(cfg, gpu, seed=9)
+    model = gen.model
+    g = torch.Generator().manual_seed(9)
+    e0 = torch.randn(1, 2, 6, 256, generator=g).to(gpu).to(model.blocks[0].modulation.dtype)
+    with torch.no_grad():
+        for _ in range(2):
+            stacked = model._stacked_modulation().unsqueeze(2) + e0.unsqueeze(0)
+            for i, b in enumerate(model.blocks):
+                assert torch.equal(stacked[i], b.modulation.unsqueeze(1) + e0)
+            model.blocks[1].modulation.mul_(2.0)          # an in-place write must not leave a stale stack behind
+    noise = torch.randn(1, 4, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    out = gen.generate(noise, ctx)
+    gen2 = StreamingGenerator(cfg, gpu, seed=9)
+    with torch.no_grad():
+        gen2.model.blocks[1].modulation.mul_(4.0)
+    block_forward = DiTBlock.forward
+    def per_block(self, *args, modulated=None, **kwargs):   # the path without the stacked tensor
+        return block_forward(self, *args, modulated=None, **kwargs)
+    DiTBlock.forward = per_block
+    try:
+        ref = gen2.generate(noise, ctx)
+    finally:
+        DiTBlock.forward = block_forward
+    assert torch.equal(out, ref)
+
+
 def test_block_forward_recorded_into_a_graph_replays_bit_for_bit(gpu):
     """One DiT block forward over an FP4 cache slot recorded into a HIP graph (27 kernels of the library, seven amax
     tickets) and replayed with new inputs.  A recorded launch runs again with the epoch it was recorded with, so
