@@ -380,8 +380,11 @@ class CausalDiT(nn.Module):
         tt = t.flatten()
         e = self.time_embedding(sinusoidal_embedding_1d(cfg.freq_dim, tt).unflatten(0, t.shape).type_as(x))
         e0 = self.time_projection(e).unflatten(2, (6, cfg.dim))
-        ctx = torch.cat([context, context.new_zeros(cfg.text_len - context.size(0), context.size(1))]).unsqueeze(0)
-        ctx = self.text_embedding(ctx)
+        if crossattn_cache is not None and all(c.get("is_init") for c in crossattn_cache):
+            ctx = None  # every layer holds the projected K / V of this prompt: the text embedding has no reader
+        else:
+            ctx = torch.cat([context, context.new_zeros(cfg.text_len - context.size(0), context.size(1))]).unsqueeze(0)
+            ctx = self.text_embedding(ctx)
         # the multi-shot phase offset applies to absolute positions only (causal_model.py:478-486, 1588)
         cos, sin = self._rope(f, h, w, current_start // frame_seqlen, x.device, self.rope_temporal_offset)
         sink_tokens = cfg.sink_size * frame_seqlen
