@@ -14,7 +14,7 @@ import torch
 
 from .. import _native
 from ..fouroversix import QuantizationConfig, QuantizedTensor, quantize_to_fp4
-from .quant import SlotPointerTable, clone_quantized_tensor, copy_quantized_into, k_smooth
+from .quant import SlotPointerTable, clone_quantized_tensor, k_smooth
 
 
 def initialize_kv_cache(num_layers: int, block_token_size: int, max_blocks: int, num_heads: int, head_dim: int,
@@ -51,12 +51,15 @@ def initialize_kv_cache(num_layers: int, block_token_size: int, max_blocks: int,
 
 
 def _tables_for(cache: dict, slot_ids: tuple[int, ...]):
-    entry = cache["_tables"].get(slot_ids)
+    # keyed by the buffers, not by the positions: a roll moves the buffers through the positions (apply_cache_update),
+    # and the handful of arrangements that a streaming run cycles through are each built once
+    key = tuple(cache["k"][i].values.data_ptr() for i in slot_ids)
+    entry = cache["_tables"].get(key)
     if entry is None:
         kt = SlotPointerTable([cache["k"][i] for i in slot_ids])
         vt = SlotPointerTable([cache["v"][i] for i in slot_ids])
         entry = (kt, vt)
-        cache["_tables"][slot_ids] = entry
+        cache["_tables"][key] = entry
     return entry
 
 
@@ -209,15 +212,24 @@ def kv_cache_attention_relative(q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
 
 def apply_cache_update(cache: dict, current_end: int, local_end_index: int, info: dict | None,
                        kv_quant_config: QuantizationConfig) -> None:
-    """Roll whole slots and quantize the chunk's K / V into their slots, in place."""
+    """Roll whole slots and quantize the chunk's K / V into their slots, in place.
+
+    The reference rolls by copying slot contents forward (causal_model.py:1404-1409) so that slot addresses stay
+    put for its CUDA graphs.  The attention kernel here reads the slots through a pointer table, so a roll moves
+    the slot buffers through the list instead - the evicted buffers go behind the rolled ones, where the chunk is
+    written next - and nothing is copied (18 small device copies per layer and roll otherwise).  Position i of
+    ``cache["k"]`` / ``cache["v"]`` holds the same data as after the reference's copies wherever that data is
+    meaningful."""
     if info is not None:
         blk = cache["block_token_size"]
         if info["action"] == "roll_and_insert":
             sink_b = info["sink_tokens"] // blk
             ev_b = info["num_evicted_tokens"] // blk
-            for i in range(info["num_rolled_tokens"] // blk):
-                copy_quantized_into(cache["k"][sink_b + i], cache["k"][sink_b + ev_b + i])
-                copy_quantized_into(cache["v"][sink_b + i], cache["v"][sink_b + ev_b + i])
+            n_roll = info["num_rolled_tokens"] // blk
+            for name in ("k", "v"):
+                slots = cache[name]
+                slots[sink_b:sink_b + ev_b + n_roll] = (slots[sink_b + ev_b:sink_b + ev_b + n_roll]
+                                                       + slots[sink_b:sink_b + ev_b])
             if info.get("pinned_shift", 0) > 0:  # a floating pinned region moves with the data (:1437-1443)
                 cache["pinned_start"].sub_(info["pinned_shift"])
                 cache["_pinned_start"] -= info["pinned_shift"]
