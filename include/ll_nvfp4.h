@@ -242,8 +242,10 @@ int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads,
  *                        workgroups pass through device memory that the library allocates on the first such
  *                        launch on a (device, stream) pair and keeps (69 MB on a 256-CU device); launches that
  *                        use it must not overlap on one stream's memory, which same-stream order guarantees.
- * The three give the same result up to the order of fp32 additions (each is deterministic).  Callers that must
- * not allocate during a launch (graph capture) select NARROW or WIDE.  The setting is process-wide.
+ * The three give the same result up to the order of fp32 additions (each is deterministic).  The setting is
+ * process-wide.  A launch on a stream that is being captured into a graph never allocates: it uses the memory an
+ * earlier launch or ll_kv_attention_reserve left on that stream, and without such memory the automatic choice
+ * takes the cheaper of NARROW and WIDE while an explicit LL_ATTENTION_SPLIT returns LL_ENOSUP.
  */
 #define LL_ATTENTION_AUTO (-1)
 #define LL_ATTENTION_NARROW 0
@@ -251,6 +253,15 @@ int ll_kv_attention_amax(const void* q, int64_t Lq, int num_heads,
 #define LL_ATTENTION_SPLIT 2
 int ll_kv_attention_set_policy(int policy); /* LL_OK, or LL_EINVAL for an unknown policy */
 int ll_kv_attention_get_policy(void);
+/* Sets up, on (current device, stream), the memory that a launch of Lq queries x num_heads heads over n_keys keys
+ * would need under the current policy (nothing when that launch would not take the split division), so that the
+ * launch itself allocates nothing: call it ahead of a graph recording or a latency-critical loop.  May allocate,
+ * and may free a smaller set (which waits for the device).  LL_ENOSUP while the stream is being captured.  No
+ * counterpart in the reference. */
+int ll_kv_attention_reserve(int64_t Lq, int num_heads, int64_t n_keys, void* stream);
+/* Frees the memory the split division holds for (current device, stream), if any; waits for the launches that
+ * still use it.  For callers that create streams as they go: the library keeps one set per stream it has seen. */
+int ll_kv_attention_release(void* stream);
 /* What a launch of Lq queries x num_heads heads over n_keys keys would do on a device with `compute_units` CUs
  * under `policy` (pure host arithmetic, no GPU needed): the division taken (an LL_ATTENTION_SPLIT request falls
  * back to WIDE when there is nothing to split), the number of workgroups, the whole rounds of tiles all of them

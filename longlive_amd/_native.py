@@ -73,6 +73,8 @@ _SIGNATURES = {
                                  c_void_p, c_void_p]),
     "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
     "ll_layer_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p]),
+    "ll_kv_attention_reserve": (c_int, [c_int64, c_int, c_int64, c_void_p]),
+    "ll_kv_attention_release": (c_int, [c_void_p]),
     "ll_nvfp4_quantize_noalloc_max_elements": (c_int64, []),
     "ll_nvfp4_quantize_noalloc": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p,
                                           c_void_p]),
@@ -495,6 +497,20 @@ def attention_plan(Lq: int, num_heads: int, n_keys: int, compute_units: int = 25
     names = {v: k for k, v in ATTENTION_POLICIES.items()}
     return {"division": names[division.value], "workgroups": groups.value, "whole_rounds": rounds.value,
             "split_tiles": split.value}
+
+
+def attention_reserve(Lq: int, num_heads: int, n_keys: int, device=None) -> None:
+    """Set up, on the current stream, the memory an attention launch of these sizes would pass partial tiles
+    through (nothing if it would not split), so that the launch itself - for instance inside a graph recording -
+    allocates nothing."""
+    with torch.cuda.device(device if device is not None else torch.cuda.current_device()):
+        _check(load().ll_kv_attention_reserve(Lq, num_heads, n_keys, _stream()), "ll_kv_attention_reserve")
+
+
+def attention_release(device=None) -> None:
+    """Free the memory the split division holds for the current stream, if any."""
+    with torch.cuda.device(device if device is not None else torch.cuda.current_device()):
+        _check(load().ll_kv_attention_release(_stream()), "ll_kv_attention_release")
 
 
 class attention_policy:

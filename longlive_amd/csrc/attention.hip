@@ -674,7 +674,11 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
           store_shared_f32(mine + 64 * 64, m_run);
           store_shared_f32(mine + 65 * 64, l_run);
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");  // the stores have left before the arrival is counted
+        // Every wave waits until its own record stores are complete (vmcnt(0): a write-through store is
+        // acknowledged once it is visible device-wide) before it reaches the barrier; thread 0 counts the arrival
+        // behind that barrier, so no workgroup can see the count without the whole record being in memory.
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
         if (tid == 0)
           tab.last_arrival = __hip_atomic_fetch_add(c.arrivals + split_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
@@ -790,8 +794,21 @@ struct SplitWorkspace {
 static std::mutex g_split_mutex;
 static std::map<std::pair<int, hipStream_t>, SplitWorkspace> g_split_workspaces;
 
-static int split_workspace(int dev, hipStream_t stream, uint32_t groups, int tiles, SplitWorkspace& out) {
+// `may_allocate` false (the stream is being captured into a graph): only a set that is already large enough is
+// handed out; *missing tells the caller that there is none.
+static int split_workspace(int dev, hipStream_t stream, uint32_t groups, int tiles, bool may_allocate, SplitWorkspace& out,
+                           bool* missing) {
   std::lock_guard<std::mutex> lock(g_split_mutex);
+  if (missing) *missing = false;
+  if (!may_allocate) {
+    const auto it = g_split_workspaces.find({dev, stream});
+    if (it == g_split_workspaces.end() || it->second.groups < groups || it->second.tiles < tiles) {
+      if (missing) *missing = true;
+      return LL_OK;
+    }
+    out = it->second;
+    return LL_OK;
+  }
   SplitWorkspace& w = g_split_workspaces[{dev, stream}];
   if (w.groups < groups || w.tiles < tiles) {
     if (w.partials) (void)hipFree(w.partials);  // waits for the launches that still use it
@@ -806,7 +823,7 @@ static int split_workspace(int dev, hipStream_t stream, uint32_t groups, int til
                 (size_t)2 * groups * kPartialFloats * sizeof(float), hipGetErrorString(e));
       if (w.partials) (void)hipFree(w.partials);
       if (w.arrivals) (void)hipFree(w.arrivals);
-      w = SplitWorkspace{};
+      g_split_workspaces.erase({dev, stream});
       return LL_ELAUNCH;
     }
     w.groups = groups;
@@ -814,6 +831,27 @@ static int split_workspace(int dev, hipStream_t stream, uint32_t groups, int til
   }
   out = w;
   return LL_OK;
+}
+
+static int release_split_workspace(int dev, hipStream_t stream) {
+  std::lock_guard<std::mutex> lock(g_split_mutex);
+  const auto it = g_split_workspaces.find({dev, stream});
+  if (it == g_split_workspaces.end()) return LL_OK;
+  if (it->second.partials) (void)hipFree(it->second.partials);  // waits for the launches that still use it
+  if (it->second.arrivals) (void)hipFree(it->second.arrivals);
+  g_split_workspaces.erase(it);
+  return LL_OK;
+}
+
+// Whether work submitted to `stream` is being recorded into a graph instead of run.  A failing query (the legacy
+// stream while another stream of the thread captures) counts as recording: then nothing may be allocated either.
+static bool stream_is_capturing(hipStream_t stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;
+  }
+  return status != hipStreamCaptureStatusNone;
 }
 
 static std::atomic<int> g_attention_policy{LL_ATTENTION_AUTO};
@@ -848,7 +886,27 @@ static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
   if (int rc = compute_units_of(dev, cus)) return rc;
   const int64_t n_iter = (p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys;
   LL_REQUIRE(p.H * ((p.Lq + kWgQueries - 1) / kWgQueries) * n_iter < (1ll << 32), "ll_kv_attention: too many (tile, iteration) units");
-  const AttentionPlan plan = plan_attention(p.Lq, p.H, p.n_cached + p.n_new, cus, g_attention_policy.load(std::memory_order_relaxed));
+  const int policy = g_attention_policy.load(std::memory_order_relaxed);
+  AttentionPlan plan = plan_attention(p.Lq, p.H, p.n_cached + p.n_new, cus, policy);
+  SplitWorkspace w;
+  if (plan.mode == LL_ATTENTION_SPLIT) {
+    // The split division passes partial tiles through device memory of the library's own.  While the stream is
+    // being captured nothing may be allocated (and the clearing of a new set must not become a graph node): a set
+    // that an earlier launch or ll_kv_attention_reserve left on this stream is used as it is; without one the
+    // automatic choice falls back to the cheaper of the two divisions that need no memory, and an explicit
+    // request for the split division is refused.
+    const bool capturing = stream_is_capturing(stream);
+    bool missing = false;
+    if (int rc = split_workspace(dev, stream, plan.d.G, (int)plan.split_tiles, !capturing, w, &missing)) return rc;
+    if (missing) {
+      if (policy == LL_ATTENTION_SPLIT) {
+        set_error("ll_kv_attention: the split division needs device memory that cannot be allocated while the stream "
+                  "is being captured; call ll_kv_attention_reserve for this shape first, or select another division");
+        return LL_ENOSUP;
+      }
+      plan = plan_attention(p.Lq, p.H, p.n_cached + p.n_new, cus, policy, /*allow_split=*/false);
+    }
+  }
   p.n_qtiles = plan.n_qtiles;
   p.full_qtiles = plan.full_qtiles;
   p.d = plan.d;
@@ -858,8 +916,6 @@ static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
     hipLaunchKernelGGL(kv_attention_kernel<false>, dim3(p.d.G), dim3(kAttnThreads), smem, stream, p);
   } else {
     if (plan.mode == LL_ATTENTION_SPLIT) {
-      SplitWorkspace w;
-      if (int rc = split_workspace(dev, stream, plan.d.G, (int)plan.split_tiles, w)) return rc;
       p.partials = w.partials;
       p.arrivals = w.arrivals;
     }
@@ -880,6 +936,34 @@ extern "C" int ll_kv_attention_set_policy(int policy) {
 }
 
 extern "C" int ll_kv_attention_get_policy(void) { return ll::g_attention_policy.load(); }
+
+extern "C" int ll_kv_attention_reserve(int64_t Lq, int num_heads, int64_t n_keys, void* stream) {
+  using namespace ll;
+  LL_REQUIRE(Lq > 0 && num_heads > 0 && n_keys > 0 && Lq < (1ll << 30) && n_keys < (1ll << 30), "ll_kv_attention_reserve: bad sizes");
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    set_error("ll_kv_attention_reserve: hipGetDevice failed");
+    return LL_ELAUNCH;
+  }
+  if (int rc = compute_units_of(dev, cus)) return rc;
+  const AttentionPlan plan = plan_attention(Lq, num_heads, n_keys, cus, g_attention_policy.load(std::memory_order_relaxed));
+  if (plan.mode != LL_ATTENTION_SPLIT) return LL_OK;
+  if (stream_is_capturing(static_cast<hipStream_t>(stream))) {
+    set_error("ll_kv_attention_reserve: the stream is being captured; reserve before the recording starts");
+    return LL_ENOSUP;
+  }
+  SplitWorkspace w;
+  return split_workspace(dev, static_cast<hipStream_t>(stream), plan.d.G, (int)plan.split_tiles, true, w, nullptr);
+}
+
+extern "C" int ll_kv_attention_release(void* stream) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    ll::set_error("ll_kv_attention_release: hipGetDevice failed");
+    return LL_ELAUNCH;
+  }
+  return ll::release_split_workspace(dev, static_cast<hipStream_t>(stream));
+}
 
 extern "C" int ll_kv_attention_plan(int64_t Lq, int num_heads, int64_t n_keys, int compute_units, int policy,
                                     int* division, uint32_t* workgroups, uint32_t* whole_rounds, int64_t* split_tiles) {

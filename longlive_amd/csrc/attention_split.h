@@ -113,7 +113,9 @@ struct AttentionPlan {
   int64_t split_tiles;  // tiles of the split part
 };
 
-inline AttentionPlan plan_attention(int64_t Lq, int H, int64_t n_keys, int cus, int policy) {
+// `allow_split` false leaves the split division out of the automatic choice (a launch that may not use the memory
+// partial tiles pass through).
+inline AttentionPlan plan_attention(int64_t Lq, int H, int64_t n_keys, int cus, int policy, bool allow_split = true) {
   constexpr double kWideIteration = 1.64;  // an iteration of the 256-query kernel takes this much longer for twice the work
   constexpr double kCombine = 6.0;         // partial results when every workgroup shares: writing, counting, combining
   constexpr double kCombineFew = 1.5;      // the same when only the workgroups without a whole extra tile share
@@ -162,6 +164,7 @@ inline AttentionPlan plan_attention(int64_t Lq, int H, int64_t n_keys, int cus, 
     const Shape a = weigh(full_tiles / cus, full_tiles % cus);
     if (a.cost <= best.cost * 1.04) best = a;
   }
+  if (!allow_split) best.cost = 1e300;
   const double cost_narrow = (double)((tiles_narrow + cus - 1) / cus) * ((double)n_iter + kRound);
   const double cost_wide = (double)((tiles_wide + cus - 1) / cus) * (kWideIteration * (double)n_iter + kRound);
   int mode = cost_narrow <= cost_wide && cost_narrow <= best.cost ? 0 : (cost_wide <= best.cost ? 1 : 2);

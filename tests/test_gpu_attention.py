@@ -301,6 +301,51 @@ def test_layer_norm_against_oracle_and_torch(gpu, L, C, affine):
     assert torch.equal(xq_sink.values, xq_pass.values)
 
 
+def _tile_samples(Lq, H, n_keys):
+    """(kind, head, query rows) samples chosen from the launcher's own plan for a shape: a tile that one workgroup
+    runs whole, a tile whose parts two or more workgroups compute and one of them combines, and a head's last,
+    partly filled group of queries (a "light" tile).  Tile numbering as in the kernel: full tiles first
+    (head * full_qtiles + group), the heads' last groups behind them when they are light."""
+    from helpers import DIVISION_FIELDS, attention_full_plan, attention_parts
+
+    plan = attention_full_plan(Lq, H, n_keys)
+    assert plan["mode"] == 2, plan
+    d = {k: plan[k] for k in DIVISION_FIELDS}
+    n_full = H * plan["full_qtiles"]
+
+    def rows_of(tile):
+        head, group = (tile // plan["full_qtiles"], tile % plan["full_qtiles"]) if tile < n_full else (tile - n_full, plan["full_qtiles"])
+        first, last = group * 256, min(Lq, group * 256 + 256)
+        # both ends of the tile and the boundary between two waves' queries
+        rows = sorted({first, first + 1, first + 31, first + 32, min(first + 127, last - 1), min(first + 128, last - 1), last - 2, last - 1})
+        return head, np.array(rows)
+
+    first_split = plan["whole_rounds"] * plan["G"] + plan["extra"]
+    samples = []
+    if first_split > 0:
+        samples.append(("whole", *rows_of(first_split - 1)))   # the last tile that is run whole (an extra one, if any)
+        samples.append(("whole", *rows_of(first_split // 2)))
+    shared = [t for t in range(plan["split_tiles"]) if len(set(attention_parts(t, d))) == 2]
+    assert shared
+    for t in (shared[0], shared[len(shared) // 2], shared[-1]):
+        tile = first_split + t
+        samples.append(("light+shared" if tile >= n_full else "shared", *rows_of(tile)))
+    if n_full < H * plan["n_qtiles"]:
+        alone = [t for t in range(plan["split_tiles"]) if len(set(attention_parts(t, d))) == 1 and first_split + t >= n_full]
+        for t in alone[:1]:
+            samples.append(("light", *rows_of(first_split + t)))
+    return samples
+
+
+def _check_samples_against_oracle(out, q, k_all, v_all, samples):
+    """fp64-softmax oracle on the sampled query rows (out, q: [Lq, H, 128]; k_all, v_all: [Lk, H, 128])."""
+    for kind, h, rows in samples:
+        want = o.attention(q[rows, h:h + 1].float().cpu().numpy(), k_all[:, h:h + 1].float().cpu().numpy(),
+                           v_all[:, h:h + 1].float().cpu().numpy())
+        err = np.abs(out[rows, h:h + 1].float().cpu().numpy() - want).max()
+        assert err <= 2e-2, (kind, h, rows, err)
+
+
 def test_config3_full_size_fused_decode_equals_attention_over_the_dequantized_cache(gpu):
     """Benchmark shape (24 heads, 2640 queries, 4 FP4 slots of 2640 tokens + the bf16 chunk = 13200 keys):
     the kernel that decodes FP4 on load must agree with plain bf16 attention over the cache dequantized by
@@ -328,6 +373,11 @@ def test_config3_full_size_fused_decode_equals_attention_over_the_dequantized_ca
         want = o.attention(q[0, :16, h:h + 1].float().cpu().numpy(), k_all[:, h:h + 1].float().cpu().numpy(),
                            v_all[:, h:h + 1].float().cpu().numpy())
         assert np.abs(out[0, :16, h:h + 1].float().cpu().numpy() - want).max() <= 2e-2
+    # ... and on queries from each kind of tile in the launcher's plan for this shape: tiles run whole by one
+    # workgroup, light tiles (queries 2560-2639) computed alone, and light tiles that two workgroups share
+    samples = _tile_samples(T, H, 5 * T)
+    assert {kind for kind, _, _ in samples} >= {"whole", "light+shared", "light"}
+    _check_samples_against_oracle(out[0], q[0], k_all, v_all, samples)
     # rows of the softmax sum to one at full size
     out_c = _native.attention_bf16(q[0].contiguous(), k_all, torch.full_like(v_all, 0.75), 128 ** -0.5)
     assert (out_c.float() - 0.75).abs().max().item() <= 2 ** -7
@@ -435,6 +485,12 @@ def test_release_shape_rolling_window_equals_attention_over_the_dequantized_slot
                 want = o.attention(q[0, rows, h:h + 1].float().cpu().numpy(), k_all[:, h:h + 1].float().cpu().numpy(),
                                    v_all[:, h:h + 1].float().cpu().numpy())
                 assert np.abs(out[0, rows, h:h + 1].float().cpu().numpy() - want).max() <= 2e-2
+            if c == 4:
+                # queries from every kind of tile of this launch's plan: two whole rounds, 136 full tiles cut
+                # into parts for several workgroups, and the 128-query last groups (light, shared as well)
+                samples = _tile_samples(T, H, blocks * T)
+                assert {kind for kind, _, _ in samples} >= {"whole", "shared", "light+shared"}
+                _check_samples_against_oracle(out[0], q[0], k_all, v_all, samples)
             del kd, vd, k_all, v_all, ref
         kvc.apply_cache_update(cache, ce, le, info, CFG)
 
@@ -716,3 +772,57 @@ def test_random_shapes_under_every_division(gpu, policy):
             n_new = int(rng.integers(0 if n_cached else 1, 300))
             Lq = int(rng.integers(1, 700))
             test_kernel_accepts_any_number_of_cached_tokens(gpu, H, bts, n_cached, n_new, Lq)
+
+
+def test_launch_on_a_capturing_stream_never_allocates(gpu):
+    """A launch recorded into a graph must not allocate, and the clearing of a fresh set of partial-tile records
+    must not become a graph node.  On a stream the library has not seen, the automatic choice therefore takes a
+    division that needs no memory while the stream is being captured, and an explicit request for the split
+    division is refused; once the memory has been reserved on that stream, the recording takes the split division
+    and every replay reproduces the eager result bit for bit."""
+    Lq, Lk, H = 700, 900, 2
+    assert _native.attention_plan(Lq, H, Lk)["division"] == "split"
+    q, k, v = (_randn((n, H, 128), s).to(gpu) for n, s in ((Lq, 81), (Lk, 82), (Lk, 83)))
+    eager = _native.attention_bf16(q, k, v, 128 ** -0.5)          # split division, memory of the test's stream
+    for policy in ("narrow", "wide"):                                # every kernel has run once before a recording
+        with _native.attention_policy(policy):
+            _native.attention_bf16(q, k, v, 128 ** -0.5)
+    ref = o.attention(q.float().cpu().numpy(), k.float().cpu().numpy(), v.float().cpu().numpy())
+    side = torch.cuda.Stream(device=gpu)
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out = _native.attention_bf16(q, k, v, 128 ** -0.5)
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.abs(out.float().cpu().numpy() - ref).max() <= 2e-2
+    assert (out.float() - eager.float()).abs().max().item() <= 4e-3   # another division: other order of additions
+    side2 = torch.cuda.Stream(device=gpu)
+    side2.wait_stream(torch.cuda.current_stream())
+    with _native.attention_policy("split"):
+        graph2 = torch.cuda.CUDAGraph()
+        with pytest.raises(RuntimeError, match="captured"):
+            with torch.cuda.graph(graph2, stream=side2):
+                _native.attention_bf16(q, k, v, 128 ** -0.5)
+    del graph2
+    torch.cuda.synchronize()
+    # with the memory reserved on the stream ahead of the recording, the split division is recorded
+    side3 = torch.cuda.Stream(device=gpu)
+    side3.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side3):
+        _native.attention_reserve(Lq, H, Lk)
+    side3.synchronize()
+    graph3 = torch.cuda.CUDAGraph()
+    with _native.attention_policy("split"), torch.cuda.graph(graph3, stream=side3):
+        out3 = _native.attention_bf16(q, k, v, 128 ** -0.5)
+    for _ in range(3):
+        out3.zero_()
+        graph3.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out3, eager)
+        _native.attention_bf16(q, k, v, 128 ** -0.5)   # eager work between the replays
+    with torch.cuda.stream(side3):
+        _native.attention_release()
+    _native.attention_release()   # a stream without memory: nothing to do
