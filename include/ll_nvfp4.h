@@ -42,6 +42,19 @@ enum { LL_DTYPE_BF16 = 0, LL_DTYPE_F16 = 1, LL_DTYPE_F32 = 2 }; /* utils/kernel/
 const char* ll_last_error(void);
 int ll_version(void);
 
+/*
+ * Memory of the library's own.  Two kernels let several workgroups compute parts of one output tile and pass the
+ * parts through device memory: the attention's split division (ll_kv_attention_set_policy) and the W4A4 GEMM at
+ * sizes where whole tiles would leave compute units idle (ll_nvfp4_gemm_reserve).  That memory is allocated per
+ * (device, stream) by the first launch that needs it, grown when a later launch needs more (which frees the old
+ * set and so waits for the device), shared by both kernels and kept.  ll_release_stream_memory frees the set of
+ * (current device, stream), if any, after waiting for the launches that still use it - for callers that create
+ * streams as they go.  Launches on a stream that is being captured into a graph never allocate: they use the set a
+ * reserve call or an earlier launch left on that stream, or fall back to a division of the work that needs none.
+ * No counterpart in the reference.
+ */
+int ll_release_stream_memory(void* stream);
+
 /* Number of floats of scratch ll_nvfp4_quantize needs when it computes amax itself. */
 size_t ll_nvfp4_quantize_workspace_floats(void);
 
@@ -188,6 +201,32 @@ int ll_nvfp4_gemm_tnt_grouped(const uint8_t* A_values, const uint8_t* A_scales, 
                               const ll_gemm_product* products, void* stream);
 
 /*
+ * The GEMM entry points run one of two kernels.  Products large enough to give every compute unit several K steps
+ * (and with Kp a multiple of 128) run as one persistent launch: one workgroup per compute unit, output tiles of
+ * 128 x 512, and the sequence of (tile, K step) pairs cut into equal shares, so that no compute unit waits for
+ * another (the reference's kernel is a persistent tile scheduler too, csrc/fp4_gemm.cu:67-92).  A tile whose K range
+ * is shared by several workgroups is summed from their fp32 partial tiles in a fixed order, so results are
+ * deterministic; they differ from those of the other kernel (one workgroup per tile, the whole K range in one
+ * accumulator) by the order of the fp32 additions only.  The partial tiles pass through memory of the library's own
+ * (see ll_release_stream_memory; 2 x 256 KB per compute unit).  ll_nvfp4_gemm_reserve sets that memory up ahead
+ * of a launch of the given sizes (n_products = 1 for the plain entry points) and does nothing when such a launch
+ * would take the other kernel; on a capturing stream without it, a launch takes the other kernel.
+ * ll_nvfp4_gemm_set_schedule chooses: LL_GEMM_AUTO (initial), LL_GEMM_TILES (always one workgroup per tile) or
+ * LL_GEMM_PERSISTENT (wherever the shapes allow); process-wide.
+ */
+#define LL_GEMM_AUTO (-1)
+#define LL_GEMM_TILES 0
+#define LL_GEMM_PERSISTENT 1
+int ll_nvfp4_gemm_set_schedule(int schedule);
+int ll_nvfp4_gemm_get_schedule(void);
+int ll_nvfp4_gemm_reserve(int64_t M, int64_t N, int64_t Kp, int n_products, void* stream);
+/* What a launch of these sizes would do on a device with `compute_units` CUs under `schedule` (host arithmetic
+ * only): *persistent = 1 and the numbers of workgroups, output tiles and K steps per tile, or *persistent = 0.
+ * Output pointers may be NULL. */
+int ll_nvfp4_gemm_plan(int64_t M, int64_t N, int64_t Kp, int n_products, int compute_units, int schedule,
+                       int* persistent, uint32_t* workgroups, uint32_t* tiles, uint32_t* k_steps);
+
+/*
  * Replaces torch.ops.longlive_kernels.dequantize_kv_cache_fp4 (utils/kernel/kv_dequant.cpp:14,
  * utils/kernel/kv_dequant_cuda.cu:59-239): n_blocks cache slots, each NVFP4 [rows_padded, 128] holding
  * block_token_size*num_heads logical rows, are dequantized to out[1, n_blocks*block_token_size, num_heads, 128]
@@ -259,8 +298,7 @@ int ll_kv_attention_get_policy(void);
  * and may free a smaller set (which waits for the device).  LL_ENOSUP while the stream is being captured.  No
  * counterpart in the reference. */
 int ll_kv_attention_reserve(int64_t Lq, int num_heads, int64_t n_keys, void* stream);
-/* Frees the memory the split division holds for (current device, stream), if any; waits for the launches that
- * still use it.  For callers that create streams as they go: the library keeps one set per stream it has seen. */
+/* ll_release_stream_memory under its first name. */
 int ll_kv_attention_release(void* stream);
 /* What a launch of Lq queries x num_heads heads over n_keys keys would do on a device with `compute_units` CUs
  * under `policy` (pure host arithmetic, no GPU needed): the division taken (an LL_ATTENTION_SPLIT request falls

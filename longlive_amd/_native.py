@@ -73,6 +73,11 @@ _SIGNATURES = {
                                  c_void_p, c_void_p]),
     "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
     "ll_layer_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p]),
+    "ll_release_stream_memory": (c_int, [c_void_p]),
+    "ll_nvfp4_gemm_set_schedule": (c_int, [c_int]),
+    "ll_nvfp4_gemm_get_schedule": (c_int, []),
+    "ll_nvfp4_gemm_reserve": (c_int, [c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "ll_nvfp4_gemm_plan": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ll_kv_attention_reserve": (c_int, [c_int64, c_int, c_int64, c_void_p]),
     "ll_kv_attention_release": (c_int, [c_void_p]),
     "ll_nvfp4_quantize_noalloc_max_elements": (c_int64, []),
@@ -438,6 +443,51 @@ def gemm_grouped(a_values, a_scales, amax_a, denom_a: float, M: int, N: int, pro
                                                 ctypes.cast(structs, c_void_p), _stream())
     _check(code, "ll_nvfp4_gemm_tnt_grouped")
     return outs
+
+
+GEMM_SCHEDULES = {"auto": -1, "tiles": 0, "persistent": 1}
+
+
+def gemm_plan(M: int, N: int, Kp: int, n_products: int = 1, compute_units: int = 256, schedule: str = "auto") -> dict:
+    """What a GEMM launch of these sizes would do on a device with ``compute_units`` CUs (host arithmetic only):
+    whether it runs as one persistent launch, and then its workgroups, output tiles and K steps per tile."""
+    persistent, groups, tiles, steps = c_int(), ctypes.c_uint32(), ctypes.c_uint32(), ctypes.c_uint32()
+    _check(load().ll_nvfp4_gemm_plan(M, N, Kp, n_products, compute_units, GEMM_SCHEDULES[schedule], ctypes.byref(persistent),
+                                     ctypes.byref(groups), ctypes.byref(tiles), ctypes.byref(steps)), "ll_nvfp4_gemm_plan")
+    return {"persistent": bool(persistent.value), "workgroups": groups.value, "tiles": tiles.value, "k_steps": steps.value}
+
+
+def gemm_reserve(M: int, N: int, Kp: int, n_products: int = 1, device=None) -> None:
+    """Set up, on the current stream, the memory through which a GEMM launch of these sizes would pass partial
+    tiles (nothing if it would run one workgroup per tile), so that the launch itself allocates nothing."""
+    with torch.cuda.device(device if device is not None else torch.cuda.current_device()):
+        _check(load().ll_nvfp4_gemm_reserve(M, N, Kp, n_products, _stream()), "ll_nvfp4_gemm_reserve")
+
+
+class gemm_schedule:
+    """``with gemm_schedule("tiles"): ...`` - which kernel the GEMM entry points run ("auto", "tiles": one workgroup
+    per output tile, "persistent": one workgroup per compute unit wherever the shapes allow; process-wide,
+    restored on exit)."""
+
+    def __init__(self, name: str):
+        if name not in GEMM_SCHEDULES:
+            raise ValueError(f"unknown GEMM schedule {name!r}; one of {sorted(GEMM_SCHEDULES)}")
+        self.value = GEMM_SCHEDULES[name]
+
+    def __enter__(self):
+        self.previous = load().ll_nvfp4_gemm_get_schedule()
+        _check(load().ll_nvfp4_gemm_set_schedule(self.value), "ll_nvfp4_gemm_set_schedule")
+        return self
+
+    def __exit__(self, *exc):
+        _check(load().ll_nvfp4_gemm_set_schedule(self.previous), "ll_nvfp4_gemm_set_schedule")
+        return False
+
+
+def release_stream_memory(device=None) -> None:
+    """Free the memory the library holds for the current stream (partial tiles of the attention and the GEMM)."""
+    with torch.cuda.device(device if device is not None else torch.cuda.current_device()):
+        _check(load().ll_release_stream_memory(_stream()), "ll_release_stream_memory")
 
 
 # --------------------------------------------------------------------------- KV cache

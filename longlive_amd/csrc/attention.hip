@@ -782,90 +782,7 @@ __global__ __launch_bounds__(kAttnThreads) void kv_attention_kernel(AttnParams p
   }  // segments
 }
 
-// Memory for the partial results of a launch that splits tiles between workgroups: one set per (device, stream),
-// created at the first such launch there, grown when a later launch needs more, never released.  Launches on one
-// stream run one after the other, so they can share a set; launches on different streams get different sets.
-struct SplitWorkspace {
-  float* partials = nullptr;
-  int* arrivals = nullptr;
-  uint32_t groups = 0;
-  int tiles = 0;
-};
-static std::mutex g_split_mutex;
-static std::map<std::pair<int, hipStream_t>, SplitWorkspace> g_split_workspaces;
-
-// `may_allocate` false (the stream is being captured into a graph): only a set that is already large enough is
-// handed out; *missing tells the caller that there is none.
-static int split_workspace(int dev, hipStream_t stream, uint32_t groups, int tiles, bool may_allocate, SplitWorkspace& out,
-                           bool* missing) {
-  std::lock_guard<std::mutex> lock(g_split_mutex);
-  if (missing) *missing = false;
-  if (!may_allocate) {
-    const auto it = g_split_workspaces.find({dev, stream});
-    if (it == g_split_workspaces.end() || it->second.groups < groups || it->second.tiles < tiles) {
-      if (missing) *missing = true;
-      return LL_OK;
-    }
-    out = it->second;
-    return LL_OK;
-  }
-  SplitWorkspace& w = g_split_workspaces[{dev, stream}];
-  if (w.groups < groups || w.tiles < tiles) {
-    if (w.partials) (void)hipFree(w.partials);  // waits for the launches that still use it
-    if (w.arrivals) (void)hipFree(w.arrivals);
-    w = SplitWorkspace{};
-    const int want_tiles = tiles < 1024 ? 1024 : tiles;
-    hipError_t e = hipMalloc(reinterpret_cast<void**>(&w.partials), (size_t)2 * groups * kPartialFloats * sizeof(float));
-    if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&w.arrivals), (size_t)want_tiles * sizeof(int));
-    if (e == hipSuccess) e = hipMemsetAsync(w.arrivals, 0, (size_t)want_tiles * sizeof(int), stream);
-    if (e != hipSuccess) {
-      set_error("ll_kv_attention: cannot set up %zu bytes for partial results: %s",
-                (size_t)2 * groups * kPartialFloats * sizeof(float), hipGetErrorString(e));
-      if (w.partials) (void)hipFree(w.partials);
-      if (w.arrivals) (void)hipFree(w.arrivals);
-      g_split_workspaces.erase({dev, stream});
-      return LL_ELAUNCH;
-    }
-    w.groups = groups;
-    w.tiles = want_tiles;
-  }
-  out = w;
-  return LL_OK;
-}
-
-static int release_split_workspace(int dev, hipStream_t stream) {
-  std::lock_guard<std::mutex> lock(g_split_mutex);
-  const auto it = g_split_workspaces.find({dev, stream});
-  if (it == g_split_workspaces.end()) return LL_OK;
-  if (it->second.partials) (void)hipFree(it->second.partials);  // waits for the launches that still use it
-  if (it->second.arrivals) (void)hipFree(it->second.arrivals);
-  g_split_workspaces.erase(it);
-  return LL_OK;
-}
-
-// Whether work submitted to `stream` is being recorded into a graph instead of run.  A failing query (the legacy
-// stream while another stream of the thread captures) counts as recording: then nothing may be allocated either.
-static bool stream_is_capturing(hipStream_t stream) {
-  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
-    (void)hipGetLastError();
-    return true;
-  }
-  return status != hipStreamCaptureStatusNone;
-}
-
 static std::atomic<int> g_attention_policy{LL_ATTENTION_AUTO};
-
-static int compute_units_of(int dev, int& cus) {
-  static std::atomic<int> cached[64];
-  if (dev >= 0 && dev < 64 && (cus = cached[dev].load(std::memory_order_relaxed)) > 0) return LL_OK;
-  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) {
-    set_error("ll_kv_attention: cannot read the number of compute units of device %d", dev);
-    return LL_ELAUNCH;
-  }
-  if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
-  return LL_OK;
-}
 
 // Three ways to run a launch, all one workgroup per compute unit at a time (LDS):
 //  * 128 queries per workgroup, the key range halved between two sets of waves; one workgroup per tile;
@@ -883,12 +800,12 @@ static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
     set_error("ll_kv_attention: hipGetDevice failed");
     return LL_ELAUNCH;
   }
-  if (int rc = compute_units_of(dev, cus)) return rc;
+  if (int rc = compute_units_of(dev, cus, "ll_kv_attention")) return rc;
   const int64_t n_iter = (p.n_cached + p.n_new + kIterKeys - 1) / kIterKeys;
   LL_REQUIRE(p.H * ((p.Lq + kWgQueries - 1) / kWgQueries) * n_iter < (1ll << 32), "ll_kv_attention: too many (tile, iteration) units");
   const int policy = g_attention_policy.load(std::memory_order_relaxed);
   AttentionPlan plan = plan_attention(p.Lq, p.H, p.n_cached + p.n_new, cus, policy);
-  SplitWorkspace w;
+  StreamScratch w;
   if (plan.mode == LL_ATTENTION_SPLIT) {
     // The split division passes partial tiles through device memory of the library's own.  While the stream is
     // being captured nothing may be allocated (and the clearing of a new set must not become a graph node): a set
@@ -897,7 +814,8 @@ static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
     // request for the split division is refused.
     const bool capturing = stream_is_capturing(stream);
     bool missing = false;
-    if (int rc = split_workspace(dev, stream, plan.d.G, (int)plan.split_tiles, !capturing, w, &missing)) return rc;
+    if (int rc = stream_scratch(dev, stream, (size_t)2 * plan.d.G * kPartialFloats * sizeof(float), (size_t)plan.split_tiles, !capturing, w,
+                                &missing, "ll_kv_attention")) return rc;
     if (missing) {
       if (policy == LL_ATTENTION_SPLIT) {
         set_error("ll_kv_attention: the split division needs device memory that cannot be allocated while the stream "
@@ -916,8 +834,8 @@ static int launch_attention(const AttnParams& p_in, hipStream_t stream) {
     hipLaunchKernelGGL(kv_attention_kernel<false>, dim3(p.d.G), dim3(kAttnThreads), smem, stream, p);
   } else {
     if (plan.mode == LL_ATTENTION_SPLIT) {
-      p.partials = w.partials;
-      p.arrivals = w.arrivals;
+      p.partials = reinterpret_cast<float*>(w.records);
+      p.arrivals = w.counters;
     }
     static std::atomic<uint64_t> lds_allowed_w{0};
     if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&kv_attention_kernel<true>), smem, lds_allowed_w, "ll_kv_attention")) return rc;
@@ -945,25 +863,19 @@ extern "C" int ll_kv_attention_reserve(int64_t Lq, int num_heads, int64_t n_keys
     set_error("ll_kv_attention_reserve: hipGetDevice failed");
     return LL_ELAUNCH;
   }
-  if (int rc = compute_units_of(dev, cus)) return rc;
+  if (int rc = compute_units_of(dev, cus, "ll_kv_attention")) return rc;
   const AttentionPlan plan = plan_attention(Lq, num_heads, n_keys, cus, g_attention_policy.load(std::memory_order_relaxed));
   if (plan.mode != LL_ATTENTION_SPLIT) return LL_OK;
   if (stream_is_capturing(static_cast<hipStream_t>(stream))) {
     set_error("ll_kv_attention_reserve: the stream is being captured; reserve before the recording starts");
     return LL_ENOSUP;
   }
-  SplitWorkspace w;
-  return split_workspace(dev, static_cast<hipStream_t>(stream), plan.d.G, (int)plan.split_tiles, true, w, nullptr);
+  StreamScratch w;
+  return stream_scratch(dev, static_cast<hipStream_t>(stream), (size_t)2 * plan.d.G * kPartialFloats * sizeof(float),
+                        (size_t)plan.split_tiles, true, w, nullptr, "ll_kv_attention_reserve");
 }
 
-extern "C" int ll_kv_attention_release(void* stream) {
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) {
-    ll::set_error("ll_kv_attention_release: hipGetDevice failed");
-    return LL_ELAUNCH;
-  }
-  return ll::release_split_workspace(dev, static_cast<hipStream_t>(stream));
-}
+extern "C" int ll_kv_attention_release(void* stream) { return ll_release_stream_memory(stream); }
 
 extern "C" int ll_kv_attention_plan(int64_t Lq, int num_heads, int64_t n_keys, int compute_units, int policy,
                                     int* division, uint32_t* workgroups, uint32_t* whole_rounds, int64_t* split_tiles) {

@@ -19,9 +19,8 @@
 // two workgroups share a CU: while one wave decodes, another wave's MFMAs run.  K is consumed in a
 // permuted order (lanes 0-31 and 32-63 take alternate 32-element runs), identical for A and B, so
 // the sum is unchanged.
-#include <stdlib.h>
-
 #include "ll_common.h"
+#include "gemm_split.h"
 
 namespace ll {
 
@@ -112,6 +111,97 @@ struct GemmGroups {
   int tiles_n_each;  // column tiles per product
   GemmGroup more[kMaxGemmGroups - 1];
 };
+
+// Epilogue of one wave: acc[g][f][r] holds output row m = row_base + 32 f + lane % 32 and output column
+// n = col_base + 32 g + 8 (r / 4) + 4 (lane / 32) + r % 4.  The wave transposes one 32-row slab at a time through its
+// own LDS patch (the stages of the main loop are free by now) and writes rows with coalesced 16-byte stores.
+template <int FA, int FB>
+__device__ __forceinline__ void gemm_epilogue(float16v (&acc)[FB][FA], float alpha, uint8_t* smem, int wave, int lane, int row_base,
+                                              int col_base, int M, int N, uint16_t* __restrict__ D, int64_t ldd,
+                                              const uint16_t* __restrict__ bias, int act, const GemmEpilogue& epi,
+                                              uint32_t sink_slot) {
+  const int l32 = lane & 31, lh = lane >> 5;
+  constexpr int kEpiPitch = 64 * FB + 16;  // bytes per slab row: 32*FB bf16 + pad
+  uint8_t* ebuf = smem + wave * (32 * kEpiPitch);
+  constexpr int kChunksPerRow = 4 * FB;     // 16-byte chunks (8 columns) per slab row
+  const int ch = lane % kChunksPerRow;      // this lane's chunk column, the same in every pass
+  const int n_lane = col_base + 8 * ch;
+  const bool vec_ok = ((ldd & 7) == 0) && ((reinterpret_cast<uintptr_t>(D) & 15) == 0);
+  float out_max = 0.0f;
+  float bias_f[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) bias_f[i] = (bias && n_lane + i < N) ? bf16_bits_to_f32(bias[n_lane + i]) : 0.0f;
+#pragma unroll
+  for (int f = 0; f < FA; ++f) {
+#pragma unroll
+    for (int g = 0; g < FB; ++g)
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        *reinterpret_cast<uint2*>(ebuf + l32 * kEpiPitch + (32 * g + 8 * rg + 4 * lh) * 2) =
+            make_uint2(pack_bf16x2(acc[g][f][4 * rg] * alpha, acc[g][f][4 * rg + 1] * alpha),
+                       pack_bf16x2(acc[g][f][4 * rg + 2] * alpha, acc[g][f][4 * rg + 3] * alpha));
+      }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int it = 0; it < (32 * kChunksPerRow) / 64; ++it) {
+      const int row = (it * 64 + lane) / kChunksPerRow;
+      const int m = row_base + 32 * f + row;
+      uint4 v = *reinterpret_cast<const uint4*>(ebuf + row * kEpiPitch + ch * 16);
+      if (m < M && n_lane < N) {
+        uint32_t w[4] = {v.x, v.y, v.z, v.w};
+        if (bias) {  // bf16 result + bf16 bias, rounded to bf16 (the separate add of the reference)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            w[i] = pack_bf16x2(__uint_as_float(w[i] << 16) + bias_f[2 * i],
+                               __uint_as_float(w[i] & 0xFFFF0000u) + bias_f[2 * i + 1]);
+          }
+        }
+        if (act == LL_ACT_GELU_TANH) {  // GELU (tanh form) of the bf16 value, computed in fp32, rounded to bf16
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            w[i] = pack_bf16x2(gelu_tanh_f32(__uint_as_float(w[i] << 16)),
+                               gelu_tanh_f32(__uint_as_float(w[i] & 0xFFFF0000u)));
+          }
+        }
+        if (epi.residual) {  // host side guarantees 16-byte aligned rows and N % 8 == 0 for this path
+          const uint4 rv = *reinterpret_cast<const uint4*>(epi.residual + (int64_t)m * epi.ldr + n_lane);
+          const uint32_t r[4] = {rv.x, rv.y, rv.z, rv.w};
+          if (epi.gate) {
+            const uint4 gv = *reinterpret_cast<const uint4*>(epi.gate + (int64_t)(m / epi.gate_rows) * epi.gate_stride + n_lane);
+            const uint32_t g[4] = {gv.x, gv.y, gv.z, gv.w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              w[i] = pack_bf16x2(__uint_as_float(w[i] << 16) * __uint_as_float(g[i] << 16),
+                                 __uint_as_float(w[i] & 0xFFFF0000u) * __uint_as_float(g[i] & 0xFFFF0000u));
+          }
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            w[i] = pack_bf16x2(__uint_as_float(r[i] << 16) + __uint_as_float(w[i] << 16),
+                               __uint_as_float(r[i] & 0xFFFF0000u) + __uint_as_float(w[i] & 0xFFFF0000u));
+        }
+        if (epi.sink.parts) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const bool lo_ok = n_lane + 2 * i < N, hi_ok = n_lane + 2 * i + 1 < N;
+            if (lo_ok) out_max = fmaxf(out_max, fabsf(__uint_as_float(w[i] << 16)));
+            if (hi_ok) out_max = fmaxf(out_max, fabsf(__uint_as_float(w[i] & 0xFFFF0000u)));
+          }
+        }
+        uint16_t* dst = D + (int64_t)m * ldd + n_lane;
+        if (vec_ok && n_lane + 8 <= N) {
+          *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+        } else {
+          for (int i = 0; i < 8 && n_lane + i < N; ++i) dst[i] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (epi.sink.parts) {  // one atomic per wave
+    out_max = wave_max(out_max);
+    if (lane == 0) amax_sink_update(epi.sink, sink_slot, out_max);
+  }
+}
 
 template <int FA, int FB>
 __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
@@ -429,97 +519,212 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_kernel(
     }
   }
 
-  // ---- epilogue.  acc[g][f][r]: output column n = col0 + wn*32*FB + 32 g + 8 (r/4) + 4 lh + r%4,
-  //                               output row    m = row0 + wm*32*FA + 32 f + l32.
-  // Each wave transposes one 32-row slab at a time through its own LDS patch (both stages are free
-  // after the last barrier) and writes rows with coalesced 16-byte stores.
+  // ---- epilogue
   float alpha;
   if (alpha_ptr) {
     alpha = alpha_ptr[0];
   } else {
     alpha = (amax_a[0] * amax_b[0]) * (inv_denom_a * inv_denom_b);
   }
-  constexpr int kEpiPitch = 64 * FB + 16;  // bytes per slab row: 32*FB bf16 + pad
-  uint8_t* ebuf = smem + wave * (32 * kEpiPitch);
-  constexpr int kChunksPerRow = 4 * FB;     // 16-byte chunks (8 columns) per slab row
-  const int ch = lane % kChunksPerRow;      // this lane's chunk column, the same in every pass
-  const int n_lane = col0 + wn * 32 * FB + 8 * ch;
-  const bool vec_ok = ((ldd & 7) == 0) && ((reinterpret_cast<uintptr_t>(D) & 15) == 0);
-  float out_max = 0.0f;
-  float bias_f[8];
+  gemm_epilogue<FA, FB>(acc, alpha, smem, wave, lane, row0 + wm * 32 * FA, col0 + wn * 32 * FB, M, N, D, ldd, bias, act, epi,
+                        (uint32_t)blockIdx.x * 4 + wave);
+}
+
+// ============================================================================ persistent kernel
+// One workgroup per compute unit, four waves, one per SIMD; each wave owns 128 rows x 128 columns of a 128 x 512
+// output tile (4 x 4 MFMA tiles: all 256 accumulator registers, and four decode instructions per MFMA instead of the
+// six to nine of the kernel above - on this chip a SIMD issues one vector instruction at a time, and under load its
+// clock follows the power drawn, so instructions per MFMA are what the speed of the loop comes down to).  The A tile
+// (128 rows) is shared by the four waves, the B rows are the wave's own.  The (tile, K step) pairs of the launch are
+// cut into one equal share per workgroup (gemm_split.h); a tile whose K range several workgroups share is summed
+// from their fp32 partial tiles by whoever arrives last, always in the same order.
+// The main loop is a generated instruction sequence (gemm_loop_gen.py), included below as one asm statement.
+constexpr int kPStage = 46080;                    // bytes per LDS stage, as in gemm_loop_gen.py
+constexpr int kPSmem = 2 * kPStage + 16;          // two stages and a flag
+constexpr int kPRecordFloats = 4 * 256 * 64;      // a workgroup's fp32 partial tile: per wave 256 registers of 64 lanes
+
+struct PersistentParams {
+  const uint8_t* Av;
+  const uint8_t* As;
+  const float* amax_a;
+  float inv_denom_a;
+  GemmGroup prod[kMaxGemmGroups];  // every product, the first one included
+  int tiles_n_each;                // column tiles per product
+  int M, N, Np, Kp, tiles_m;
+  GemmDivision d;
+  GemmEpilogue epi;                // bias and sink come from the product
+  float* records;                  // [2 G] partial tiles of kPRecordFloats floats
+  int* arrivals;                   // [split tiles], zero between launches
+};
+
+// Partial tiles travel between workgroups on different XCDs, whose L2 caches do not see each other's lines.
+// Device-scope accesses (sc1) go past the L2: the stores write through, the loads fetch from memory.  They are
+// written as instructions here because sixteen bytes at a time and many loads in flight are what makes the exchange
+// cheap (as atomic operations of the language they come out one dword at a time, each load waited for).
+typedef float float4v __attribute__((ext_vector_type(4)));
+template <int OFFSET>
+__device__ __forceinline__ void store_shared_f32x4(float* ptr, float4v v) {
+  asm volatile("global_store_dwordx4 %0, %1, off offset:%2 sc1" ::"v"(ptr), "v"(v), "n"(OFFSET) : "memory");
+}
+template <int OFFSET>
+__device__ __forceinline__ void load_shared_f32x4(const float* ptr, float4v& v) {
+  asm volatile("global_load_dwordx4 %0, %1, off offset:%2 sc1" : "=v"(v) : "v"(ptr), "n"(OFFSET) : "memory");
+}
+// Waits for the loads above; the values pass through the statement so that nothing uses them before the wait.
+__device__ __forceinline__ void wait_shared_loads(float4v (&v)[32]) {
+  asm volatile("s_waitcnt vmcnt(0)"
+               : "+v"(v[0]), "+v"(v[1]), "+v"(v[2]), "+v"(v[3]), "+v"(v[4]), "+v"(v[5]), "+v"(v[6]), "+v"(v[7]), "+v"(v[8]),
+                 "+v"(v[9]), "+v"(v[10]), "+v"(v[11]), "+v"(v[12]), "+v"(v[13]), "+v"(v[14]), "+v"(v[15]), "+v"(v[16]),
+                 "+v"(v[17]), "+v"(v[18]), "+v"(v[19]), "+v"(v[20]), "+v"(v[21]), "+v"(v[22]), "+v"(v[23]), "+v"(v[24]),
+                 "+v"(v[25]), "+v"(v[26]), "+v"(v[27]), "+v"(v[28]), "+v"(v[29])
+               :
+               : "memory");
+  asm volatile("" : "+v"(v[30]), "+v"(v[31])::"memory");
+}
+// A wave's part of a record: 64 groups of four accumulator registers, group q at floats [q * 256 + lane * 4, + 4).
+// Group q = 16 gi + 4 f + rg holds acc[gi][f][4 rg .. 4 rg + 3].
+__device__ __forceinline__ void store_partial_tile(float* rec, float16v (&acc)[4][4]) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) bias_f[i] = (bias && n_lane + i < N) ? bf16_bits_to_f32(bias[n_lane + i]) : 0.0f;
+  for (int q0 = 0; q0 < 64; q0 += 4) {
+    float* base = rec + q0 * 256;
+    const int gi = q0 >> 4, f = (q0 >> 2) & 3;
+    const float16v& a = acc[gi][f];
+    store_shared_f32x4<0>(base, float4v{a[0], a[1], a[2], a[3]});
+    store_shared_f32x4<1024>(base, float4v{a[4], a[5], a[6], a[7]});
+    store_shared_f32x4<2048>(base, float4v{a[8], a[9], a[10], a[11]});
+    store_shared_f32x4<3072>(base, float4v{a[12], a[13], a[14], a[15]});
+  }
+}
+// acc = record (ADD false) or acc += record, thirty-two loads of sixteen bytes in flight at a time.
+template <bool ADD>
+__device__ __forceinline__ void load_partial_tile(const float* rec, float16v (&acc)[4][4]) {
 #pragma unroll
-  for (int f = 0; f < FA; ++f) {
+  for (int g2 = 0; g2 < 4; g2 += 2) {
+    float4v t[32];
 #pragma unroll
-    for (int g = 0; g < FB; ++g)
+    for (int x = 0; x < 8; ++x) {  // x = 4 (gi - g2) + f
+      const float* base = rec + (g2 * 16 + x * 4) * 256;
+      load_shared_f32x4<0>(base, t[4 * x]);
+      load_shared_f32x4<1024>(base, t[4 * x + 1]);
+      load_shared_f32x4<2048>(base, t[4 * x + 2]);
+      load_shared_f32x4<3072>(base, t[4 * x + 3]);
+    }
+    wait_shared_loads(t);
 #pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        *reinterpret_cast<uint2*>(ebuf + l32 * kEpiPitch + (32 * g + 8 * rg + 4 * lh) * 2) =
-            make_uint2(pack_bf16x2(acc[g][f][4 * rg] * alpha, acc[g][f][4 * rg + 1] * alpha),
-                       pack_bf16x2(acc[g][f][4 * rg + 2] * alpha, acc[g][f][4 * rg + 3] * alpha));
+    for (int x = 0; x < 8; ++x)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        if (ADD) acc[g2 + (x >> 2)][x & 3][i] += t[4 * x + (i >> 2)][i & 3];
+        else acc[g2 + (x >> 2)][x & 3][i] = t[4 * x + (i >> 2)][i & 3];
       }
-    __builtin_amdgcn_wave_barrier();
+  }
+}
+
+#define LL_V10(a) "v" #a "0", "v" #a "1", "v" #a "2", "v" #a "3", "v" #a "4", "v" #a "5", "v" #a "6", "v" #a "7", "v" #a "8", "v" #a "9"
+
+__global__ __launch_bounds__(256) void gemm_w4a4_persistent_kernel(PersistentParams p) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // Consecutive hardware workgroup numbers go to different XCDs; every XCD gets a contiguous range of the shares
+  // instead, so that workgroups that share an L2 work on neighbouring tiles (the same B rows, adjacent A rows).
+  const uint32_t g = p.d.G % 8 == 0 ? (blockIdx.x & 7) * (p.d.G / 8) + (blockIdx.x >> 3) : blockIdx.x;
+  GemmCursor at = gemm_start_of_work(g, p.d);
+  const uint32_t row_bytes = (uint32_t)p.Kp >> 1;
+  const uint32_t rb16 = 16u * row_bytes;
+  const uint32_t swz = (l32 >> 2) & 3;
+  // What a lane contributes to the addresses of the loop (gemm_loop_gen.py): its row and 16-byte piece in a load of
+  // 16 rows; its row, piece and scale group in the LDS reads; the shift that picks its pair of scale bytes.
+  const uint32_t lane_voff = (uint32_t)(lane >> 2) * row_bytes + 16u * ((lane & 3) ^ ((lane >> 4) & 3));
+  const uint32_t lane_soff = (uint32_t)lane * 16u;
+  const uint32_t ard = (uint32_t)l32 * 64u + 16u * ((lh ^ (swz & 1)) | (swz & 2));
+  const uint32_t sard = 40960u + (uint32_t)l32 * 16u;
+  const uint32_t sh = 16u * lh;
+  int* flag = reinterpret_cast<int*>(smem + 2 * kPStage);
+
+  GemmSegment seg;
+  while (gemm_next_segment(at, g, p.d, seg)) {
+    const int tile_m = (int)(seg.tile % (uint32_t)p.tiles_m), tile_n_all = (int)(seg.tile / (uint32_t)p.tiles_m);
+    const int pi = tile_n_all / p.tiles_n_each, tile_n = tile_n_all - pi * p.tiles_n_each;
+    const GemmGroup& pr = p.prod[pi];
+    const int row0 = tile_m * kPTileM, col0 = tile_n * kPTileN;
+    // The wave's 128 rows of B; a wave whose columns lie beyond the padded matrix recomputes the last block (its
+    // output is masked).
+    const int bcol = min(col0 + 128 * wave, p.Np - 128);
+    const uint32_t nsteps = seg.end - seg.begin;
+    const uint32_t voff = lane_voff + seg.begin * 64u, soff = lane_soff + seg.begin * 1024u;
+    const uint8_t* sA = p.Av + (size_t)(row0 + 32 * wave) * row_bytes;
+    const uint8_t* sB = pr.Bv + (size_t)bcol * row_bytes;
+    const uint8_t* sAs = p.As + (size_t)(row0 >> 7) * (size_t)(p.Kp >> 6) * 512;
+    const uint8_t* sBs = pr.Bs + (size_t)(bcol >> 7) * (size_t)(p.Kp >> 6) * 512;
+    float16v acc[4][4];
 #pragma unroll
-    for (int it = 0; it < (32 * kChunksPerRow) / 64; ++it) {
-      const int row = (it * 64 + lane) / kChunksPerRow;
-      const int m = row0 + wm * 32 * FA + 32 * f + row;
-      uint4 v = *reinterpret_cast<const uint4*>(ebuf + row * kEpiPitch + ch * 16);
-      if (m < M && n_lane < N) {
-        uint32_t w[4] = {v.x, v.y, v.z, v.w};
-        if (bias) {  // bf16 result + bf16 bias, rounded to bf16 (the separate add of the reference)
+    for (int gi = 0; gi < 4; ++gi)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            w[i] = pack_bf16x2(__uint_as_float(w[i] << 16) + bias_f[2 * i],
-                               __uint_as_float(w[i] & 0xFFFF0000u) + bias_f[2 * i + 1]);
-          }
-        }
-        if (act == LL_ACT_GELU_TANH) {  // GELU (tanh form) of the bf16 value, computed in fp32, rounded to bf16
+      for (int f = 0; f < 4; ++f)
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            w[i] = pack_bf16x2(gelu_tanh_f32(__uint_as_float(w[i] << 16)),
-                               gelu_tanh_f32(__uint_as_float(w[i] & 0xFFFF0000u)));
-          }
-        }
-        if (epi.residual) {  // host side guarantees 16-byte aligned rows and N % 8 == 0 for this path
-          const uint4 rv = *reinterpret_cast<const uint4*>(epi.residual + (int64_t)m * epi.ldr + n_lane);
-          const uint32_t r[4] = {rv.x, rv.y, rv.z, rv.w};
-          if (epi.gate) {
-            const uint4 gv = *reinterpret_cast<const uint4*>(epi.gate + (int64_t)(m / epi.gate_rows) * epi.gate_stride + n_lane);
-            const uint32_t g[4] = {gv.x, gv.y, gv.z, gv.w};
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              w[i] = pack_bf16x2(__uint_as_float(w[i] << 16) * __uint_as_float(g[i] << 16),
-                                 __uint_as_float(w[i] & 0xFFFF0000u) * __uint_as_float(g[i] & 0xFFFF0000u));
-          }
-#pragma unroll
-          for (int i = 0; i < 4; ++i)
-            w[i] = pack_bf16x2(__uint_as_float(r[i] << 16) + __uint_as_float(w[i] << 16),
-                               __uint_as_float(r[i] & 0xFFFF0000u) + __uint_as_float(w[i] & 0xFFFF0000u));
-        }
-        if (epi.sink.parts) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const bool lo_ok = n_lane + 2 * i < N, hi_ok = n_lane + 2 * i + 1 < N;
-            if (lo_ok) out_max = fmaxf(out_max, fabsf(__uint_as_float(w[i] << 16)));
-            if (hi_ok) out_max = fmaxf(out_max, fabsf(__uint_as_float(w[i] & 0xFFFF0000u)));
-          }
-        }
-        uint16_t* dst = D + (int64_t)m * ldd + n_lane;
-        if (vec_ok && n_lane + 8 <= N) {
-          *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
-        } else {
-          for (int i = 0; i < 8 && n_lane + i < N; ++i) dst[i] = (uint16_t)(w[i >> 1] >> (16 * (i & 1)));
+        for (int i = 0; i < 16; ++i) acc[gi][f][i] = 0.0f;
+    __syncthreads();  // LDS is free: the previous segment's epilogue is over in every wave
+    asm volatile(
+#include "gemm_loop_gfx950.inc"
+        : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]), "+a"(acc[1][1]), "+a"(acc[1][2]),
+          "+a"(acc[1][3]), "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[2][2]), "+a"(acc[2][3]), "+a"(acc[3][0]), "+a"(acc[3][1]),
+          "+a"(acc[3][2]), "+a"(acc[3][3])
+        : "s"(nsteps), "v"(voff), "v"(soff), "v"(ard), "v"(sard), "v"(sh), "s"(sA), "s"(sB), "s"(rb16), "s"(sAs), "s"(sBs), "s"(wave)
+        : "memory", "scc", "vcc", "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", LL_V10(1), LL_V10(2), LL_V10(3), LL_V10(4),
+          LL_V10(5), LL_V10(6), LL_V10(7), LL_V10(8), LL_V10(9), LL_V10(10), LL_V10(11), LL_V10(12), LL_V10(13), LL_V10(14), LL_V10(15),
+          LL_V10(16), "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71",
+          "s72", "s73", "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87");
+
+    bool write_out = true;
+    if (seg.begin != 0 || seg.end != p.d.nk) {
+      // Part of a tile.  Whoever arrives last at a tile adds the parts up, from the part with the last K steps
+      // backwards whoever does it, so the result does not depend on the order of arrival; the others leave their
+      // accumulators in a record and count their arrival.  The workgroup that holds the last part is normally the
+      // last to arrive (shares are walked backwards): if a look at the counter shows that, it goes on from its
+      // registers without writing a record.
+      const uint32_t split_tile = seg.tile - p.d.whole_rounds * p.d.G;  // the tile's number among the split ones
+      uint32_t g_first, g_last;
+      gemm_parts_of_tile(split_tile, p.d, g_first, g_last);
+      const int others = (int)(g_last - g_first);
+      if (tid == 0)
+        *flag = g == g_last && __hip_atomic_load(p.arrivals + split_tile, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
+      __syncthreads();
+      const bool from_registers = *flag != 0;
+      write_out = from_registers;
+      if (!from_registers) {
+        store_partial_tile(p.records + (size_t)gemm_record_of_part(g, split_tile, p.d) * kPRecordFloats + wave * (256 * 64) + lane * 4, acc);
+        // Every wave waits until its own record stores are complete (a write-through store is acknowledged once it
+        // is visible device-wide) before the barrier behind which thread 0 counts the arrival.
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+        __syncthreads();
+        if (tid == 0)
+          *flag = __hip_atomic_fetch_add(p.arrivals + split_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == others;
+        __syncthreads();
+        write_out = *flag != 0;
+      }
+      if (write_out) {
+        if (tid == 0) __hip_atomic_store(p.arrivals + split_tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next launch
+        // The part with the last K steps comes first (from the registers, or read back like the others), then the
+        // parts before it one by one: the same sequence of additions whoever does it.
+        for (int gg = (int)g_last - (from_registers ? 1 : 0); gg >= (int)g_first; --gg) {
+          const float* theirs = p.records + (size_t)gemm_record_of_part((uint32_t)gg, split_tile, p.d) * kPRecordFloats + wave * (256 * 64) + lane * 4;
+          if (!from_registers && gg == (int)g_last) load_partial_tile<false>(theirs, acc);
+          else load_partial_tile<true>(theirs, acc);
         }
       }
     }
-    __builtin_amdgcn_wave_barrier();
-  }
-  if (epi.sink.parts) {  // one atomic per wave
-    out_max = wave_max(out_max);
-    if (lane == 0) amax_sink_update(epi.sink, blockIdx.x * 4 + wave, out_max);
+    if (write_out) {
+      const float alpha = pr.alpha ? pr.alpha[0] : (p.amax_a[0] * pr.amax_b[0]) * (p.inv_denom_a * pr.inv_denom_b);
+      GemmEpilogue epi = p.epi;
+      epi.sink = pr.sink;
+      gemm_epilogue<4, 4>(acc, alpha, smem, wave, lane, row0, col0 + 128 * wave, p.M, p.N, pr.D, pr.ldd, pr.bias, epi.act, epi,
+                          seg.tile * 4 + wave);
+    }
   }
 }
+#undef LL_V10
+
 
 template <int FA, int FB>
 int launch_gemm(const uint8_t* Av, const uint8_t* As, const uint8_t* Bv, const uint8_t* Bs, const float* alpha,
@@ -618,11 +823,68 @@ extern "C" int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A
 }
 
 namespace ll {
+static std::atomic<int> g_gemm_schedule{LL_GEMM_AUTO};
+
+inline size_t persistent_record_bytes(const GemmDivision& d) { return (size_t)2 * d.G * kPRecordFloats * sizeof(float); }
+
+// Launches the persistent kernel if the plan says so and its memory is at hand; *launched tells.
+static int try_persistent(const uint8_t* A_values, const uint8_t* A_scales, const uint8_t* B_values, const uint8_t* B_scales,
+                          const float* alpha, const float* amax_a, const float* amax_b, float denom_a, float denom_b, int64_t M,
+                          int64_t N, int64_t Np, int64_t Kp, void* D, int64_t ldd, const GemmEpilogue& epi,
+                          const GemmGroups& groups, hipStream_t stream, bool* launched) {
+  *launched = false;
+  const int schedule = g_gemm_schedule.load(std::memory_order_relaxed);
+  if (schedule == LL_GEMM_TILES || Kp % 128 != 0) return LL_OK;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    set_error("ll_nvfp4_gemm_tnt: hipGetDevice failed");
+    return LL_ELAUNCH;
+  }
+  if (int rc = compute_units_of(dev, cus, "ll_nvfp4_gemm_tnt")) return rc;
+  const PersistentPlan plan = plan_persistent(M, N, Kp, groups.n, cus, schedule);
+  if (!plan.use) return LL_OK;
+  StreamScratch w;
+  bool missing = false;
+  if (int rc = stream_scratch(dev, stream, persistent_record_bytes(plan.d), gemm_split_tiles(plan.d), !stream_is_capturing(stream), w, &missing,
+                              "ll_nvfp4_gemm_tnt")) return rc;
+  if (missing) return LL_OK;  // a capturing stream without the memory: one workgroup per tile, which needs none
+  PersistentParams p{};
+  p.Av = A_values;
+  p.As = A_scales;
+  p.amax_a = amax_a;
+  p.inv_denom_a = denom_a > 0.f ? 1.0f / denom_a : 0.f;
+  p.prod[0] = GemmGroup{B_values, B_scales, alpha, amax_b, denom_b > 0.f ? 1.0f / denom_b : 0.f, static_cast<uint16_t*>(D), ldd,
+                        epi.bias, epi.sink};
+  for (int i = 1; i < groups.n; ++i) p.prod[i] = groups.more[i - 1];
+  p.tiles_n_each = plan.tiles_n_each;
+  p.M = (int)M;
+  p.N = (int)N;
+  p.Np = (int)Np;
+  p.Kp = (int)Kp;
+  p.tiles_m = plan.tiles_m;
+  p.d = plan.d;
+  p.epi = epi;
+  p.records = reinterpret_cast<float*>(w.records);
+  p.arrivals = w.counters;
+  static std::atomic<uint64_t> lds_allowed{0};
+  if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_w4a4_persistent_kernel), kPSmem, lds_allowed, "ll_nvfp4_gemm_tnt")) return rc;
+  hipLaunchKernelGGL(gemm_w4a4_persistent_kernel, dim3(plan.d.G), dim3(256), kPSmem, stream, p);
+  LL_CHECK_LAUNCH("gemm_w4a4_persistent_kernel");
+  *launched = true;
+  return LL_OK;
+}
+
 // Tile choice and launch; `groups.n` products side by side count as one product of groups.n * N columns.
 int dispatch_gemm(const uint8_t* A_values, const uint8_t* A_scales, const uint8_t* B_values, const uint8_t* B_scales,
                   const float* alpha, const float* amax_a, const float* amax_b, float denom_a, float denom_b, int64_t M,
                   int64_t N, int64_t Mp, int64_t Np, int64_t Kp, void* D, int64_t ldd, const GemmEpilogue& epi,
                   const GemmGroups& groups, hipStream_t s) {
+  {
+    bool launched = false;
+    if (int rc = try_persistent(A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, M, N, Np, Kp, D, ldd,
+                                epi, groups, s, &launched)) return rc;
+    if (launched) return LL_OK;
+  }
   const int64_t n_all = N * groups.n;
   // Tile choice.  Two workgroups are resident per CU (512 slots on 256 CUs).  The 256x128 / 128x256
   // tiles need 6 decode instructions per MFMA, the 128x128 tile 8, so the larger tiles win unless
@@ -647,23 +909,14 @@ int dispatch_gemm(const uint8_t* A_values, const uint8_t* A_scales, const uint8_
     }
   }
   // Small problems: when even 128x128 tiles would occupy at most half of the CUs, 64x64 tiles (more decode
-  // work per MFMA, but four times the workgroups) finish sooner.  Configuration 3 (64x128) is only reachable
-  // through the override below.
+  // work per MFMA, but four times the workgroups) finish sooner.
   if (((M + 127) / 128) * ((n_all + 127) / 128) <= 128) best = 4;
-  // Tuning aid: LL_GEMM_TILE=0..4 in the environment when the library is first used pins one tile configuration.
-  static const int forced_tile = [] {
-    const char* force = getenv("LL_GEMM_TILE");
-    const int f = force ? atoi(force) : -1;
-    return (f >= 0 && f < 5) ? f : -1;
-  }();
-  if (forced_tile >= 0) best = forced_tile;
 #define LL_GEMM_ARGS A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, (int)M, (int)N, \
                      (int)Mp, (int)Np, (int)Kp, D, ldd, epi, groups, s
   switch (best) {
     case 0: return launch_gemm<4, 2>(LL_GEMM_ARGS);
     case 1: return launch_gemm<2, 4>(LL_GEMM_ARGS);
     case 2: return launch_gemm<2, 2>(LL_GEMM_ARGS);
-    case 3: return launch_gemm<1, 2>(LL_GEMM_ARGS);
     default: return launch_gemm<1, 1>(LL_GEMM_ARGS);
   }
 #undef LL_GEMM_ARGS
@@ -716,4 +969,48 @@ extern "C" int ll_nvfp4_gemm_tnt_grouped(const uint8_t* A_values, const uint8_t*
   return dispatch_gemm(A_values, A_scales, p0.B_values, p0.B_scales, p0.alpha, amax_a, p0.amax_b, denom_a,
                        p0.denom_b > 0.f ? p0.denom_b : 1.f, M, N, Mp, Np, Kp, p0.D, p0.ldd, epi, groups,
                        static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ll_nvfp4_gemm_set_schedule(int schedule) {
+  LL_REQUIRE(schedule >= LL_GEMM_AUTO && schedule <= LL_GEMM_PERSISTENT, "ll_nvfp4_gemm_set_schedule: unknown schedule %d", schedule);
+  ll::g_gemm_schedule.store(schedule);
+  return LL_OK;
+}
+
+extern "C" int ll_nvfp4_gemm_get_schedule(void) { return ll::g_gemm_schedule.load(); }
+
+extern "C" int ll_nvfp4_gemm_plan(int64_t M, int64_t N, int64_t Kp, int n_products, int compute_units, int schedule,
+                                  int* persistent, uint32_t* workgroups, uint32_t* tiles, uint32_t* k_steps) {
+  LL_REQUIRE(M > 0 && N > 0 && Kp > 0 && Kp % 64 == 0 && n_products >= 1 && n_products <= ll::kMaxGemmGroups && compute_units > 0 &&
+                 M < (1 << 30) && N < (1 << 30) && Kp < (1 << 30),
+             "ll_nvfp4_gemm_plan: bad sizes");
+  LL_REQUIRE(schedule >= LL_GEMM_AUTO && schedule <= LL_GEMM_PERSISTENT, "ll_nvfp4_gemm_plan: unknown schedule %d", schedule);
+  const ll::PersistentPlan plan = ll::plan_persistent(M, N, Kp, n_products, compute_units, schedule);
+  if (persistent) *persistent = plan.use ? 1 : 0;
+  if (workgroups) *workgroups = plan.d.G;
+  if (tiles) *tiles = plan.d.tiles;
+  if (k_steps) *k_steps = plan.d.nk;
+  return LL_OK;
+}
+
+extern "C" int ll_nvfp4_gemm_reserve(int64_t M, int64_t N, int64_t Kp, int n_products, void* stream) {
+  using namespace ll;
+  LL_REQUIRE(M > 0 && N > 0 && Kp > 0 && Kp % 64 == 0 && n_products >= 1 && n_products <= kMaxGemmGroups && M < (1 << 30) &&
+                 N < (1 << 30) && Kp < (1 << 30),
+             "ll_nvfp4_gemm_reserve: bad sizes");
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    set_error("ll_nvfp4_gemm_reserve: hipGetDevice failed");
+    return LL_ELAUNCH;
+  }
+  if (int rc = compute_units_of(dev, cus, "ll_nvfp4_gemm_reserve")) return rc;
+  const PersistentPlan plan = plan_persistent(M, N, Kp, n_products, cus, g_gemm_schedule.load(std::memory_order_relaxed));
+  if (!plan.use) return LL_OK;
+  if (stream_is_capturing(static_cast<hipStream_t>(stream))) {
+    set_error("ll_nvfp4_gemm_reserve: the stream is being captured; reserve before the recording starts");
+    return LL_ENOSUP;
+  }
+  StreamScratch w;
+  return stream_scratch(dev, static_cast<hipStream_t>(stream), persistent_record_bytes(plan.d), gemm_split_tiles(plan.d), true, w, nullptr,
+                        "ll_nvfp4_gemm_reserve");
 }

@@ -32,6 +32,24 @@ void set_error(const char* fmt, ...);
 
 inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
 
+// ----------------------------------------------------------------------------- memory of the library's own (stream_scratch.hip)
+// Records for partial tiles and arrival counters, one set per (device, stream).
+struct StreamScratch {
+  uint8_t* records = nullptr;
+  size_t record_bytes = 0;
+  int* counters = nullptr;  // zero whenever no launch is running
+  size_t n_counters = 0;
+};
+// A set with at least record_bytes and `counters` counters.  may_allocate false (the stream is being captured into
+// a graph): only a set that is already large enough is handed out, and *missing says that there is none.
+int stream_scratch(int dev, hipStream_t stream, size_t record_bytes, size_t counters, bool may_allocate, StreamScratch& out,
+                   bool* missing, const char* what);
+int release_stream_scratch(int dev, hipStream_t stream);
+// Whether work submitted to `stream` is being recorded into a graph instead of run.  A failing query (the legacy
+// stream while another stream of the thread captures) counts as recording: then nothing may be allocated either.
+bool stream_is_capturing(hipStream_t stream);
+int compute_units_of(int dev, int& cus, const char* what);
+
 // Kernels that need more than 64 KB of dynamic LDS have to be told so with hipFuncSetAttribute, and that setting
 // holds per device.  `done` (one per kernel, zero-initialised) keeps one bit per device ordinal so that the call
 // is made once for every device the kernel is launched on; two threads racing here both make the same call.

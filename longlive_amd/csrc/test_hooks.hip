@@ -8,6 +8,7 @@
 #include <stdint.h>
 
 #include "attention_split.h"
+#include "gemm_split.h"
 
 __global__ void convert_kernel(const float* __restrict__ in, int64_t n, int mode, uint8_t* __restrict__ out) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -89,4 +90,42 @@ extern "C" int ll_test_attention_division_on_device(const uint32_t* division, ui
 // Host counterpart of first_unit_of for the comparison.
 extern "C" uint32_t ll_test_attention_first_unit(uint32_t g, const uint32_t* division) {
   return ll::first_unit_of(g, division_of(division));
+}
+
+// ---- the persistent GEMM's division (gemm_split.h) on the host.  A division travels as four numbers: G, tiles, nk,
+// whole_rounds.
+static ll::GemmDivision gemm_division_of(const uint32_t* d) { return ll::GemmDivision{d[0], d[1], d[2], d[3]}; }
+
+// The segments of workgroup g, in the order the kernel walks them, as (tile, begin, end) triples; returns their number.
+extern "C" int ll_test_gemm_segments(const uint32_t* division, uint32_t g, int32_t* out, int max_segments) {
+  const ll::GemmDivision d = gemm_division_of(division);
+  ll::GemmCursor at = ll::gemm_start_of_work(g, d);
+  ll::GemmSegment seg;
+  int n = 0;
+  while (ll::gemm_next_segment(at, g, d, seg)) {
+    if (n < max_segments) {
+      out[3 * n] = (int32_t)seg.tile;
+      out[3 * n + 1] = (int32_t)seg.begin;
+      out[3 * n + 2] = (int32_t)seg.end;
+    }
+    ++n;
+  }
+  return n;
+}
+extern "C" void ll_test_gemm_parts(uint32_t split_tile, const uint32_t* division, uint32_t* g_first, uint32_t* g_last) {
+  ll::gemm_parts_of_tile(split_tile, gemm_division_of(division), *g_first, *g_last);
+}
+extern "C" uint32_t ll_test_gemm_record(uint32_t g, uint32_t split_tile, const uint32_t* division) {
+  return ll::gemm_record_of_part(g, split_tile, gemm_division_of(division));
+}
+// The launcher's choice for a shape: out = use, G, tiles, nk, whole_rounds, tiles_m, tiles_n_each.
+extern "C" void ll_test_gemm_plan(int64_t M, int64_t N, int64_t Kp, int n_products, int cus, int schedule, uint32_t* out) {
+  const ll::PersistentPlan plan = ll::plan_persistent(M, N, Kp, n_products, cus, schedule);
+  out[0] = plan.use ? 1u : 0u;
+  out[1] = plan.d.G;
+  out[2] = plan.d.tiles;
+  out[3] = plan.d.nk;
+  out[4] = plan.d.whole_rounds;
+  out[5] = (uint32_t)plan.tiles_m;
+  out[6] = (uint32_t)plan.tiles_n_each;
 }

@@ -183,3 +183,57 @@ def attention_division_on_device(division: dict, split_tiles: int, device):
     host = [lib.ll_test_attention_first_unit(g, arr) for g in range(G + 1)]
     host += [x for t in range(split_tiles) for x in attention_parts(t, division)]
     return got, np.array(host, dtype=np.uint32)
+
+
+GEMM_DIVISION_FIELDS = ("G", "tiles", "nk", "whole_rounds")
+
+
+def gemm_plan(M: int, N: int, Kp: int, n_products: int = 1, cus: int = 256, schedule: int = 1) -> dict:
+    """The GEMM launcher's choice for a shape from the same arithmetic compiled for the host
+    (longlive_amd/csrc/gemm_split.h): use (persistent launch or not), the keys of GEMM_DIVISION_FIELDS, tiles_m and
+    tiles_n_each.  schedule: -1 automatic, 0 one workgroup per tile, 1 persistent wherever possible."""
+    import ctypes
+
+    lib = _test_hooks()
+    lib.ll_test_gemm_plan.restype = None
+    lib.ll_test_gemm_plan.argtypes = [ctypes.c_int64, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                      ctypes.c_void_p]
+    out = (ctypes.c_uint32 * 7)()
+    lib.ll_test_gemm_plan(M, N, Kp, n_products, cus, schedule, out)
+    return dict(use=bool(out[0]), G=out[1], tiles=out[2], nk=out[3], whole_rounds=out[4], tiles_m=out[5], tiles_n_each=out[6])
+
+
+def gemm_segments(division: dict, g: int):
+    """The (tile, begin, end) segments workgroup g of the persistent GEMM walks, in order."""
+    import ctypes
+
+    lib = _test_hooks()
+    lib.ll_test_gemm_segments.restype = ctypes.c_int
+    lib.ll_test_gemm_segments.argtypes = [ctypes.c_void_p, ctypes.c_uint32, ctypes.c_void_p, ctypes.c_int]
+    arr = (ctypes.c_uint32 * 4)(*[int(division[k]) for k in GEMM_DIVISION_FIELDS])
+    buf = (ctypes.c_int32 * (3 * 4096))()
+    n = lib.ll_test_gemm_segments(arr, g, buf, 4096)
+    assert n <= 4096
+    return [(buf[3 * i], buf[3 * i + 1], buf[3 * i + 2]) for i in range(n)]
+
+
+def gemm_parts(split_tile: int, division: dict):
+    import ctypes
+
+    lib = _test_hooks()
+    lib.ll_test_gemm_parts.restype = None
+    lib.ll_test_gemm_parts.argtypes = [ctypes.c_uint32, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
+    arr = (ctypes.c_uint32 * 4)(*[int(division[k]) for k in GEMM_DIVISION_FIELDS])
+    first, last = ctypes.c_uint32(), ctypes.c_uint32()
+    lib.ll_test_gemm_parts(split_tile, arr, ctypes.byref(first), ctypes.byref(last))
+    return first.value, last.value
+
+
+def gemm_record(g: int, split_tile: int, division: dict) -> int:
+    import ctypes
+
+    lib = _test_hooks()
+    lib.ll_test_gemm_record.restype = ctypes.c_uint32
+    lib.ll_test_gemm_record.argtypes = [ctypes.c_uint32, ctypes.c_uint32, ctypes.c_void_p]
+    arr = (ctypes.c_uint32 * 4)(*[int(division[k]) for k in GEMM_DIVISION_FIELDS])
+    return lib.ll_test_gemm_record(g, split_tile, arr)

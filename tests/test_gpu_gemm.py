@@ -435,3 +435,116 @@ def test_state_dict_written_by_the_reference_module_loads_and_runs(gpu, name):
                            rule="mse", padded=tuple(qw.padded_shape), orig=tuple(qw.original_shape)))
     oy = o.round_bf16(oy + from_bits(fx[f"{name}/bias"]).float().numpy()[None, :])
     assert np.linalg.norm(got - oy) / np.linalg.norm(oy) <= 1e-3
+
+
+def _ulp_close(a, b, frac=1e-3):
+    """Two bf16 results of the same fp32 sums added up in another order: equal except where the fp32 sums round to
+    neighbouring bf16 values, on a small fraction of the elements."""
+    a, b = a.float(), b.float()
+    diff = (a - b).abs()
+    assert bool((diff <= torch.maximum(a.abs(), b.abs()) * 2 ** -7 + 1e-30).all())
+    assert float((diff != 0).float().mean()) <= frac
+
+
+@pytest.mark.parametrize("M,N,K", [(300, 1100, 5120), (2640, 3072, 3072), (130, 513, 12800), (1000, 2048, 14336)])
+def test_persistent_schedule_against_the_oracle_and_the_tile_schedule(gpu, M, N, K):
+    """The persistent launch (one workgroup per compute unit, 128 x 512 tiles, the K range of the tiles behind the
+    whole rounds shared between workgroups and summed from fp32 partial tiles) against the oracle (1e-3 relative
+    Frobenius) and against the one-workgroup-per-tile kernel, which adds the same exact products in another order;
+    twice for identical bits (the order in which parts arrive must not show).  Shapes: ragged M and N with
+    overhanging tiles; the projection shape, whose 126 tiles are all split; 4 tiles of 100 steps over 256 workgroups
+    (every tile cut into some sixty parts); a long K with 32 tiles of 112 steps."""
+    cfg = QuantizationConfig(scale_rule="mse")
+    xq = quantize_to_fp4(activations((M, K), 81).to(gpu), cfg)
+    wq = quantize_to_fp4(weights((N, K), 82).to(gpu), cfg)
+    cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+    assert _native.gemm_plan(M, N, K, compute_units=cus, schedule="persistent")["persistent"]
+    with _native.gemm_schedule("tiles"):
+        tiles = fp4_matmul(xq, wq)
+    with _native.gemm_schedule("persistent"):
+        pers = fp4_matmul(xq, wq)
+        again = fp4_matmul(xq, wq)
+    assert torch.equal(pers, again)
+    _ulp_close(pers, tiles)
+    if M * N * K <= 3e10:
+        ref = o.fp4_matmul(_as_oracle(xq), _as_oracle(wq))
+        assert _rel(pers.float().cpu().numpy(), ref) <= TOL
+    assert _native.load().ll_nvfp4_gemm_get_schedule() == -1
+
+
+def test_persistent_schedule_with_every_epilogue_and_grouped_products(gpu):
+    """Bias, GELU, gated residual, amax sink and several products in one launch under the persistent schedule: the
+    epilogue is the same code behind either kernel, so each result equals the tile schedule's up to the order of
+    the fp32 additions, and the amax left in the sink is the maximum of the result written."""
+    cfg = QuantizationConfig(scale_rule="mse")
+    M, N, K, frame = 528, 1024, 5120, 176
+    xq = quantize_to_fp4(activations((M, K), 91).to(gpu), cfg)
+    ws = [quantize_to_fp4((weights((N, K), 92 + i) * (1 + i)).to(gpu), cfg) for i in range(3)]
+    gen = torch.Generator().manual_seed(93)
+    bias = (torch.randn(N, generator=gen) * 0.5).bfloat16().to(gpu)
+    residual = torch.randn(M, N, generator=gen).bfloat16().to(gpu)
+    gate = torch.randn(M // frame, 6, N, generator=gen).bfloat16().to(gpu)[:, 2]
+    results = {}
+    for sched in ("tiles", "persistent"):
+        with _native.gemm_schedule(sched):
+            t1, t2 = _native.amax_ticket(gpu), None
+            gelu = fp4_matmul(xq, ws[0], bias=bias, activation="gelu_tanh", amax_out=t1)
+            amax_gelu = float(quantize_to_fp4(gelu, cfg, amax=t1).amax)
+            gated = fp4_matmul(xq, ws[1], bias=bias, residual=residual, gate=gate, gate_rows=frame)
+            sinks = [_native.PrivateAmaxSink(gpu) for _ in range(3)]
+            products = [dict(values=w.values, scales=w.scale_factors, amax=w.amax, denom=1536.0, bias=bias if i != 1 else None,
+                             amax_out=s.ticket()) for i, (w, s) in enumerate(zip(ws, sinks))]
+            grouped = _native.gemm_grouped(xq.values, xq.scale_factors, xq.amax, 1536.0, M, N, products)
+            amax_grouped = [float(quantize_to_fp4(y, cfg, amax=pr["amax_out"]).amax) for y, pr in zip(grouped, products)]
+            results[sched] = (gelu, amax_gelu, gated, grouped, amax_grouped)
+    cus = torch.cuda.get_device_properties(gpu).multi_processor_count
+    assert _native.gemm_plan(M, N, K, 3, cus, "persistent")["persistent"] and _native.gemm_plan(M, N, K, 1, cus, "persistent")["persistent"]
+    (g0, a0, r0, gr0, ag0), (g1, a1, r1, gr1, ag1) = results["tiles"], results["persistent"]
+    _ulp_close(g1, g0, frac=5e-3)
+    _ulp_close(r1, r0)
+    assert a1 == float(g1.float().abs().max())
+    for y0, y1, am in zip(gr0, gr1, ag1):
+        _ulp_close(y1, y0)
+        assert am == float(y1.float().abs().max())
+    with pytest.raises(ValueError):
+        _native.gemm_schedule("fastest")
+
+
+def test_persistent_schedule_on_a_capturing_stream(gpu):
+    """A GEMM launch recorded into a graph never allocates: on a stream the library holds no memory for, a shape
+    the automatic choice would run persistently takes the one-workgroup-per-tile kernel instead; after
+    ll_nvfp4_gemm_reserve on that stream the persistent launch is recorded, and replays reproduce the eager
+    result bit for bit."""
+    cfg = QuantizationConfig(scale_rule="mse")
+    M, N, K = 640, 1024, 6400
+    xq = quantize_to_fp4(activations((M, K), 95).to(gpu), cfg)
+    wq = quantize_to_fp4(weights((N, K), 96).to(gpu), cfg)
+    with _native.gemm_schedule("persistent"):
+        eager_p = fp4_matmul(xq, wq)
+        with _native.gemm_schedule("tiles"):
+            eager_t = fp4_matmul(xq, wq)
+        side = torch.cuda.Stream(device=gpu)
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            out = fp4_matmul(xq, wq)
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager_t)          # no memory on that stream: the kernel that needs none
+        side2 = torch.cuda.Stream(device=gpu)
+        side2.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side2):
+            _native.gemm_reserve(M, N, K)
+        side2.synchronize()
+        graph2 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph2, stream=side2):
+            out2 = fp4_matmul(xq, wq)
+        for _ in range(3):
+            out2.zero_()
+            graph2.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out2, eager_p)
+            fp4_matmul(xq, wq)
+        with torch.cuda.stream(side2):
+            _native.release_stream_memory()

@@ -345,3 +345,80 @@ def test_attention_work_division_covers_every_iteration_exactly_once():
         plan = dict(mode=2, n_iter=n_iter, G=G, whole_rounds=rounds, extra=extra, units=(full_split + light_split) * n_iter,
                     full_units=full_split * n_iter, light=light, split_tiles=full_split + light_split)
         _check_division(plan, rounds * G + extra + full_split + light_split)
+
+
+def test_persistent_gemm_division_covers_every_k_step_exactly_once():
+    """The persistent GEMM's division of a launch between workgroups (longlive_amd/csrc/gemm_split.h, the functions
+    the kernel calls, compiled for the host): over the launcher's plans for the benchmark shapes, the released
+    shapes, grouped products and a sweep of random sizes and compute-unit counts, every (tile, K step) is computed
+    exactly once, shares of the split part differ by at most one step, only the first and the last tile of a share
+    are partial, every workgroup between the first and the last holder of a split tile holds a part of it, and no
+    two parts that meet in one tile use the same record."""
+    from helpers import GEMM_DIVISION_FIELDS, gemm_parts, gemm_plan, gemm_record, gemm_segments
+
+    rng = np.random.default_rng(5)
+    shapes = [(2640, 14336, 3072, 1, 256), (2640, 3072, 14336, 1, 256), (2640, 3072, 3072, 3, 256), (2640, 3072, 3072, 1, 256),
+              (7040, 14336, 3072, 1, 256), (7040, 3072, 14336, 1, 256), (512, 3072, 3072, 2, 256), (128, 512, 128 * 300, 1, 256),
+              (4096, 4096, 14336, 1, 256), (129, 513, 256, 4, 8), (2640, 3072, 14336, 1, 304), (300, 700, 1280, 1, 7)]
+    for _ in range(30):
+        shapes.append((int(rng.integers(1, 6000)), int(rng.integers(1, 9000)), 128 * int(rng.integers(1, 120)),
+                       int(rng.integers(1, 5)), int(rng.choice([1, 8, 64, 104, 256, 304]))))
+    used = 0
+    for M, N, Kp, n_products, cus in shapes:
+        plan = gemm_plan(M, N, Kp, n_products, cus)
+        if not plan["use"]:
+            assert plan["tiles"] == 0 or True
+            continue
+        used += 1
+        d = {k: plan[k] for k in GEMM_DIVISION_FIELDS}
+        G, tiles, nk, rounds = (d[k] for k in GEMM_DIVISION_FIELDS)
+        assert G == cus and tiles == plan["tiles_m"] * plan["tiles_n_each"] * n_products and nk == Kp // 128
+        assert plan["tiles_m"] * 128 >= M and plan["tiles_n_each"] * 512 >= N and rounds * G <= tiles
+        covered = np.zeros((tiles, nk), dtype=np.int32)
+        split = tiles - rounds * G
+        holders = [set() for _ in range(split)]
+        records = [dict() for _ in range(split)]
+        share_sizes = []
+        for g in range(G):
+            segs = gemm_segments(d, g)
+            assert [t for t, _, _ in segs[:rounds]] == [j * G + g for j in range(rounds)]
+            steps = 0
+            partial = []
+            for i, (t, b, e) in enumerate(segs):
+                assert 0 <= t < tiles and 0 <= b < e <= nk, (M, N, Kp, g, t, b, e)
+                covered[t, b:e] += 1
+                if i >= rounds:
+                    steps += e - b
+                    st = t - rounds * G
+                    holders[st].add(g)
+                    if b != 0 or e != nk:
+                        partial.append(i)
+                        rec = gemm_record(g, st, d)
+                        assert rec // 2 == g and rec not in records[st].values()
+                        records[st][g] = rec
+            share_sizes.append(steps)
+            assert all(i in (rounds, len(segs) - 1) for i in partial)            # first walked = last tile of the share, and vice versa
+            assert len({gemm_record(g, segs[i][0] - rounds * G, d) for i in partial}) == len(partial)   # its two parts: two records
+        assert (covered == 1).all(), (M, N, Kp, n_products, cus)
+        if split:
+            assert max(share_sizes) - min(share_sizes) <= 1 and min(share_sizes) >= 1
+        for st in range(split):
+            first, last = gemm_parts(st, d)
+            assert holders[st] == set(range(first, last + 1)), (M, N, Kp, st, first, last, holders[st])
+    assert used >= 20
+
+
+def test_persistent_gemm_plan_for_the_benchmark_shapes():
+    """What the automatic choice does with the shapes of the benchmark on 256 compute units: the long-K products run
+    as one persistent launch (FFN-down: 126 tiles of 112 K steps, each shared by two workgroups), the others one
+    workgroup per tile; a K that is not a multiple of 128 never runs persistently."""
+    from longlive_amd import _native
+
+    down = _native.gemm_plan(2640, 3072, 14336)
+    assert down == {"persistent": True, "workgroups": 256, "tiles": 126, "k_steps": 112}
+    assert not _native.gemm_plan(2640, 14336, 3072)["persistent"]
+    assert not _native.gemm_plan(512, 3072, 3072, n_products=2)["persistent"]
+    assert _native.gemm_plan(2640, 14336, 3072, schedule="persistent")["persistent"]
+    assert not _native.gemm_plan(2640, 3072, 14336, schedule="tiles")["persistent"]
+    assert not _native.gemm_plan(2640, 3072, 14336 + 64, schedule="persistent")["persistent"]
+    assert not _native.gemm_plan(64, 64, 128, schedule="persistent")["persistent"]
