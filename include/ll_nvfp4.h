@@ -201,18 +201,18 @@ int ll_nvfp4_gemm_tnt_grouped(const uint8_t* A_values, const uint8_t* A_scales, 
                               const ll_gemm_product* products, void* stream);
 
 /*
- * The GEMM entry points run one of two kernels.  Products large enough to give every compute unit several K steps
- * (and with Kp a multiple of 128) run as one persistent launch: one workgroup per compute unit, output tiles of
- * 128 x 512, and the sequence of (tile, K step) pairs cut into equal shares, so that no compute unit waits for
- * another (the reference's kernel is a persistent tile scheduler too, csrc/fp4_gemm.cu:67-92).  A tile whose K range
- * is shared by several workgroups is summed from their fp32 partial tiles in a fixed order, so results are
- * deterministic; they differ from those of the other kernel (one workgroup per tile, the whole K range in one
- * accumulator) by the order of the fp32 additions only.  The partial tiles pass through memory of the library's own
- * (see ll_release_stream_memory; 2 x 256 KB per compute unit).  ll_nvfp4_gemm_reserve sets that memory up ahead
- * of a launch of the given sizes (n_products = 1 for the plain entry points) and does nothing when such a launch
- * would take the other kernel; on a capturing stream without it, a launch takes the other kernel.
- * ll_nvfp4_gemm_set_schedule chooses: LL_GEMM_AUTO (initial), LL_GEMM_TILES (always one workgroup per tile) or
- * LL_GEMM_PERSISTENT (wherever the shapes allow); process-wide.
+ * The GEMM entry points can run one of two kernels.  LL_GEMM_TILES: one workgroup per output tile, two workgroups
+ * per compute unit.  LL_GEMM_PERSISTENT (wherever Kp is a multiple of 128 and there is at least one K step per
+ * compute unit): one workgroup per compute unit, output tiles of 128 x 512, whole rounds of tiles first and the
+ * (tile, K step) pairs of the tiles behind them cut into equal shares, so that no compute unit waits for another
+ * (the reference's kernel is a persistent tile scheduler too, csrc/fp4_gemm.cu:67-92).  A tile whose K range is
+ * shared by several workgroups is summed from their fp32 partial tiles in a fixed order, so results are
+ * deterministic; they differ from the other kernel's by the order of the fp32 additions only.  The partial tiles
+ * pass through memory of the library's own (see ll_release_stream_memory; 2 x 256 KB per compute unit).
+ * ll_nvfp4_gemm_reserve sets that memory up ahead of a launch of the given sizes (n_products = 1 for the plain
+ * entry points) and does nothing when such a launch would take the other kernel; on a capturing stream without it,
+ * a launch takes the other kernel.  LL_GEMM_AUTO (initial) takes the faster of the two as measured on MI355X,
+ * which at the sizes of the DiT block is LL_GEMM_TILES throughout.  ll_nvfp4_gemm_set_schedule is process-wide.
  */
 #define LL_GEMM_AUTO (-1)
 #define LL_GEMM_TILES 0

@@ -101,13 +101,12 @@ inline PersistentPlan plan_persistent(int64_t M, int64_t N, int64_t Kp, int n_pr
   const int64_t tiles_m = (M + kPTileM - 1) / kPTileM, tiles_n_each = (N + kPTileN - 1) / kPTileN;
   const int64_t tiles = tiles_m * tiles_n_each * n_products, nk = Kp / 128;
   if (tiles >= (1ll << 30) || tiles * nk < cus) return plan;
-  if (schedule == -1 /* LL_GEMM_AUTO */) {
-    // One wave per SIMD has nobody to hide a tile's first loads and its epilogue behind, which costs about five K
-    // steps per tile: the persistent kernel wins where tiles are long (measured: from about 48 K steps on), where
-    // every workgroup gets enough of them, and where the 128 x 512 tiles do not overhang the matrix by much.
-    if (nk < 48 || tiles * nk < 16 * (int64_t)cus) return plan;
-    if (M * 4 < tiles_m * kPTileM * 3 || N * 4 < tiles_n_each * kPTileN * 3) return plan;
-  }
+  // The automatic choice never takes the persistent launch.  Its main loop does more MFMAs per cycle and per joule
+  // (sustained, K = 14336: 0.53 - 0.58 of the f16 peak against 0.47 - 0.53), but one wave per SIMD has nobody to hide
+  // a tile's first loads and its epilogue behind, and the tiles behind the whole rounds pay for their partial tiles:
+  // inside the DiT block, with bias, GELU or the gated residual in the epilogue, every product measured slower
+  // (FFN-down 243 against 221 us, FFN-up 300 against 224 us).
+  if (schedule == -1 /* LL_GEMM_AUTO */) return plan;
   int64_t rounds = tiles / cus;
   // A few left-over tiles would be cut into many thin parts each (or leave workgroups without a single K step, and
   // every workgroup of [first, last] must hold a part of a split tile): then one whole round joins the split part.

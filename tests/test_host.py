@@ -409,16 +409,18 @@ def test_persistent_gemm_division_covers_every_k_step_exactly_once():
 
 
 def test_persistent_gemm_plan_for_the_benchmark_shapes():
-    """What the automatic choice does with the shapes of the benchmark on 256 compute units: the long-K products run
-    as one persistent launch (FFN-down: 126 tiles of 112 K steps, each shared by two workgroups), the others one
-    workgroup per tile; a K that is not a multiple of 128 never runs persistently."""
+    """The launcher's choice for the shapes of the benchmark on 256 compute units: the automatic choice runs one
+    workgroup per tile everywhere (the persistent launch measured slower inside the block); on request, FFN-down
+    runs as 126 tiles of 112 K steps, each shared by two workgroups; a K that is not a multiple of 128, or less work
+    than one K step per workgroup, never runs persistently."""
     from longlive_amd import _native
 
-    down = _native.gemm_plan(2640, 3072, 14336)
-    assert down == {"persistent": True, "workgroups": 256, "tiles": 126, "k_steps": 112}
+    assert not _native.gemm_plan(2640, 3072, 14336)["persistent"]
     assert not _native.gemm_plan(2640, 14336, 3072)["persistent"]
-    assert not _native.gemm_plan(512, 3072, 3072, n_products=2)["persistent"]
+    down = _native.gemm_plan(2640, 3072, 14336, schedule="persistent")
+    assert down == {"persistent": True, "workgroups": 256, "tiles": 126, "k_steps": 112}
     assert _native.gemm_plan(2640, 14336, 3072, schedule="persistent")["persistent"]
+    assert _native.gemm_plan(512, 3072, 3072, n_products=2, schedule="persistent")["persistent"]
     assert not _native.gemm_plan(2640, 3072, 14336, schedule="tiles")["persistent"]
     assert not _native.gemm_plan(2640, 3072, 14336 + 64, schedule="persistent")["persistent"]
     assert not _native.gemm_plan(64, 64, 128, schedule="persistent")["persistent"]
