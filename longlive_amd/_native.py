@@ -163,17 +163,19 @@ class AmaxTicket:
     """One use of a device's amax sink: handed to the kernel that writes a tensor (``amax_out=``) and then to
     the quantization of that tensor (``amax=``), which reads the maximum the producer left."""
 
-    __slots__ = ("parts", "epoch", "key", "offset")
+    __slots__ = ("parts", "epoch", "entry", "offset")
 
-    def __init__(self, parts: torch.Tensor, epoch: int, key=None, offset: torch.Tensor | None = None) -> None:
-        self.parts, self.epoch, self.key, self.offset = parts, epoch, key, offset
+    def __init__(self, parts: torch.Tensor, epoch: int, entry=None, offset: torch.Tensor | None = None) -> None:
+        # entry: the bookkeeping of the sink the ticket belongs to, [buffer, last epoch issued, (epoch, stream) of
+        # the last producer launch]; it lives as long as the sink or any of its tickets
+        self.parts, self.epoch, self.entry, self.offset = parts, epoch, entry, offset
 
     def struct(self) -> AmaxSinkStruct:
         return AmaxSinkStruct(self.parts.data_ptr(), self.epoch, None if self.offset is None else self.offset.data_ptr())
 
 
-# per sink: [sink buffer, last epoch issued, (epoch, stream) of the last producer launch]; the key of a device's own
-# sink is (device type, index), that of a graph's sink ("graph", id)
+# the devices' shared sinks, (device type, index) -> [sink buffer, last epoch issued, (epoch, stream) of the last
+# producer launch]; private and graph sinks keep their entry themselves and go away with their owner
 _sinks: dict = {}
 # device key -> the ReplayableAmaxSink whose tickets amax_ticket hands out at the moment
 _active_graph_sinks: dict = {}
@@ -191,19 +193,20 @@ class PrivateAmaxSink:
 
     def __init__(self, device) -> None:
         self.parts = torch.zeros(AMAX_PARTS, dtype=torch.int64, device=torch.device(device))
-        self.key = ("private", id(self))
         self.entry = [self.parts, 0, None]
-        _sinks[self.key] = self.entry
 
-    def ticket(self) -> "AmaxTicket":
-        key = _device_key(self.parts.device)
-        if key in _active_graph_sinks:  # a recording: epochs have to move with the replays
-            return _active_graph_sinks[key].ticket()
+    def ticket(self) -> "AmaxTicket | None":
+        """The next ticket, or None while launches are being recorded into a graph: a recording has one sink for
+        all its producers, whose slots the next producer overwrites, and no place for a maximum that is consumed
+        after the forward.  Without a ticket the producer leaves nothing behind and the consumer reduces the tensor
+        itself."""
+        if _device_key(self.parts.device) in _active_graph_sinks:
+            return None
         if self.entry[1] >= 0xFFFFFFFE:
             self.parts.zero_()
             self.entry[1] = 0
         self.entry[1] += 1
-        return AmaxTicket(self.parts, self.entry[1], self.key)
+        return AmaxTicket(self.parts, self.entry[1], self.entry)
 
 
 class ReplayableAmaxSink:
@@ -223,7 +226,6 @@ class ReplayableAmaxSink:
         self.device = torch.device(device)
         self.parts = torch.zeros(AMAX_PARTS, dtype=torch.int64, device=self.device)
         self.offset = torch.zeros(1, dtype=torch.int32, device=self.device)
-        self.key = ("graph", id(self))
         self.entry = [self.parts, 0, None]
 
     def __enter__(self):
@@ -231,7 +233,6 @@ class ReplayableAmaxSink:
         if dkey in _active_graph_sinks:
             raise RuntimeError("another replayable amax sink is active on this device")
         self.entry[1], self.entry[2] = 0, None
-        _sinks[self.key] = self.entry
         _active_graph_sinks[dkey] = self
         with torch.cuda.device(self.device):
             _check(load().ll_amax_epoch_advance(self.offset.data_ptr(), self.STEP, self.parts.data_ptr(), _stream()),
@@ -246,7 +247,7 @@ class ReplayableAmaxSink:
 
     def ticket(self) -> "AmaxTicket":
         self.entry[1] += 1
-        return AmaxTicket(self.parts, self.entry[1], self.key, self.offset)
+        return AmaxTicket(self.parts, self.entry[1], self.entry, self.offset)
 
 
 def amax_ticket(device: torch.device) -> AmaxTicket:
@@ -263,7 +264,7 @@ def amax_ticket(device: torch.device) -> AmaxTicket:
         entry = [torch.zeros(AMAX_PARTS, dtype=torch.int64, device=device), 0, None]
         _sinks[key] = entry
     entry[1] += 1
-    return AmaxTicket(entry[0], entry[1], key)
+    return AmaxTicket(entry[0], entry[1], entry)
 
 
 def _stream_of(ticket: AmaxTicket) -> int:
@@ -276,7 +277,7 @@ def _sink_struct(ticket):
         return AmaxSinkStruct(None, 0)
     if not isinstance(ticket, AmaxTicket):
         raise TypeError("amax_out must be an AmaxTicket (see amax_ticket)")
-    entry = _sinks.get(ticket.key)
+    entry = ticket.entry
     if entry is not None and entry[0] is ticket.parts:
         entry[2] = (ticket.epoch, _stream_of(ticket))
     return ticket.struct()
@@ -287,7 +288,7 @@ def _check_consumer(ticket: AmaxTicket) -> None:
     on the device's sink, and on the stream the producer ran on.  Anything else (another producer launched in
     between, the producer never launched, a different stream) would make the kernel read partial maxima of
     another tensor or none at all and quantize against a wrong amax without any error, so it is refused here."""
-    entry = _sinks.get(ticket.key)
+    entry = ticket.entry
     if entry is None or entry[0] is not ticket.parts:
         raise RuntimeError("this amax ticket belongs to a sink buffer that has been replaced")
     last = entry[2]

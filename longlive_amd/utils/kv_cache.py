@@ -14,7 +14,7 @@ import torch
 
 from .. import _native
 from ..fouroversix import QuantizationConfig, QuantizedTensor, quantize_to_fp4
-from .quant import SlotPointerTable, clone_quantized_tensor, k_smooth
+from .quant import SlotPointerTable, clone_quantized_tensor, copy_quantized_into, dequantize_kv_cache, k_smooth
 
 
 def initialize_kv_cache(num_layers: int, block_token_size: int, max_blocks: int, num_heads: int, head_dim: int,
@@ -35,31 +35,44 @@ def initialize_kv_cache(num_layers: int, block_token_size: int, max_blocks: int,
             "max_blocks": max_blocks,
             "num_heads": num_heads,
             "num_filled_blocks": 0,
-            "global_end_index": torch.tensor([0], dtype=torch.long, device=device),
-            "local_end_index": torch.tensor([0], dtype=torch.long, device=device),
-            "pinned_start": torch.tensor([-1], dtype=torch.long, device=device),
-            "pinned_len": torch.tensor([0], dtype=torch.long, device=device),
-            # host copies of the four scalars: the reference publishes them once per forward to avoid
-            # device syncs (utils/wan_5b_wrapper.py:355-366); here they are kept in step on the host
+            # The four scalars of the reference's schema (pipeline/causal_diffusion_inference.py:804-812).  There
+            # they live on the device and are published to the host once per forward (utils/wan_5b_wrapper.py:355-366);
+            # nothing on the device reads them here, so they are host tensors (an update is then no launch: with
+            # device tensors the streaming run issued two small fills per layer and cache write), mirrored as
+            # plain ints for the planner.
+            "global_end_index": torch.tensor([0], dtype=torch.long),
+            "local_end_index": torch.tensor([0], dtype=torch.long),
+            "pinned_start": torch.tensor([-1], dtype=torch.long),
+            "pinned_len": torch.tensor([0], dtype=torch.long),
             "_global_end": 0,
             "_local_end": 0,
             "_pinned_start": -1,
             "_pinned_len": 0,
             "_tables": {},
+            # True: a roll copies slot contents forward like the reference's copy_quantized_into, so that
+            # cache["k"][i] keeps its device address for good (utils/quant.py:783-794); False: a roll moves the slot
+            # buffers through the lists and copies nothing (see apply_cache_update)
+            "stable_slot_addresses": False,
         })
     return cache
+
+
+_MAX_TABLES = 16
 
 
 def _tables_for(cache: dict, slot_ids: tuple[int, ...]):
     # keyed by the buffers, not by the positions: a roll moves the buffers through the positions (apply_cache_update),
     # and the handful of arrangements that a streaming run cycles through are each built once
     key = tuple(cache["k"][i].values.data_ptr() for i in slot_ids)
-    entry = cache["_tables"].get(key)
+    tables = cache["_tables"]
+    entry = tables.pop(key, None)
     if entry is None:
         kt = SlotPointerTable([cache["k"][i] for i in slot_ids])
         vt = SlotPointerTable([cache["v"][i] for i in slot_ids])
         entry = (kt, vt)
-        cache["_tables"][key] = entry
+        while len(tables) >= _MAX_TABLES:   # scene cuts and varying windows multiply the arrangements: keep the
+            tables.pop(next(iter(tables)))  # most recently used ones (dicts keep insertion order)
+    tables[key] = entry
     return entry
 
 
@@ -110,14 +123,19 @@ def plan_cache_step(cache: dict, current_start: int, num_new_tokens: int, sink_t
     if local_start % blk or local_start < 0 or local_end > size:
         raise NotImplementedError("chunks must start on a block boundary of the cache and fit into it")
 
-    def slots(a: int, b: int) -> tuple[int, ...]:
-        """Slots that hold rows a..b of the buffer as it will look after the roll."""
-        if a % blk or b % blk or b > local_start:
-            raise NotImplementedError("attended ranges must cover whole cached blocks")
-        ids = []
-        for p in range(a, b, blk):
-            ids.append((p + evicted if effective_sink <= p < effective_sink + rolled else p) // blk)
-        return tuple(ids)
+    def pieces(a: int, b: int) -> list[tuple[int, int, int]]:
+        """(slot, first token, end token) pieces that hold rows a..b of the buffer as it will look after the roll."""
+        if a < 0 or b > local_start or a > b:
+            raise NotImplementedError("attended ranges must lie in the cached part of the buffer (a window shorter than "
+                                      "the protected prefix plus the chunk would cut into the chunk itself)")
+        out, p = [], a
+        while p < b:
+            src = p + evicted if effective_sink <= p < effective_sink + rolled else p   # whole blocks move in a roll
+            lo = src % blk
+            n = min(blk - lo, b - p)
+            out.append((src // blk, lo, lo + n))
+            p += n
+        return out
 
     window = size if max_attention_size is None else max_attention_size
     window_start = max(0, local_end - window)
@@ -126,16 +144,34 @@ def plan_cache_step(cache: dict, current_start: int, num_new_tokens: int, sink_t
     prepend_pinned = has_pinned and effective_sink <= ps < window_start
     if prepend_sink and prepend_pinned:
         lws = max(effective_sink, local_end - (window - effective_sink - pl))
-        slot_ids = slots(0, effective_sink) + slots(ps, ps + pl) + slots(lws, local_start)
+        attended = pieces(0, effective_sink) + pieces(ps, ps + pl) + pieces(lws, local_start)
     elif prepend_sink:
         lws = max(effective_sink, local_end - (window - effective_sink))
-        slot_ids = slots(0, effective_sink) + slots(lws, local_start)
+        attended = pieces(0, effective_sink) + pieces(lws, local_start)
     elif prepend_pinned:
         lws = max(0, local_end - (window - pl))
-        slot_ids = slots(ps, ps + pl) + slots(lws, local_start)
+        attended = pieces(ps, ps + pl) + pieces(lws, local_start)
     else:
-        slot_ids = slots(window_start, local_start)
+        attended = pieces(min(window_start, local_start), local_start)
+    # Whole slots go to the attention kernel as they are (it decodes FP4 on load).  A window that does not end on
+    # block boundaries (wan_5b/modules/causal_model.py:687-724 slices token rows) attends part of a slot: then the
+    # caller dequantizes the slots concerned and attends the bf16 rows, as the reference does for every window.
+    info["attended_pieces"] = attended
+    whole = all(lo == 0 and hi == blk for _, lo, hi in attended)
+    slot_ids = tuple(sl for sl, _, _ in attended) if whole else None
     return slot_ids, info, local_end
+
+
+def _materialize_pieces(cache: dict, pieces, dtype, device):
+    """bf16 K and V rows [n, H, 128] of (slot, first token, end token) pieces, in order: one dequantization launch
+    per operand over the slots concerned, then row slices."""
+    blk, H = cache["block_token_size"], cache["num_heads"]
+    order = sorted({sl for sl, _, _ in pieces})
+    pos = {sl: i for i, sl in enumerate(order)}
+    kd = dequantize_kv_cache([cache["k"][i] for i in order], len(order), H, blk, dtype, device)[0]
+    vd = dequantize_kv_cache([cache["v"][i] for i in order], len(order), H, blk, dtype, device)[0]
+    rows = [slice(pos[sl] * blk + lo, pos[sl] * blk + hi) for sl, lo, hi in pieces]
+    return torch.cat([kd[r] for r in rows]), torch.cat([vd[r] for r in rows])
 
 
 def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Tensor, cache: dict,
@@ -161,6 +197,10 @@ def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Ten
     k_new = (k_smooth(key_to_cache) if smoothed_key is None else smoothed_key)[0]
     scale = D ** -0.5 if softmax_scale is None else softmax_scale
     rule = cache["k"][0].scale_rule
+    if slot_ids is None:   # part of a slot is attended: bf16 rows of the window, then the plain attention kernel
+        wk, wv = _materialize_pieces(cache, info["attended_pieces"], q.dtype, q.device)
+        out = _native.attention_bf16(q[0].contiguous(), torch.cat([wk, k_new]), torch.cat([wv, v[0]]), scale, amax_out=amax_out)
+        return out.unsqueeze(0), (current_start + S, local_end, info)
     if slot_ids:
         kt, vt = _tables_for(cache, slot_ids)
         tables = (kt.values, kt.scales, kt.amax, vt.values, vt.scales, vt.amax)
@@ -193,14 +233,14 @@ def kv_cache_attention_relative(q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
     slot_ids, info, local_end = plan_cache_step(cache, current_start, S, sink_tokens, max_attention_size,
                                                 global_sink_tokens)
     info["new_k"], info["new_v"] = k, v
-    blk = cache["block_token_size"]
     keys, values = [k_smooth(k)[0]], [v[0]]
-    if slot_ids:
-        from .quant import dequantize_kv_cache
-        n = len(slot_ids)
-        keys.insert(0, dequantize_kv_cache([cache["k"][i] for i in slot_ids], n, H, blk, q.dtype, q.device)[0])
-        values.insert(0, dequantize_kv_cache([cache["v"][i] for i in slot_ids], n, H, blk, q.dtype, q.device)[0])
+    if info["attended_pieces"]:
+        wk, wv = _materialize_pieces(cache, info["attended_pieces"], q.dtype, q.device)
+        keys.insert(0, wk)
+        values.insert(0, wv)
     window_k, window_v = torch.cat(keys), torch.cat(values)
+    if window_k.shape[0] % frame_seqlen:
+        raise ValueError("relative RoPE needs an attended window of whole frames")
     window_frames, new_frames = window_k.shape[0] // frame_seqlen, S // frame_seqlen
     from .rope import rope_apply
     roped_k = rope_apply(window_k, *rope_fn(window_frames, 0))
@@ -228,8 +268,17 @@ def apply_cache_update(cache: dict, current_end: int, local_end_index: int, info
             n_roll = info["num_rolled_tokens"] // blk
             for name in ("k", "v"):
                 slots = cache[name]
-                slots[sink_b:sink_b + ev_b + n_roll] = (slots[sink_b + ev_b:sink_b + ev_b + n_roll]
-                                                       + slots[sink_b:sink_b + ev_b])
+                if sink_b < 0 or ev_b < 0 or n_roll < 0 or sink_b + ev_b + n_roll > len(slots):
+                    raise IndexError(f"roll of {n_roll} blocks behind {sink_b} protected and {ev_b} evicted ones does not fit "
+                                     f"a cache of {len(slots)} blocks")
+                if cache.get("stable_slot_addresses"):
+                    for i in range(n_roll):
+                        copy_quantized_into(slots[sink_b + i], slots[sink_b + ev_b + i])
+                else:
+                    n_slots = len(slots)
+                    slots[sink_b:sink_b + ev_b + n_roll] = (slots[sink_b + ev_b:sink_b + ev_b + n_roll]
+                                                           + slots[sink_b:sink_b + ev_b])
+                    assert len(slots) == n_slots
             if info.get("pinned_shift", 0) > 0:  # a floating pinned region moves with the data (:1437-1443)
                 cache["pinned_start"].sub_(info["pinned_shift"])
                 cache["_pinned_start"] -= info["pinned_shift"]

@@ -132,9 +132,11 @@ def kvc(monkeypatch):
 def planner_ids(kvc, cache, start, sink, gsink, max_att):
     slot_ids, info, local_end = kvc.plan_cache_step(cache, start, BLK, sink, max_att, gsink)
     ids = []
-    for s in slot_ids:
+    whole = all(lo == 0 and hi == BLK for _, lo, hi in info["attended_pieces"])
+    assert (slot_ids is not None) == whole and (slot_ids is None or list(slot_ids) == [s for s, _, _ in info["attended_pieces"]])
+    for s, lo, hi in info["attended_pieces"]:
         first = int(cache["k"][s].values[0])
-        ids += list(range(first, first + BLK))
+        ids += list(range(first + lo, first + hi))
     ids += list(range(start, start + BLK))
     new = torch.arange(start, start + BLK, dtype=torch.float64).view(1, BLK, 1, 1).expand(1, BLK, 1, 2)
     info["new_k"], info["new_v"] = new, new
@@ -148,7 +150,7 @@ def test_planner_attends_what_the_oracle_attends(kvc):
     for trial in range(200):
         sink = rnd.choice([0, BLK, 2 * BLK])
         gsink = rnd.choice([0, sink])
-        max_att = rnd.choice([SIZE, SIZE, SIZE - BLK])
+        max_att = rnd.choice([SIZE, SIZE, SIZE - BLK, SIZE - BLK // 2, SIZE - BLK - 3])   # windows that end inside a block too
         if max_att - max(sink, gsink) - (BLK if gsink else 0) < 2 * BLK:
             continue
         cuts = tuple(sorted(rnd.sample(range(1, 16), rnd.randint(0, 3)))) if sink else ()

@@ -826,3 +826,57 @@ def test_launch_on_a_capturing_stream_never_allocates(gpu):
     with torch.cuda.stream(side3):
         _native.attention_release()
     _native.attention_release()   # a stream without memory: nothing to do
+
+
+@pytest.mark.parametrize("window_tokens,sink_blocks", [(2 * 128 + 40, 1), (3 * 128 - 1, 0), (128 + 64, 0)])
+def test_windows_that_end_inside_a_block_against_the_policy_oracle(gpu, window_tokens, sink_blocks):
+    """max_attention_size that is not a multiple of the block size (wan_5b/modules/causal_model.py:673-724 slices token
+    rows): the local window then begins inside a cached slot.  Token list from the policy oracle, cached values from
+    the oracle's quantize-on-write, textbook attention; the cache bytes stay those of whole-block writes."""
+    import cache_policy_oracle as cpo
+
+    H, T, max_blocks, n_chunks = 2, 128, 4, 7
+    sink = sink_blocks * T
+    cache = kvc.initialize_kv_cache(1, T, max_blocks, H, 128, CFG, gpu)[0]
+    st = cpo.new_state(max_blocks * T)
+    content, partial = {}, 0
+    for c in range(n_chunks):
+        q, k, v = (_randn((1, T, H, 128), 3000 + 10 * c + s) for s in (1, 2, 3))
+        ids, upd = cpo.attend(st, c * T, T, sink, 0, window_tokens)
+        out, (ce, le, info) = kvc.kv_cache_attention(q.to(gpu), k.to(gpu), v.to(gpu), cache, c * T, sink_tokens=sink,
+                                                     max_attention_size=window_tokens)
+        cached = ids[:-T]
+        partial += int(any(lo != 0 or hi != T for _, lo, hi in info["attended_pieces"]))
+        wk = np.concatenate([content[int(i) // T][0][int(i) % T][None] for i in cached] + [o.k_smooth(k[0].float().numpy())])
+        wv = np.concatenate([content[int(i) // T][1][int(i) % T][None] for i in cached] + [v[0].float().numpy()])
+        ref = o.attention(q[0].float().numpy(), wk, wv)
+        err = np.abs(out[0].float().cpu().numpy() - ref).max()
+        assert err <= 2e-2, (c, err)
+        cpo.apply(st, upd)
+        kvc.apply_cache_update(cache, ce, le, info, CFG)
+        content[c] = (_oracle_slot(k[0])[0], _oracle_slot(v[0])[0])
+        assert int(cache["local_end_index"]) == st["local_end"]
+    assert partial >= 2   # the window did begin inside a slot
+
+
+def test_roll_with_stable_slot_addresses_copies_like_the_reference(gpu):
+    """cache["stable_slot_addresses"] = True: a roll copies slot contents forward (utils/quant.py:783-794), so every
+    position of cache["k"] / cache["v"] keeps its buffers for good; outputs and cache contents equal those of the
+    default roll, which moves the buffers through the lists."""
+    H, T, max_blocks, n_chunks = 2, 64, 3, 6
+    caches = [kvc.initialize_kv_cache(1, T, max_blocks, H, 128, CFG, gpu)[0] for _ in range(2)]
+    caches[1]["stable_slot_addresses"] = True
+    addresses = [[(s.values.data_ptr(), s.scale_factors.data_ptr(), s.amax.data_ptr()) for s in caches[1][n]] for n in ("k", "v")]
+    for c in range(n_chunks):
+        q, k, v = (_randn((1, T, H, 128), 4000 + 10 * c + s).to(gpu) for s in (1, 2, 3))
+        outs = []
+        for cache in caches:
+            out, (ce, le, info) = kvc.kv_cache_attention(q, k, v, cache, c * T, sink_tokens=T)
+            kvc.apply_cache_update(cache, ce, le, info, CFG)
+            outs.append(out)
+        assert torch.equal(outs[0], outs[1])
+        assert addresses == [[(s.values.data_ptr(), s.scale_factors.data_ptr(), s.amax.data_ptr()) for s in caches[1][n]] for n in ("k", "v")]
+    for n in ("k", "v"):
+        for a, b in zip(caches[0][n], caches[1][n]):
+            assert torch.equal(a.values, b.values) and torch.equal(a.scale_factors.view(torch.uint8), b.scale_factors.view(torch.uint8))
+            assert torch.equal(a.amax, b.amax)

@@ -198,3 +198,33 @@ def test_gelu_tanh_equals_logistic_form_in_fp64():
     assert o.gelu_tanh(np.array([0.0], dtype=np.float32))[0] == 0.0
     big = o.gelu_tanh(np.array([8.0, -8.0], dtype=np.float32))
     assert big[0] == 8.0 and abs(big[1]) < 1e-12
+
+
+@pytest.mark.parametrize("affine", [True, False])
+@pytest.mark.parametrize("rows,C,scale,offset", [(64, 256, 1.0, 0.0), (16, 3072, 3.0, 5.0), (33, 1000, 0.02, -0.5)])
+def test_layer_norm_affine_matches_torch_layer_norm(rows, C, scale, offset, affine):
+    """dit_oracle.layer_norm_affine (the LayerNorm ahead of cross-attention, wan_5b/modules/model.py:101-111: fp32
+    statistics and affine map on the bf16 input, one rounding to bf16) against torch's CPU layer_norm on the same
+    values in fp32, rounded to bf16 by torch: identical except where the fp32 result sits within rounding noise of
+    a bf16 tie (the oracle forms the statistics in double), there one bf16 ulp apart; and against the bf16 kernel of
+    torch (which keeps fp32 internally), to the same bar."""
+    import dit_oracle
+
+    g = torch.Generator().manual_seed(rows * 7 + C)
+    x = (torch.randn(rows, C, generator=g) * scale + offset).bfloat16()
+    w = (1 + 0.2 * torch.randn(C, generator=g)).bfloat16() if affine else torch.ones(C).bfloat16()
+    b = (0.3 * torch.randn(C, generator=g)).bfloat16() if affine else torch.zeros(C).bfloat16()
+    xn, wn, bn = (t.float().numpy() for t in (x, w, b))
+    got = dit_oracle.layer_norm_affine(xn, wn, bn, 1e-6)
+    for want in (torch.nn.functional.layer_norm(x.float(), (C,), w.float() if affine else None, b.float() if affine else None, 1e-6).bfloat16(),
+                 torch.nn.functional.layer_norm(x, (C,), w if affine else None, b if affine else None, 1e-6)):
+        want = want.float().numpy()
+        diff = np.abs(got - want)
+        # one bf16 ulp of the result, or - where the affine map cancels - of the terms that went into it
+        terms = np.abs(want) + np.abs(bn)[None, :]
+        assert (diff <= terms * 2.0 ** -7).all(), float((diff / terms).max())
+        assert (diff != 0).mean() <= 5e-3   # most on the row set whose mean lies 25 standard deviations from zero (fp32 statistics)
+    # closed form: a constant row normalizes to the bias
+    const = np.full((2, C), 3.0, dtype=np.float32)
+    out = dit_oracle.layer_norm_affine(const, wn, bn, 1e-6)
+    assert np.array_equal(out, np.broadcast_to(bn, (2, C)))
