@@ -65,7 +65,9 @@ size_t ll_nvfp4_quantize_workspace_floats(void);
  *   x        bf16 [M, K], row stride ldx elements
  *   values   u8 [Mp, Kp/2]      every byte written (padding rows/cols quantize zeros)
  *   scales   u8 [Mp*Kp/16]      every byte written
- *   amax     f32[1]             written unless amax_given != 0, in which case it is read
+ *   amax     f32[1]             written unless amax_given != 0, in which case it is read: then it must cover the
+ *                               tensor (blocks whose maximum exceeds it by more than a fifth would need block
+ *                               scales beyond e4m3, NaN in the reference; their bytes are unspecified)
  *   workspace  f32[ll_nvfp4_quantize_workspace_floats()], may be NULL when amax_given != 0
  */
 int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ldx, int rule,

@@ -312,14 +312,18 @@ __device__ __forceinline__ bool pick_four(const float (&X)[16], const ScaleEntry
 }
 
 // Returns false when the block has to take the exact path (an element would round past the e2m1 range).
+// `bound`: the tensor amax when the caller supplied it (it need not be the true maximum: a block that exceeds it
+// would get a scale beyond the e4m3 range, where the hardware conversion saturates and the reference does not),
+// infinity when the amax was computed from the tensor.
 template <int RULE>
 __device__ __forceinline__ bool quantize_block_fast(const float (&X)[16], float enc, const ScaleEntry* tab,
-                                                    bool approx_ok, uint32_t& lo, uint32_t& hi,
+                                                    bool approx_ok, float bound, uint32_t& lo, uint32_t& hi,
                                                     uint32_t& scale_byte) {
   constexpr bool kStatic = (RULE == LL_RULE_STATIC_6 || RULE == LL_RULE_STATIC_4);
   float bmax = fabsf(X[0]);
 #pragma unroll
   for (int i = 1; i < 16; ++i) bmax = fmaxf(bmax, fabsf(X[i]));
+  if (!(bmax <= bound)) return false;
   float quot;
   if (RULE == LL_RULE_STATIC_4) {
     quot = bmax * 0.25f;
@@ -396,13 +400,15 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
     if (blockIdx.x == 0 && threadIdx.x == 0) amax_io[0] = amax;
   }
 
-  // The fast path needs amax to be the true maximum (so block scales stay within e4m3 range) and far
-  // from the ends of the fp32 range (so powers of two scale exactly); otherwise every block takes the
-  // exact path.  The decision is uniform over the whole launch.
+  // The fast path needs every block maximum to stay below amax (so block scales stay within e4m3 range: true by
+  // construction when the amax was computed here, checked block by block when the caller supplied it) and amax far
+  // from the ends of the fp32 range (so powers of two scale exactly; uniform over the launch); otherwise the exact
+  // path is taken.
   constexpr bool kStaticRule = (RULE == LL_RULE_STATIC_6 || RULE == LL_RULE_STATIC_4);
   constexpr float kE2 = (RULE == LL_RULE_STATIC_4) ? 4.0f : 6.0f;
   constexpr float kE4 = kStaticRule ? 448.0f : 256.0f;
-  const bool fast = !amax_given && amax >= 0x1p-100f && amax <= 0x1p100f;
+  const bool fast = amax >= 0x1p-100f && amax <= 0x1p100f;
+  const float bound = amax_given ? amax : __builtin_inff();
   const bool approx_ok = amax >= 0x1p-30f && amax <= 0x1p30f;  // squares of errors stay normal fp32 numbers
   const float enc = (kE2 * kE4) / amax;
   const float dec = 1.0f / enc;
@@ -483,7 +489,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
       X[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
     }
     uint32_t lo, hi, sb;
-    if (!fast || !quantize_block_fast<RULE>(X, enc, s_tab, approx_ok, lo, hi, sb)) quantize_block<RULE>(X, amax, enc, dec, lo, hi, sb);
+    if (!fast || !quantize_block_fast<RULE>(X, enc, s_tab, approx_ok, bound, lo, hi, sb)) quantize_block<RULE>(X, amax, enc, dec, lo, hi, sb);
     uint8_t* dst = values + ((int64_t)t.ty * 128 * vrow + (int64_t)t.tx * 32) + thread_v + (int64_t)it * 64 * vrow;
     *reinterpret_cast<uint2*>(dst) = make_uint2(lo, hi);
     s_bytes[s_off0 + it * 8] = (uint8_t)sb;

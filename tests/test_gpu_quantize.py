@@ -105,6 +105,24 @@ def test_strided_input_and_given_amax(gpu):
     assert np.array_equal(u8(vals), v2) and np.array_equal(u8(sc), s2) and float(am.cpu()) == float(a2)
 
 
+@pytest.mark.parametrize("rule,factor", [(r, f) for r in ("mse", "mae", "static_6", "abs_max") for f in (1.0, 1.7, 30.0)]
+                         + [(r, 0.9) for r in ("mse", "mae", "abs_max")])   # the static rules put the amax itself at 448, the end of e4m3
+def test_caller_supplied_amax_bit_exact(gpu, rule, factor):
+    """A precomputed amax (quantize/pytorch/reference.py:244) that is the true maximum, larger than it, or a little
+    smaller (the blocks above the given amax, here by up to 11 %, get scales above 256 that e4m3 still holds; they
+    take the reference's own arithmetic block by block, the others the fast path), against the oracle bit for bit.
+    An amax so far below the maximum that block scales leave the e4m3 range (NaN in the reference) is not a
+    supported input."""
+    x = activations((384, 1024), 23).to(gpu)
+    true_amax = float(x.float().abs().max())
+    given = np.float32(true_amax * factor)
+    vals, sc, am = _native.quantize(x, rule, amax=torch.tensor([given], device=gpu))
+    v, s, a, _ = o.quantize_to_fp4(bits_of(x), rule, amax=given)
+    assert float(am.cpu()) == float(a) == float(given)
+    assert np.array_equal(u8(sc), s)
+    assert np.array_equal(u8(vals), v)
+
+
 def test_rejects_non_bf16_and_cpu_input(gpu):
     with pytest.raises(ValueError, match="bfloat16"):
         quantize_to_fp4(torch.zeros(128, 64, device=gpu))
