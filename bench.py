@@ -21,9 +21,8 @@ import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for p in (ROOT, os.path.join(ROOT, "tests")):
-    if p not in sys.path:
-        sys.path.insert(0, p)
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
 
 M_TOKENS, M_TEXT, DIM, FFN, HEADS = 2640, 512, 3072, 14336, 24
 # (name, M, K, N, count)
@@ -34,6 +33,7 @@ LINEAR_SET = [
     ("ffn_down", M_TOKENS, FFN, DIM, 1),
 ]
 PEAK_F16_TFLOPS = 2500.0  # MI355X dense fp16/bf16 MFMA peak (the GEMM runs v_mfma_f32_32x32x16_f16)
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense FP8 MFMA peak: the figure BASELINE.json's W4A4 target is quoted against
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E peak
 PREWARM_SECONDS = 0.5  # untimed load ahead of the warm-up steps (clock ramp-up), reported as config.prewarm_s
 # rocprofv3 counter summary of the FFN-up GEMM launch (FETCH_SIZE / WRITE_SIZE per dispatch and the factors a plain
@@ -97,7 +97,7 @@ def cpu_baseline(work) -> dict:
     import numpy as np
     import nvfp4_oracle as o
     import torch
-    from helpers import bits_of
+    from longlive_amd.utils.synthetic import bits_of
 
     from threadpoolctl import threadpool_limits
 
@@ -268,7 +268,7 @@ def run_quantize(torch, dev, steps, rule="mse"):
     """The quantize kernel alone on the FFN-down activation (2640 x 14336 bf16, the tensor with the most blocks),
     tensor amax taken from the amax sink its producer filled, as in the DiT block (no reduction pass): the launch
     the `roofline_quantize` record and the instruction-count profile are about."""
-    from helpers import activations, weights
+    from longlive_amd.utils.synthetic import activations, weights
     from longlive_amd import _native
     from longlive_amd.fouroversix import QuantizationConfig, fp4_matmul, quantize_to_fp4
 
@@ -283,6 +283,21 @@ def run_quantize(torch, dev, steps, rule="mse"):
     gbs = 2.5625 * x.numel() / ms / 1e6
     return {"quantize_ms": ms, "GB_per_s": gbs, "frac_of_hbm_8TBs": gbs / PEAK_HBM_GBS, "rule": rule,
             "workload": "quantize_kernel alone, 2640 x 14336 bf16 -> NVFP4, 96.98 MB algorithmic traffic, amax from a sink"}
+
+
+def run_copy(torch, dev, steps):
+    """Plain device-to-device copies, the yardstick for what the memory system gives a streaming kernel: 608 MiB
+    (read + write beyond the 256 MB last-level cache, so every byte moves through HBM) and 76 MB (the bytes of the
+    FFN-down activation, which stay in the last-level cache between launches)."""
+    rows = {}
+    for key, n in (("beyond_cache", 304 << 20), ("cached", 75_694_080)):
+        src = torch.empty(n, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        ms = _time_events(torch, lambda: dst.copy_(src), steps)
+        gbs = 2.0 * n / ms / 1e6
+        rows[key] = {"bytes_read_plus_written": 2 * n, "ms": ms, "GB_per_s": gbs, "frac_of_hbm_8TBs": gbs / PEAK_HBM_GBS}
+        del src, dst
+    return rows
 
 
 def run_gemm_shapes(torch, dev, work, cfg, steps):
@@ -324,7 +339,7 @@ def main() -> None:
 
     import torch
 
-    from helpers import activations, weights
+    from longlive_amd.utils.synthetic import activations, weights
     from longlive_amd.fouroversix import QuantizationConfig, fp4_matmul, quantize_to_fp4
 
     if not torch.cuda.is_available():
@@ -451,7 +466,10 @@ def main() -> None:
                    "prewarm_s": PREWARM_SECONDS},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_F16_TFLOPS, "traffic": measured_traffic_bytes(),
-                     "kernel": "gemm_w4a4_kernel M=2640 N=14336 K=3072", "avg_ms": gemm_ms},
+                     "kernel": "gemm_w4a4_kernel M=2640 N=14336 K=3072", "avg_ms": gemm_ms,
+                     "frac_of_fp8_peak": achieved / PEAK_FP8_TFLOPS,
+                     "note": "peak = dense f16 MFMA, the instruction the exact scheme runs on; frac_of_fp8_peak is the "
+                             "same rate against the 5 PFLOP/s dense FP8 figure"},
         "quantize": {"shape": [M_TOKENS, FFN], "avg_ms": q_ms, "GB_per_s": q_gbs, "frac_of_hbm_8TBs": q_gbs / 8000.0,
                      "note": "amax + quantize kernels, 2.5625 algorithmic bytes per element",
                      "amax_from_producer": {"avg_ms": qs_ms, "GB_per_s": qs_gbs, "frac_of_hbm_8TBs": qs_gbs / 8000.0,
@@ -470,6 +488,8 @@ def main() -> None:
                                 "with_amax_pass_frac": q_gbs / PEAK_HBM_GBS,
                                 "note": "achieved = 2.5625 algorithmic bytes per element / kernel time; traffic = the "
                                         "same bytes (FETCH_SIZE + WRITE_SIZE of the kernel equal them, profiles/)"}
+    # what a plain copy reaches on this box in this run: the ceiling any streaming kernel is measured against
+    out["roofline_quantize"]["device_copy"] = run_copy(torch, dev, reps)
     if not args.no_extras:
         extras = {}
         for key, fn in (("gemm_shapes", lambda: run_gemm_shapes(torch, dev, work, cfg, 10)),

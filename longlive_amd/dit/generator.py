@@ -120,7 +120,7 @@ class StreamingGenerator:
             x = initial_latent[0, start:start + nb].transpose(0, 1).contiguous()
             out[0, start:start + nb] = initial_latent[0, start:start + nb]
             for cache, text in zip(caches, (first_text, negative_context)):
-                self.model(x, torch.zeros((1, nb), device=self.device), text, cache, start * fs)
+                self.model(x, torch.zeros((1, nb), device=self.device), text, cache, start * fs, timestep_key=(0.0, nb))
         # projected text K / V per layer: one prompt per call, so they are computed by the first forward only
         xcache = [{"is_init": False} for _ in range(cfg.num_layers)] if self.cache_text_kv else None
         contexts = list(context) if isinstance(context, (list, tuple)) else None
@@ -155,10 +155,10 @@ class StreamingGenerator:
                 # forward before anything reads them (the chunk attends its own K / V in bf16), so only the
                 # clean-context pass below writes; the cache after the chunk is the same either way.
                 flow = self.model(x, tt, context, self.kv_cache, start * fs, crossattn_cache=xcache,
-                                  apply_cache_updates=not self.skip_dead_cache_writes)
+                                  apply_cache_updates=not self.skip_dead_cache_writes, timestep_key=(float(t), f))
                 if use_cfg:
                     uncond = self.model(x, tt, negative_context, self.kv_cache_neg, start * fs, crossattn_cache=xcache_neg,
-                                        apply_cache_updates=not self.skip_dead_cache_writes)
+                                        apply_cache_updates=not self.skip_dead_cache_writes, timestep_key=(float(t), f))
                     flow = uncond + self.guidance_scale * (flow - uncond)
                 if scheduler is not None:
                     x = scheduler.step(flow, t, x, return_dict=False)[0]
@@ -181,7 +181,8 @@ class StreamingGenerator:
             for cache, text, xc in zip(caches, (context, negative_context), (xcache, xcache_neg)):
                 if is_scene_cut and self.shot_clean_recache:
                     kvc.zero_kv_data(cache, start * fs, self.global_sink_size * fs)
-                self.model(x, torch.zeros((1, f), device=self.device), text, cache, start * fs, crossattn_cache=xc)
+                self.model(x, torch.zeros((1, f), device=self.device), text, cache, start * fs, crossattn_cache=xc,
+                           timestep_key=(0.0, f))
                 if is_scene_cut:
                     kvc.pin_current_chunk(cache, f * fs, cfg.sink_size * fs)
             if on_chunk is not None:

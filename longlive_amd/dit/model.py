@@ -309,6 +309,7 @@ class CausalDiT(nn.Module):
         self.rope_temporal_offset = 0.0               # frames added to every temporal position (causal_model.py:1097)
         self.kv_quant_config = None
         self._rope_cache: dict = {}
+        self._time_cache: dict = {}
         self.init_weights()
 
     def init_weights(self) -> None:
@@ -367,19 +368,44 @@ class CausalDiT(nn.Module):
         return cached[1]
 
     @torch.no_grad()
+    def _time_conditioning(self, t: torch.Tensor, like: torch.Tensor, timestep_key):
+        """(e, e0, modulated) of the timesteps t [1, F]: the time embedding, its projection to the six modulation
+        vectors per frame (wan_5b/modules/causal_model.py:1554-1564) and modulation + e0 of every block in one
+        operation (the same additions and roundings as block by block, :862-863).  A sampler evaluates the model at
+        a handful of timestep values over and over; with ``timestep_key`` (a hashable that names the values of t,
+        for instance ``(250.0, 3)``) the three tensors are computed once per value and kept until a parameter they
+        depend on is replaced or written."""
+        cfg = self.cfg
+        params = [p for seq in (self.time_embedding, self.time_projection) for p in seq.parameters()] + \
+                 [b.modulation for b in self.blocks]
+        version = tuple((p.data_ptr(), p._version) for p in params)
+        if self._time_cache.get("version") != version:
+            self._time_cache = {"version": version}
+        key = None if timestep_key is None else (timestep_key, tuple(t.shape), like.dtype, str(like.device))
+        if key is not None and key in self._time_cache:
+            return self._time_cache[key]
+        e = self.time_embedding(sinusoidal_embedding_1d(cfg.freq_dim, t.flatten()).unflatten(0, t.shape).type_as(like))
+        e0 = self.time_projection(e).unflatten(2, (6, cfg.dim))
+        modulated = self._stacked_modulation().unsqueeze(2) + e0.unsqueeze(0)   # [blocks, 1, F, 6, C]
+        if key is not None:
+            if len(self._time_cache) > 32:
+                self._time_cache = {"version": version}
+            self._time_cache[key] = (e, e0, modulated)
+        return e, e0, modulated
+
+    @torch.no_grad()
     def forward(self, x: torch.Tensor, t: torch.Tensor, context: torch.Tensor, kv_cache: list[dict],
                 current_start: int, apply_cache_updates: bool = True,
-                crossattn_cache: list[dict] | None = None) -> torch.Tensor:
+                crossattn_cache: list[dict] | None = None, timestep_key=None) -> torch.Tensor:
         """x [C_in, F, H, W] latents of one chunk, t [1, F] timesteps, context [L, text_dim];
         returns the flow prediction [C_out, F, H, W] and updates the KV cache like the reference
         (all layers' updates applied after the last block).  ``crossattn_cache``: one dictionary per layer
-        holding the projected text K / V of the current prompt (filled on first use)."""
+        holding the projected text K / V of the current prompt (filled on first use).  ``timestep_key``: a
+        hashable naming the values of ``t``; the time conditioning is then computed once per key."""
         cfg = self.cfg
         x, (f, h, w) = self.patch_embed(x)
         frame_seqlen = h * w
-        tt = t.flatten()
-        e = self.time_embedding(sinusoidal_embedding_1d(cfg.freq_dim, tt).unflatten(0, t.shape).type_as(x))
-        e0 = self.time_projection(e).unflatten(2, (6, cfg.dim))
+        e, e0, modulated = self._time_conditioning(t, x, timestep_key)
         if crossattn_cache is not None and all(c.get("is_init") for c in crossattn_cache):
             ctx = None  # every layer holds the projected K / V of this prompt: the text embedding has no reader
         else:
@@ -390,8 +416,6 @@ class CausalDiT(nn.Module):
         sink_tokens = cfg.sink_size * frame_seqlen
         max_attn = cfg.local_attn_size * frame_seqlen
         updates = []
-        # modulation + e0 of every block in one operation (the same additions and roundings as block by block)
-        modulated = self._stacked_modulation().unsqueeze(2) + e0.unsqueeze(0)   # [blocks, 1, F, 6, C]
         for i, block in enumerate(self.blocks):
             x, upd = block(x, e0, cos, sin, ctx, kv_cache[i], current_start, sink_tokens, max_attn,
                            None if crossattn_cache is None else crossattn_cache[i],

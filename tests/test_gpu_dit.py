@@ -834,3 +834,40 @@ def test_streaming_decode_hook_decodes_every_chunk_in_order_on_a_side_stream(gpu
     for i, chunk in enumerate(chunks):
         want = offline(plain[:, i * nb:(i + 1) * nb].transpose(1, 2).contiguous())
         assert torch.equal(chunk, want), i
+
+
+def test_time_conditioning_cached_per_timestep_value_gives_identical_latents(gpu):
+    """The time embedding, its projection and modulation + e0 are computed once per timestep value when the caller
+    names the value (the streaming generator does: five values per run); the latents are bit for bit those of a run
+    that recomputes them in every forward, and a parameter written in place invalidates what was kept."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=6, sink_size=2)
+    g = torch.Generator().manual_seed(12)
+    noise = torch.randn(1, 6, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    gen = StreamingGenerator(cfg, gpu, seed=12)
+    out = gen.generate(noise, ctx)
+    kept = [k for k in gen.model._time_cache if k != "version"]
+    assert len(kept) == 5 and {k[0][0] for k in kept} == {1000.0, 750.0, 500.0, 250.0, 0.0}
+    gen2 = StreamingGenerator(cfg, gpu, seed=12)
+    forward = type(gen2.model).forward
+
+    def uncached(self, *args, timestep_key=None, **kwargs):
+        return forward(self, *args, timestep_key=None, **kwargs)
+    type(gen2.model).forward = uncached
+    try:
+        ref = gen2.generate(noise, ctx)
+    finally:
+        type(gen2.model).forward = forward
+    assert torch.equal(out, ref)
+    with torch.no_grad():
+        gen.model.time_projection[1].bias.add_(0.5)
+        gen2.model.time_projection[1].bias.add_(0.5)
+    gen.kv_cache = gen2.kv_cache = None
+    again = gen.generate(noise, ctx)
+    type(gen2.model).forward = uncached
+    try:
+        ref2 = gen2.generate(noise, ctx)
+    finally:
+        type(gen2.model).forward = forward
+    assert torch.equal(again, ref2) and not torch.equal(again, out)
