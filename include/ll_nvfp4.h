@@ -354,6 +354,31 @@ int ll_gate_residual(const void* x, const void* y, int64_t B, int64_t L, int C, 
 int ll_layer_norm(const void* x, int64_t rows, int C, const void* weight, const void* bias, float eps, void* out,
                   const ll_amax_sink* amax_sink, void* stream);
 
+/*
+ * ll_adaln_modulate_amax followed by ll_nvfp4_quantize_from_sink of its result (the pairs at
+ * wan_5b/modules/causal_model.py:869-878 and :909-918 with a quantized linear layer behind them) as one launch that
+ * never writes the modulated tensor: values [Mp, C/2], scales [Mp * C / 16] in the blocked layout and amax [1] are
+ * byte for byte what the two calls give (M = B * L rows, Mp = M rounded up to 128).  The launch is one resident
+ * grid whose workgroups exchange their maxima through amax_sink (required: a buffer of LL_AMAX_PARTS slots and a
+ * fresh epoch, as for ll_adaln_modulate_amax; nothing has to read it afterwards).  A workgroup waits for the others
+ * at most spin_limit looks (about a microsecond each; a few thousand is plenty, 0 = one look) and then computes the
+ * tensor maximum itself, so the launch ends whatever else occupies the device; spin_limit < 0 makes every
+ * workgroup do that (tests of that path).  LL_ENOSUP when C is not a multiple of 64 or exceeds 3072, or when the
+ * device does not hold one wave per row of Mp at once (3072 rows on 256 compute units; with more rows per wave the
+ * launch was measured no faster than the two kernels): call the two separate entry points then.  No allocation, safe
+ * under stream capture.
+ */
+int ll_adaln_quantize(const void* x, int64_t B, int64_t L, int C, const void* scale, const void* shift,
+                      int64_t scale_stride_b, int64_t scale_stride_f, int64_t shift_stride_b, int64_t shift_stride_f,
+                      int64_t frame_seqlen, float eps, int add_one_to_scale, int rule, uint8_t* values,
+                      uint8_t* scales, float* amax, const ll_amax_sink* amax_sink, int64_t spin_limit, void* stream);
+
+/* ll_layer_norm followed by ll_nvfp4_quantize_from_sink of its result (norm3 ahead of the cross-attention query
+ * projection, wan_5b/modules/causal_model.py:892-906) as one launch; everything else as ll_adaln_quantize. */
+int ll_layer_norm_quantize(const void* x, int64_t rows, int C, const void* weight, const void* bias, float eps,
+                           int rule, uint8_t* values, uint8_t* scales, float* amax, const ll_amax_sink* amax_sink,
+                           int64_t spin_limit, void* stream);
+
 /* WanRMSNorm (wan_5b/modules/model.py:82-98): y = bf16(bf16(x * rsqrt(mean(x^2) + eps)) * w) over the
  * last dim C of x bf16 [rows, C]; w bf16 [C]. */
 int ll_rms_norm(const void* x, int64_t rows, int C, const void* weight, float eps, void* out, void* stream);

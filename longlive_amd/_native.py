@@ -72,6 +72,11 @@ _SIGNATURES = {
     "ll_gate_residual": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p, c_int64, c_int64, c_int64,
                                  c_void_p, c_void_p]),
     "ll_rms_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_float, c_void_p, c_void_p]),
+    "ll_adaln_quantize": (c_int, [c_void_p, c_int64, c_int64, c_int, c_void_p, c_void_p, c_int64, c_int64, c_int64,
+                                  c_int64, c_int64, c_float, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                  c_int64, c_void_p]),
+    "ll_layer_norm_quantize": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_float, c_int, c_void_p,
+                                       c_void_p, c_void_p, c_void_p, c_int64, c_void_p]),
     "ll_layer_norm": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_void_p]),
     "ll_release_stream_memory": (c_int, [c_void_p]),
     "ll_nvfp4_gemm_set_schedule": (c_int, [c_int]),
@@ -676,6 +681,67 @@ def adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps=1e-6, add_one_to_scale
                                              out.data_ptr(), ctypes.byref(sink), _stream())
     _check(code, "ll_adaln_modulate")
     return out
+
+
+NORM_QUANTIZE_SPIN_LIMIT = 4096  # looks a workgroup of the one-launch normalize-and-quantize kernels waits for the others
+
+
+def _norm_quantize_outputs(M: int, C: int, device):
+    Mp, Kp = padded_shape((M, C))
+    return (torch.empty((Mp, Kp // 2), dtype=torch.uint8, device=device),
+            torch.empty(Mp * Kp // 16, dtype=torch.uint8, device=device),
+            torch.empty(1, dtype=torch.float32, device=device))
+
+
+def _norm_quantize_result(code: int, what: str, values, scales, amax):
+    """None when the kernel does not take the shape (the caller runs the separate operations)."""
+    if code == -3:
+        return None
+    _check(code, what)
+    return values, scales.view(torch.float8_e4m3fn), amax
+
+
+def adaln_quantize(x, e_scale, e_shift, frame_seqlen, rule: str, eps=1e-6, add_one_to_scale=True, spin_limit=None):
+    """``quantize(adaln_modulate(x, ...).reshape(-1, C), rule)`` as one launch that never writes the modulated
+    tensor: (values, scales, amax) with the same bytes, or None when the kernel does not take the shape."""
+    _require_cuda(x, e_scale, e_shift)
+    if x.ndim != 3 or x.dtype != torch.bfloat16 or not x.is_contiguous():
+        raise ValueError("x must be a contiguous bfloat16 [B, L, C] tensor")
+    B, L, C = x.shape
+    F = L // frame_seqlen
+    for name, e in (("e_scale", e_scale), ("e_shift", e_shift)):
+        if e.shape != (B, F, 1, C) or e.dtype != torch.bfloat16 or e.stride(3) != 1:
+            raise ValueError(f"{name} must be bfloat16 [B, F, 1, C] = {(B, F, 1, C)}, got {tuple(e.shape)}")
+    values, scales, amax = _norm_quantize_outputs(B * L, C, x.device)
+    sink = _sink_struct(amax_ticket(x.device))
+    with torch.cuda.device(x.device):
+        code = load().ll_adaln_quantize(x.data_ptr(), B, L, C, e_scale.data_ptr(), e_shift.data_ptr(),
+                                        e_scale.stride(0), e_scale.stride(1), e_shift.stride(0), e_shift.stride(1),
+                                        frame_seqlen, float(eps), int(add_one_to_scale), RULE_IDS[rule],
+                                        values.data_ptr(), scales.data_ptr(), amax.data_ptr(), ctypes.byref(sink),
+                                        NORM_QUANTIZE_SPIN_LIMIT if spin_limit is None else int(spin_limit), _stream())
+    return _norm_quantize_result(code, "ll_adaln_quantize", values, scales, amax)
+
+
+def layer_norm_quantize(x, weight, bias, rule: str, eps=1e-6, spin_limit=None):
+    """``quantize(layer_norm(x, weight, bias).reshape(-1, C), rule)`` as one launch, like :func:`adaln_quantize`."""
+    _require_cuda(x, weight, bias)
+    if x.dtype != torch.bfloat16 or any(t is not None and t.dtype != torch.bfloat16 for t in (weight, bias)):
+        raise ValueError("layer_norm takes bfloat16 input, weight and bias")
+    C = x.shape[-1]
+    x2 = x.reshape(-1, C)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    w = None if weight is None else weight.contiguous()
+    b = None if bias is None else bias.contiguous()
+    values, scales, amax = _norm_quantize_outputs(x2.shape[0], C, x.device)
+    sink = _sink_struct(amax_ticket(x.device))
+    with torch.cuda.device(x.device):
+        code = load().ll_layer_norm_quantize(x2.data_ptr(), x2.shape[0], C, _ptr(w), _ptr(b), float(eps), RULE_IDS[rule],
+                                             values.data_ptr(), scales.data_ptr(), amax.data_ptr(), ctypes.byref(sink),
+                                             NORM_QUANTIZE_SPIN_LIMIT if spin_limit is None else int(spin_limit),
+                                             _stream())
+    return _norm_quantize_result(code, "ll_layer_norm_quantize", values, scales, amax)
 
 
 def gate_residual(x, y, gate, frame_seqlen):

@@ -1,25 +1,11 @@
 // Memory-bound fused kernels of the DiT block for gfx950: 3-D RoPE apply, adaLN modulate, RMSNorm.
 // All of them read bf16 with 128-bit loads, compute in fp32 and round where the reference rounds.
 #include "ll_common.h"
+#include "norm_rows.h"
 
 #pragma clang fp contract(off)
 
 namespace ll {
-
-__device__ __forceinline__ void unpack8(const uint4& v, float (&f)[8]) {
-  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    f[2 * i] = __uint_as_float(w[i] << 16);
-    f[2 * i + 1] = __uint_as_float(w[i] & 0xFFFF0000u);
-  }
-}
-__device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
-  uint32_t w[4];
-#pragma unroll
-  for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(f[2 * i], f[2 * i + 1]);
-  return make_uint4(w[0], w[1], w[2], w[3]);
-}
 
 // ----------------------------------------------------------------------------- RoPE
 // utils/rope_triton.py:36-81.  One thread = 8 consecutive elements (4 rotation pairs) of one (token, head).
@@ -53,13 +39,6 @@ __global__ __launch_bounds__(256) void rope_kernel(const uint16_t* __restrict__ 
   *reinterpret_cast<uint4*>(out + (s * N + n) * (int64_t)D + c) = o;
 }
 
-// Row kernels: one wave per row (no workgroup barrier; a row's sums are wave reductions), four rows per
-// workgroup.  A lane holds NCH groups of 8 elements: NCH = 6 covers C = 3072 exactly, 16 anything up to 8192.
-constexpr int kRowThreads = 256;
-constexpr int kRowsPerWg = kRowThreads / 64;
-constexpr int kMaxChunks = 16;  // 8 elements each: C <= 64 * 16 * 8 = 8192
-constexpr int kMaxRowLength = 64 * kMaxChunks * 8;
-
 // ----------------------------------------------------------------------------- adaLN
 // utils/adaln_triton.py:36-86.  One workgroup = one token row.
 template <int NCH>
@@ -73,60 +52,14 @@ __global__ __launch_bounds__(kRowThreads) void adaln_kernel(const uint16_t* __re
   const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
   if (row >= rows) return;
   const int64_t b = row / L, l = row - b * L, f = l / frame_seqlen;
-  const uint16_t* xr = x + row * (int64_t)C;
-  const int nchunks = C >> 3;
-  const uint16_t* scr = scale + b * sc_sb + f * sc_sf;
-  const uint16_t* shr = shift + b * sh_sb + f * sh_sf;
-  float v[NCH][8];
-  uint4 sraw[NCH], hraw[NCH];  // requested up front: their latency runs under the two reductions
-  float sum = 0.0f;
-#pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int c = lane + i * 64;
-    if (c < nchunks) {
-      unpack8(*reinterpret_cast<const uint4*>(xr + c * 8), v[i]);
-      sraw[i] = *reinterpret_cast<const uint4*>(scr + c * 8);
-      hraw[i] = *reinterpret_cast<const uint4*>(shr + c * 8);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) sum += v[i][j];
-    }
-  }
-  const float inv_c = 1.0f / (float)C;
-  const float mean = wave_sum_dpp(sum) * inv_c;
-  float sq = 0.0f;
-#pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int c = lane + i * 64;
-    if (c < nchunks) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        v[i][j] -= mean;
-        sq += v[i][j] * v[i][j];
-      }
-    }
-  }
-  const float var = wave_sum_dpp(sq) * inv_c;
-  const float rstd = 1.0f / sqrtf(var + eps);
+  uint4 packed[NCH];
+  float out_max = adaln_row<NCH>(x + row * (int64_t)C, scale + b * sc_sb + f * sc_sf, shift + b * sh_sb + f * sh_sf, C, eps,
+                                 add_one, lane, packed);
   uint16_t* orow = out + row * (int64_t)C;
-  float out_max = 0.0f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = lane + i * 64;
-    if (c < nchunks) {
-      float s8[8], h8[8], y[8];
-      unpack8(sraw[i], s8);
-      unpack8(hraw[i], h8);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const float xn = round_to_bf16(v[i][j] * rstd);
-        const float s = add_one ? round_to_bf16(s8[j] + 1.0f) : s8[j];
-        const float prod = round_to_bf16(xn * s);
-        y[j] = prod + h8[j];
-      }
-      const uint4 packed = pack8(y);
-      *reinterpret_cast<uint4*>(orow + c * 8) = packed;
-      out_max = abs_max_bf16x8(packed, out_max);
-    }
+    if (c < (C >> 3)) *reinterpret_cast<uint4*>(orow + c * 8) = packed[i];
   }
   if (sink.parts) {
     out_max = wave_max(out_max);
@@ -145,53 +78,13 @@ __global__ __launch_bounds__(kRowThreads) void layernorm_kernel(const uint16_t* 
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * kRowsPerWg + (threadIdx.x >> 6);
   if (row >= rows) return;
-  const uint16_t* xr = x + row * (int64_t)C;
-  const int nchunks = C >> 3;
-  float v[NCH][8];
-  uint4 wraw[NCH], braw[NCH];  // requested up front: their latency runs under the two reductions
-  float sum = 0.0f;
-#pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int c = lane + i * 64;
-    if (c < nchunks) {
-      unpack8(*reinterpret_cast<const uint4*>(xr + c * 8), v[i]);
-      wraw[i] = w ? *reinterpret_cast<const uint4*>(w + c * 8) : make_uint4(0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u);
-      braw[i] = b ? *reinterpret_cast<const uint4*>(b + c * 8) : make_uint4(0, 0, 0, 0);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) sum += v[i][j];
-    }
-  }
-  const float inv_c = 1.0f / (float)C;
-  const float mean = wave_sum_dpp(sum) * inv_c;
-  float sq = 0.0f;
-#pragma unroll
-  for (int i = 0; i < NCH; ++i) {
-    const int c = lane + i * 64;
-    if (c < nchunks) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        v[i][j] -= mean;
-        sq += v[i][j] * v[i][j];
-      }
-    }
-  }
-  const float var = wave_sum_dpp(sq) * inv_c;
-  const float rstd = 1.0f / sqrtf(var + eps);
+  uint4 packed[NCH];
+  float out_max = layernorm_row<NCH>(x + row * (int64_t)C, w, b, C, eps, lane, packed);
   uint16_t* orow = out + row * (int64_t)C;
-  float out_max = 0.0f;
 #pragma unroll
   for (int i = 0; i < NCH; ++i) {
     const int c = lane + i * 64;
-    if (c < nchunks) {
-      float w8[8], b8[8], y[8];
-      unpack8(wraw[i], w8);
-      unpack8(braw[i], b8);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) y[j] = (v[i][j] * rstd) * w8[j] + b8[j];
-      const uint4 packed = pack8(y);
-      *reinterpret_cast<uint4*>(orow + c * 8) = packed;
-      out_max = abs_max_bf16x8(packed, out_max);
-    }
+    if (c < (C >> 3)) *reinterpret_cast<uint4*>(orow + c * 8) = packed[i];
   }
   if (sink.parts) {
     out_max = wave_max(out_max);

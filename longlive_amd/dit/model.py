@@ -70,15 +70,30 @@ class WanLayerNorm(nn.LayerNorm):
         return super().forward(x).type_as(x)
 
 
-def _project_shared(x: torch.Tensor, layers, amax: torch.Tensor | None = None, amax_outs=None) -> list[torch.Tensor]:
+class QuantizedActivation:
+    """An activation that exists only as the NVFP4 operand of the layers that read it (``operand``, built for
+    ``layers[0]``'s activation config) together with the shape the bf16 tensor would have had."""
+
+    def __init__(self, operand, shape) -> None:
+        self.operand, self.shape = operand, tuple(shape)
+        self.device = operand.values.device
+
+
+def _project_shared(x, layers, amax: torch.Tensor | None = None, amax_outs=None) -> list[torch.Tensor]:
     """Apply several linear layers to the same input.  Quantized layers with the same activation config
     share one quantized operand (bit-identical to quantizing per layer, as the reference does).  ``amax`` is
     the amax ticket that the kernel which produced ``x`` was given; ``amax_outs`` (one entry per layer, ``None``
     for none) are tickets that receive the absolute maximum of a layer's output, which only the quantized path
-    can deliver: the return value says whether it did."""
+    can deliver: the return value says whether it did.  ``x`` may be a :class:`QuantizedActivation`."""
     first = layers[0]
-    if all(isinstance(m, FourOverSixLinear) for m in layers) and all(
-            m.config.get_activation_config() == first.config.get_activation_config() for m in layers):
+    same_config = all(isinstance(m, FourOverSixLinear) for m in layers) and all(
+        m.config.get_activation_config() == first.config.get_activation_config() for m in layers)
+    if isinstance(x, QuantizedActivation):
+        if not same_config:
+            raise ValueError("a quantized activation can only feed quantized layers with one activation config")
+        outs = FourOverSixLinear.forward_quantized_together(layers, x.operand, amax_outs)
+        return [y.reshape(*x.shape[:-1], -1) for y in outs], True
+    if same_config:
         xq = first.quantize_input(x.reshape(-1, x.shape[-1]), amax=amax)
         outs = FourOverSixLinear.forward_quantized_together(layers, xq, amax_outs)
         return [y.reshape(*x.shape[:-1], -1) for y in outs], True
@@ -222,6 +237,9 @@ class CrossAttention(nn.Module):
 
 
 class DiTBlock(nn.Module):
+    # normalize and quantize in one launch where a quantized layer reads the result (the same bytes either way)
+    fuse_norm_quantize = True
+
     def __init__(self, dim: int, ffn_dim: int, num_heads: int, eps: float = 1e-6) -> None:
         super().__init__()
         self.dim, self.eps = dim, eps
@@ -240,8 +258,9 @@ class DiTBlock(nn.Module):
         up, act, down = self.ffn
         if isinstance(up, FourOverSixLinear) and getattr(act, "approximate", None) == "tanh":
             h_amax = _native.amax_ticket(y.device) if isinstance(down, FourOverSixLinear) else None
-            h = up.forward_quantized(up.quantize_input(y.reshape(-1, y.shape[-1]), amax=y_amax),
-                                     activation="gelu_tanh", amax_out=h_amax).reshape(*y.shape[:-1], -1)
+            yq = y.operand if isinstance(y, QuantizedActivation) else up.quantize_input(
+                y.reshape(-1, y.shape[-1]), amax=y_amax)
+            h = up.forward_quantized(yq, activation="gelu_tanh", amax_out=h_amax).reshape(*y.shape[:-1], -1)
         else:
             h, h_amax = act(up(y)), None
         return _project_out(down, h, h_amax, residual, gate, gate_rows)
@@ -255,18 +274,41 @@ class DiTBlock(nn.Module):
         num_frames, frame_seqlen = e.shape[1], x.shape[1] // e.shape[1]
         e = (self.modulation.unsqueeze(1) + e if modulated is None else modulated).chunk(6, dim=2)
         gates = [g.reshape(-1, g.shape[-1]) for g in (e[2], e[5])]  # [B*F, C] views, one row per frame
-        y_amax = _native.amax_ticket(x.device) if isinstance(self.self_attn.q, FourOverSixLinear) else None
-        y = adaln_modulate(x, e[1], e[0], frame_seqlen, eps=self.eps, amax_out=y_amax)
+        sa = self.self_attn
+        y, y_amax = self._normalized_for([sa.q, sa.k, sa.v], x, scale=e[1], shift=e[0], frame_seqlen=frame_seqlen)
         x, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size,
                                    input_amax=y_amax, residual=x, gate=gates[0], gate_rows=frame_seqlen,
                                    global_sink_tokens=global_sink_tokens, rope_fn=rope_fn,
                                    collect_kv_amax=collect_kv_amax)
-        y_amax = _native.amax_ticket(x.device) if isinstance(self.cross_attn.q, FourOverSixLinear) else None
-        x = self.cross_attn(self.norm3(x, amax_out=y_amax), context, crossattn_cache, residual=x, input_amax=y_amax)
-        y_amax = _native.amax_ticket(x.device) if isinstance(self.ffn[0], FourOverSixLinear) else None
-        y = adaln_modulate(x, e[4], e[3], frame_seqlen, eps=self.eps, amax_out=y_amax)
+        y, y_amax = self._normalized_for([self.cross_attn.q], x, norm=self.norm3)
+        x = self.cross_attn(y, context, crossattn_cache, residual=x, input_amax=y_amax)
+        up = self.ffn[0]
+        fused_ffn = isinstance(up, FourOverSixLinear) and getattr(self.ffn[1], "approximate", None) == "tanh"
+        y, y_amax = self._normalized_for([up], x, scale=e[4], shift=e[3], frame_seqlen=frame_seqlen,
+                                         operand_ok=fused_ffn)
         x = self._feed_forward(y, y_amax, x, gates[1], frame_seqlen)
         return x, update
+
+    def _normalized_for(self, layers, x, *, scale=None, shift=None, frame_seqlen=0, norm=None, operand_ok=True):
+        """The adaLN modulation of ``x`` (``scale`` / ``shift`` given) or ``norm(x)`` as input of ``layers``:
+        ``(activation, amax ticket)``.  When the layers are quantized with one activation config, the activation
+        is produced directly as their NVFP4 operand (a :class:`QuantizedActivation`, no ticket) where the
+        one-launch kernel takes the shapes; else as a bf16 tensor whose maximum the ticket carries."""
+        first = layers[0]
+        quantized = isinstance(first, FourOverSixLinear)
+        if (quantized and operand_ok and self.fuse_norm_quantize and all(isinstance(m, FourOverSixLinear)
+                and m.config.get_activation_config() == first.config.get_activation_config() for m in layers)):
+            if norm is None:
+                xq = first.quantize_normalized_input(x, scale=scale, shift=shift, frame_seqlen=frame_seqlen,
+                                                     eps=self.eps)
+            else:
+                xq = first.quantize_normalized_input(x, weight=norm.weight, bias=norm.bias, eps=norm.eps)
+            if xq is not None:
+                return QuantizedActivation(xq, x.shape), None
+        ticket = _native.amax_ticket(x.device) if quantized else None
+        if norm is None:
+            return adaln_modulate(x, scale, shift, frame_seqlen, eps=self.eps, amax_out=ticket), ticket
+        return norm(x, amax_out=ticket), ticket
 
 
 class CausalHead(nn.Module):

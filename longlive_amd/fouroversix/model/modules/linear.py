@@ -129,6 +129,35 @@ class FourOverSixLinear(nn.Linear):
         the amax ticket of the kernel that produced ``x2d``, if it was given one."""
         return quantize_to_fp4(x2d, self.config.get_activation_config(), amax=amax)
 
+    def quantize_normalized_input(self, x: torch.Tensor, *, scale=None, shift=None, frame_seqlen: int = 0,
+                                  weight=None, bias=None, eps: float = 1e-6) -> QuantizedTensor | None:
+        """``quantize_input`` of the adaLN modulation of ``x`` [B, L, C] (``scale`` / ``shift`` [B, F, 1, C] given:
+        ``LayerNorm(x) * (1 + scale) + shift``) or of its LayerNorm with optional ``weight`` / ``bias``, flattened
+        to 2-D, as one launch that never writes the normalized tensor (an extension; the reference runs the
+        normalization and the layer's quantization separately, wan_5b/modules/causal_model.py:869-878, 892-906,
+        909-918).  The bytes are those of the separate operations.  ``None`` when that launch does not take the
+        input or the activation config, and the caller runs the separate operations."""
+        from .... import _native
+        from ...quantize.frontend import _unsupported
+
+        config = self.config.get_activation_config()
+        if not (x.is_cuda and x.dtype == torch.bfloat16 and x.ndim == 3 and x.is_contiguous()) or \
+                _unsupported(x[0], config) is not None:
+            return None
+        rule = config.scale_rule.value
+        if scale is not None:
+            if scale.dtype != torch.bfloat16 or shift.dtype != torch.bfloat16:
+                return None
+            out = _native.adaln_quantize(x, scale, shift, frame_seqlen, rule, eps=eps)
+        else:
+            if any(t is not None and t.dtype != torch.bfloat16 for t in (weight, bias)):
+                return None
+            out = _native.layer_norm_quantize(x, weight, bias, rule, eps=eps)
+        if out is None:
+            return None
+        shape = (x.shape[0] * x.shape[1], x.shape[2])
+        return QuantizedTensor(*out, config.dtype, shape, config.scale_rule, _native.padded_shape(shape))
+
     @staticmethod
     def forward_quantized_together(layers, xq: QuantizedTensor, amax_outs=None) -> list[torch.Tensor]:
         """``[m.forward_quantized(xq) for m in layers]`` as one GEMM launch when the layers have the same shape

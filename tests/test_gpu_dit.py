@@ -871,3 +871,29 @@ def test_time_conditioning_cached_per_timestep_value_gives_identical_latents(gpu
     finally:
         type(gen2.model).forward = forward
     assert torch.equal(again, ref2) and not torch.equal(again, out)
+
+
+@pytest.mark.parametrize("dim,heads,ffn,F,h,w", [(256, 2, 512, 2, 8, 8), (3072, 24, 14336, 3, 22, 40)])
+def test_normalizing_and_quantizing_in_one_launch_leaves_the_block_bit_identical(gpu, dim, heads, ffn, F, h, w):
+    """The three normalizations of a block that feed quantized layers (adaLN ahead of self-attention and of the
+    FFN, norm3 ahead of cross-attention) produce the layers' NVFP4 operand directly; the block's output and the
+    K / V it hands to the cache are those of the separate operations, bit for bit."""
+    torch.manual_seed(1)
+    L, T = F * h * w, 32
+    block = DiTBlock(dim, ffn, heads).to(gpu).bfloat16()
+    block, _ = quantize_model_with_filter(block, ModelQuantizationConfig(), use_default_filtered_modules=True,
+                                          materialize_for_inference=True, verbose=False)
+    cache = kvc.initialize_kv_cache(1, L, 3, heads, 128, KV, gpu)[0]
+    cos, sin = rope_cos_sin(build_rope_angles(128), F, h, w, 0, gpu)
+    g = torch.Generator().manual_seed(5)
+    x = (torch.randn(1, L, dim, generator=g) * 2).bfloat16().to(gpu)
+    e = torch.randn(1, F, 6, dim, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(1, T, dim, generator=g).bfloat16().to(gpu)
+    outs = []
+    with torch.no_grad():
+        for fuse in (True, False):
+            block.fuse_norm_quantize = fuse
+            y, (_, _, info) = block(x, e, cos, sin, ctx, cache, 0, sink_tokens=L)
+            outs.append((y.clone(), info["new_k"].clone(), info["new_v"].clone()))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
