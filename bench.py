@@ -333,6 +333,9 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the attention / block / end-to-end figures")
     ap.add_argument("--workload", choices=["linears", "attention", "block", "block_release", "e2e", "copy", "quantize", "quantize_static"], default="linears")
+    ap.add_argument("--separate-norm-quantize", action="store_true",
+                    help="block / e2e workloads: adaLN or LayerNorm and the quantization behind it as two launches "
+                         "(for comparisons; the default is the one-launch kernel where it applies)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives are part of this path); use --gpus 1")
@@ -346,6 +349,9 @@ def main() -> None:
         sys.exit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     cfg = QuantizationConfig(scale_rule="mse")
+    if args.separate_norm_quantize:
+        from longlive_amd.dit import DiTBlock
+        DiTBlock.fuse_norm_quantize = False
     if args.workload == "copy":
         # plain device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
