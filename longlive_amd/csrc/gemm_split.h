@@ -105,7 +105,10 @@ inline PersistentPlan plan_persistent(int64_t M, int64_t N, int64_t Kp, int n_pr
   // (sustained, K = 14336: 0.53 - 0.58 of the f16 peak against 0.47 - 0.53), but one wave per SIMD has nobody to hide
   // a tile's first loads and its epilogue behind, and the tiles behind the whole rounds pay for their partial tiles:
   // inside the DiT block, with bias, GELU or the gated residual in the epilogue, every product measured slower
-  // (FFN-down 243 against 221 us, FFN-up 300 against 224 us).
+  // (FFN-down 243 against 221 us, FFN-up 300 against 224 us).  Alone, the launch wins where K is long and every
+  // workgroup has at least a whole tile (7040 x 3072 x 14336: 505 against 542 us; 4096 x 4096 x 14336: 355 against
+  // 385 us); an automatic choice that takes it for exactly those shapes left the block of 7040 tokens where it was
+  // (4.55 - 4.57 against 4.54 - 4.55 ms), so it is not made.
   if (schedule == -1 /* LL_GEMM_AUTO */) return plan;
   int64_t rounds = tiles / cus;
   // A few left-over tiles would be cut into many thin parts each (or leave workgroups without a single K step, and

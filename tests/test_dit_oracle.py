@@ -143,3 +143,39 @@ def test_cached_keys_are_attended_together_with_the_chunk():
     cvc = np.broadcast_to(o.round_bf16(rng.standard_normal((1, H, D)).astype(np.float32)), (8, H, D)).copy()
     q_like = dit_oracle.block_forward(x, e, ctx, p, cos, sin, big, cvc, H, FS)[0]
     assert np.isfinite(q_like).all()
+
+
+def test_requantization_turns_a_relative_difference_into_about_two_thirds_of_its_square_root():
+    """Where the block's end-to-end bar comes from.  Two bf16 tensors a relative Frobenius distance eps apart
+    (eps = 1e-3 is the bar of one W4A4 linear against the oracle) quantize to NVFP4 tensors that are about
+    0.65 * sqrt(eps) apart: a fraction ~eps / step of the elements lands on the other side of a rounding boundary
+    and moves by a whole e2m1 step, a quarter to a third of its value.  A difference that moves the tensor maximum
+    re-derives every block scale: one bf16 ulp on that one element puts the quantized tensors 5e-2 apart, and no
+    difference can do more than the quantization noise itself (8.7e-2 for Gaussian data).  The block re-quantizes
+    its activations three times behind the attention, each time diluted by the residual stream it is added to;
+    its bar of 6e-2 on the output is one such re-derivation of the scales (measured: 3.4e-2)."""
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((256, 1024)).astype(np.float32)
+
+    def quantized(t):
+        bits = o.f32_to_bf16(t)
+        v, s, a, pad = o.quantize_to_fp4(bits, "mse")
+        return o.dequantize(v, s, a, "mse", pad, t.shape).astype(np.float64)
+
+    base = quantized(x)
+    noise_floor = np.linalg.norm(base - x) / np.linalg.norm(x)
+    assert 0.08 < noise_floor < 0.095
+    big = np.unravel_index(np.argmax(np.abs(x)), x.shape)
+    for eps in (1e-4, 3e-4, 1e-3):
+        n = rng.standard_normal(x.shape).astype(np.float32)
+        n[big] = 0.0  # the tensor maximum stays where it is
+        moved = x + eps * n * np.linalg.norm(x) / np.linalg.norm(n)
+        r = np.linalg.norm(quantized(moved) - base) / np.linalg.norm(base)
+        assert 0.5 * np.sqrt(eps) <= r <= 0.8 * np.sqrt(eps), (eps, r)
+    # the tensor maximum alone, moved by one bf16 ulp (2^-8): every block scale is re-derived from it, 92 % of the
+    # dequantized values change and the tensors are 5e-2 apart; moved by 5 % they are as far apart as the noise floor
+    for factor, lo, hi in ((1.0 + 2.0 ** -8, 0.03, 0.065), (1.05, 0.07, 1.5 * noise_floor)):
+        moved = x.copy()
+        moved[big] *= factor
+        r = np.linalg.norm(quantized(moved) - base) / np.linalg.norm(base)
+        assert lo <= r <= hi, (factor, r)
