@@ -60,6 +60,7 @@ def test_block_against_oracle_with_cache(gpu, dim, heads, ffn):
         ref, rk, v = dit_oracle.block_forward(_f(x)[0], _f(e0)[0], _f(ctx)[0], params, ocs, osn, cached_k, cached_v,
                                               heads, fs)
         r = _rel(_f(y)[0], ref)
+        print(f"block against oracle, dim {dim}, chunk {chunk}: relative Frobenius {r:.3e}")
         assert r <= 6e-2, (chunk, r)
         kvc.apply_cache_update(cache, ce, le, info, KV)
         # oracle cache: quantize-on-write of this chunk's un-smoothed K and V
