@@ -361,8 +361,10 @@ int ll_layer_norm(const void* x, int64_t rows, int C, const void* weight, const 
  * byte for byte what the two calls give (M = B * L rows, Mp = M rounded up to 128).  The launch is one resident
  * grid whose workgroups exchange their maxima through amax_sink (required: a buffer of LL_AMAX_PARTS slots and a
  * fresh epoch, as for ll_adaln_modulate_amax; nothing has to read it afterwards).  A workgroup waits for the others
- * at most spin_limit looks (about a microsecond each; a few thousand is plenty, 0 = one look) and then computes the
- * tensor maximum itself, so the launch ends whatever else occupies the device; spin_limit < 0 makes every
+ * at most spin_limit + 1 looks at the slots (one to two microseconds each; with the device to itself a launch's
+ * workgroups arrive within ~10 us of each other, and 64 is plenty) and then computes the maxima of the rows of the
+ * workgroups it has not seen itself, so the launch ends whatever else occupies the device (another stream may hold
+ * compute units for milliseconds) and costs at most one extra pass over the rows; spin_limit < 0 makes every
  * workgroup do that (tests of that path).  LL_ENOSUP when C is not a multiple of 64 or exceeds 3072, or when the
  * device does not hold one wave per row of Mp at once (3072 rows on 256 compute units; with more rows per wave the
  * launch was measured no faster than the two kernels): call the two separate entry points then.  No allocation, safe

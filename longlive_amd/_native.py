@@ -683,7 +683,7 @@ def adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps=1e-6, add_one_to_scale
     return out
 
 
-NORM_QUANTIZE_SPIN_LIMIT = 4096  # looks a workgroup of the one-launch normalize-and-quantize kernels waits for the others
+NORM_QUANTIZE_SPIN_LIMIT = 64  # looks (1-2 us each) a workgroup of the one-launch normalize-and-quantize kernels waits for the others
 
 
 def _norm_quantize_outputs(M: int, C: int, device):

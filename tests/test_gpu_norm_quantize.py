@@ -132,3 +132,22 @@ def test_one_launch_recorded_into_a_graph_replays_with_fresh_inputs(gpu):
         _, want = _separate_adaln(x, scale, shift, L, "mse")
         torch.cuda.synchronize()
         _same(recorded, want, f"replay with seed {seed}")
+
+
+def test_results_hold_while_another_stream_occupies_the_device(gpu):
+    """Large matrix products on a side stream compete for the compute units while the one-launch kernel runs: its
+    workgroups then do not all start together, some give up waiting and compute the missing rows' maxima
+    themselves.  Every launch ends and every result equals the two-launch bytes."""
+    L, C, frames = 2640, 3072, 3
+    x, scale, shift = _inputs(gpu, L, C, frames, seed=51)
+    _, want = _separate_adaln(x, scale, shift, L // frames, "mse")
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    a = torch.randn(8192, 8192, device=gpu, dtype=torch.bfloat16)
+    with torch.cuda.stream(side):
+        for _ in range(40):
+            a @ a
+    results = [_native.adaln_quantize(x, scale, shift, L // frames, "mse", spin_limit=2) for _ in range(40)]
+    torch.cuda.synchronize()
+    for i, got in enumerate(results):
+        _same(got, want, f"launch {i} beside the side stream")
