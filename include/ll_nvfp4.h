@@ -51,7 +51,9 @@ int ll_version(void);
  * (current device, stream), if any, after waiting for the launches that still use it - for callers that create
  * streams as they go.  Launches on a stream that is being captured into a graph never allocate: they use the set a
  * reserve call or an earlier launch left on that stream, or fall back to a division of the work that needs none.
- * No counterpart in the reference.
+ * A set that a captured launch has used belongs to the recorded graph as well: it is not freed when the stream
+ * later needs a larger one (the old set is kept aside), only by ll_release_stream_memory, which must therefore not
+ * be called while such a graph may still be replayed.  No counterpart in the reference.
  */
 int ll_release_stream_memory(void* stream);
 

@@ -6,13 +6,21 @@
 // counters are zero whenever no launch is running: every kernel that uses them leaves them at zero.
 #include <map>
 #include <mutex>
+#include <vector>
 
 #include "ll_common.h"
 
 namespace ll {
 
+// A set that a capturing stream has used is part of a recorded graph, which will use the same addresses at every
+// replay: such a set is never freed when a later launch needs a larger one (it is kept aside until the release call).
+struct ScratchEntry {
+  StreamScratch current{};
+  bool recorded = false;
+  std::vector<StreamScratch> retired;
+};
 static std::mutex g_scratch_mutex;
-static std::map<std::pair<int, hipStream_t>, StreamScratch> g_scratch;
+static std::map<std::pair<int, hipStream_t>, ScratchEntry> g_scratch;
 
 static void free_scratch(StreamScratch& w) {
   if (w.records) (void)hipFree(w.records);  // waits for the launches that still use it
@@ -24,28 +32,37 @@ int stream_scratch(int dev, hipStream_t stream, size_t record_bytes, size_t coun
                    bool* missing, const char* what) {
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   if (missing) *missing = false;
-  if (!may_allocate) {
+  if (!may_allocate) {  // the stream is being captured
     const auto it = g_scratch.find({dev, stream});
-    if (it == g_scratch.end() || it->second.record_bytes < record_bytes || it->second.n_counters < counters) {
+    if (it == g_scratch.end() || it->second.current.record_bytes < record_bytes ||
+        it->second.current.n_counters < counters) {
       if (missing) *missing = true;
       return LL_OK;
     }
-    out = it->second;
+    it->second.recorded = true;
+    out = it->second.current;
     return LL_OK;
   }
-  StreamScratch& w = g_scratch[{dev, stream}];
+  ScratchEntry& entry = g_scratch[{dev, stream}];
+  StreamScratch& w = entry.current;
   if (w.record_bytes < record_bytes || w.n_counters < counters) {
     const size_t want_bytes = record_bytes > w.record_bytes ? record_bytes : w.record_bytes;
     size_t want_counters = counters > w.n_counters ? counters : w.n_counters;
     if (want_counters < 4096) want_counters = 4096;
-    free_scratch(w);
+    if (entry.recorded && w.records) {
+      entry.retired.push_back(w);
+      w = StreamScratch{};
+      entry.recorded = false;
+    } else {
+      free_scratch(w);
+    }
     hipError_t e = hipMalloc(reinterpret_cast<void**>(&w.records), want_bytes);
     if (e == hipSuccess) e = hipMalloc(reinterpret_cast<void**>(&w.counters), want_counters * sizeof(int));
     if (e == hipSuccess) e = hipMemsetAsync(w.counters, 0, want_counters * sizeof(int), stream);
     if (e != hipSuccess) {
       set_error("%s: cannot set up %zu bytes for partial results: %s", what, want_bytes, hipGetErrorString(e));
       free_scratch(w);
-      g_scratch.erase({dev, stream});
+      if (entry.retired.empty()) g_scratch.erase({dev, stream});
       return LL_ELAUNCH;
     }
     w.record_bytes = want_bytes;
@@ -59,7 +76,8 @@ int release_stream_scratch(int dev, hipStream_t stream) {
   std::lock_guard<std::mutex> lock(g_scratch_mutex);
   const auto it = g_scratch.find({dev, stream});
   if (it == g_scratch.end()) return LL_OK;
-  free_scratch(it->second);
+  free_scratch(it->second.current);
+  for (StreamScratch& old : it->second.retired) free_scratch(old);
   g_scratch.erase(it);
   return LL_OK;
 }

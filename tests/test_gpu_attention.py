@@ -823,6 +823,18 @@ def test_launch_on_a_capturing_stream_never_allocates(gpu):
         torch.cuda.synchronize()
         assert torch.equal(out3, eager)
         _native.attention_bf16(q, k, v, 128 ** -0.5)   # eager work between the replays
+    # The recorded launches keep the addresses they were recorded with.  When the stream later needs a larger set
+    # (the persistent GEMM's partial tiles are larger than the attention's), the recorded one is kept aside, not
+    # freed: the graph still replays.
+    with torch.cuda.stream(side3):
+        _native.gemm_reserve(4096, 4096, 14336)
+        _native.attention_bf16(q, k, v, 128 ** -0.5)
+    side3.synchronize()
+    out3.zero_()
+    graph3.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out3, eager)
+    del graph3
     with torch.cuda.stream(side3):
         _native.attention_release()
     _native.attention_release()   # a stream without memory: nothing to do
