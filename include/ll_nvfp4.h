@@ -122,6 +122,15 @@ int ll_nvfp4_quantize_from_sink(const void* x, int64_t M, int64_t K, int64_t ldx
                                 uint8_t* values, uint8_t* scales, float* amax,
                                 const ll_amax_sink* amax_sink, void* stream);
 
+/* Two ll_nvfp4_quantize_from_sink calls on tensors of the same shape, leading dimension and rule as one launch: the
+ * K and the V of a chunk on their way into the cache (wan_5b/modules/causal_model.py:1420-1429 quantizes one after
+ * the other).  Each tensor has its own sink (two buffers: one launch cannot read two epochs of one buffer apart),
+ * outputs and amax word; the bytes equal those of the two separate calls. */
+int ll_nvfp4_quantize_pair_from_sinks(const void* x0, const void* x1, int64_t M, int64_t K, int64_t ldx, int rule,
+                                      uint8_t* values0, uint8_t* values1, uint8_t* scales0, uint8_t* scales1,
+                                      float* amax0, float* amax1, const ll_amax_sink* amax_sink0,
+                                      const ll_amax_sink* amax_sink1, void* stream);
+
 /*
  * Replaces QuantizedTensor.dequantize (fouroversix/src/fouroversix/quantize/quantized_tensor.py:184-214):
  * out[r, c] = cast(((e2m1 * e4m3) * amax) / (e2m1_max * e4m3_max)) for r < M, c < K; ldo in elements.

@@ -31,6 +31,8 @@ _SIGNATURES = {
                                   c_void_p, c_void_p]),
     "ll_nvfp4_quantize_from_sink": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p, c_void_p,
                                             c_void_p, c_void_p]),
+    "ll_nvfp4_quantize_pair_from_sinks": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_void_p,
+                                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ll_nvfp4_dequantize": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64, c_int64, c_int64,
                                     c_void_p, c_int, c_int64, c_void_p]),
     "ll_nvfp4_gemm_tnt": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float,
@@ -354,6 +356,43 @@ def quantize(x: torch.Tensor, rule: str, amax: torch.Tensor | None = None, out=N
     if out is not None:
         return out
     return values, scales.view(torch.float8_e4m3fn), amax_t
+
+
+def quantize_pair(x0: torch.Tensor, x1: torch.Tensor, rule: str, ticket0: AmaxTicket, ticket1: AmaxTicket, out0, out1):
+    """``quantize(x0, rule, amax=ticket0, out=out0)`` and ``quantize(x1, rule, amax=ticket1, out=out1)`` as one
+    launch (the K and the V of a chunk on their way into the cache): two bf16 [M, K] tensors of the same shape and
+    row stride, each with the amax ticket of its producer (tickets of two different sink buffers) and its
+    (values, scale_factors, amax) buffers.  The bytes equal those of the two calls."""
+    for t in (ticket0, ticket1):
+        if not isinstance(t, AmaxTicket):
+            raise TypeError("quantize_pair needs the amax tickets of the two producers")
+        _check_consumer(t)
+    if ticket0.parts.data_ptr() == ticket1.parts.data_ptr():
+        raise ValueError("the two tickets must belong to two sink buffers")
+    _require_cuda(x0, x1)
+    if x0.ndim != 2 or x0.shape != x1.shape or x0.dtype != torch.bfloat16 or x1.dtype != torch.bfloat16:
+        raise ValueError("quantize_pair expects two 2-D bfloat16 tensors of the same shape")
+    if x0.stride(1) != 1:
+        x0 = x0.contiguous()
+    if x1.stride(1) != 1 or x1.stride(0) != x0.stride(0):
+        x1 = x1.contiguous()
+        if x1.stride(0) != x0.stride(0):
+            x0 = x0.contiguous()
+    M, K = x0.shape
+    Mp, Kp = padded_shape((M, K))
+    for values, scales, amax_t in (out0, out1):
+        if (values.shape != (Mp, Kp // 2) or values.dtype != torch.uint8 or scales.numel() != Mp * Kp // 16
+                or scales.element_size() != 1 or amax_t.numel() != 1 or amax_t.dtype != torch.float32
+                or not (values.is_contiguous() and scales.is_contiguous())):
+            raise ValueError("out buffers do not match the padded NVFP4 shape of the inputs")
+    s0, s1 = ticket0.struct(), ticket1.struct()
+    with torch.cuda.device(x0.device):
+        code = load().ll_nvfp4_quantize_pair_from_sinks(
+            x0.data_ptr(), x1.data_ptr(), M, K, x0.stride(0), RULE_IDS[rule], out0[0].data_ptr(), out1[0].data_ptr(),
+            out0[1].data_ptr(), out1[1].data_ptr(), out0[2].data_ptr(), out1[2].data_ptr(), ctypes.byref(s0),
+            ctypes.byref(s1), _stream())
+    _check(code, "ll_nvfp4_quantize_pair_from_sinks")
+    return out0, out1
 
 
 def dequantize(values, scales, amax, rule: str, padded, original, dtype: torch.dtype) -> torch.Tensor:

@@ -60,15 +60,37 @@ __global__ __launch_bounds__(kThreads) void amax_partial_kernel(const uint16_t* 
 // GENERIC = false: x is 16-byte aligned with ldx a multiple of 8 and K a multiple of 64, so every block is two
 // whole 16-byte pieces and only rows beyond M need care (zeros).  GENERIC = true handles any K, ldx and
 // alignment element by element at the edges.
+// What differs between the tensors of one launch (one or two tensors of the same shape: the K and V of a chunk).
+struct QuantJob {
+  const uint16_t* x;
+  uint8_t* values;
+  uint8_t* scales;
+  float* amax_io;
+  const float* parts;
+  const unsigned long long* sink_parts;
+  uint32_t sink_epoch_base;
+  const uint32_t* sink_epoch_offset;
+};
+struct QuantJobs {
+  QuantJob j[2];
+  int n;  // the first half of the workgroups takes j[0], the second half j[1]
+};
+
 template <int RULE, bool GENERIC>
-__global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __restrict__ x, int64_t M, int64_t K,
-                                                            int64_t ldx, int64_t Kp, uint8_t* __restrict__ values,
-                                                            uint8_t* __restrict__ scales, float* __restrict__ amax_io,
-                                                            const float* __restrict__ parts, int amax_given,
-                                                            int64_t total_tiles,
-                                                            const unsigned long long* __restrict__ sink_parts,
-                                                            uint32_t sink_epoch_base,
-                                                            const uint32_t* __restrict__ sink_epoch_offset) {
+__global__ __launch_bounds__(kThreads) void quantize_kernel(QuantJobs jobs, int64_t M, int64_t K, int64_t ldx, int64_t Kp,
+                                                            int amax_given, int64_t total_tiles) {
+  // The tensor this workgroup works on (uniform selects, no indexing of the argument block).
+  const uint32_t per_job = jobs.n == 2 ? gridDim.x >> 1 : gridDim.x;
+  const bool second = jobs.n == 2 && blockIdx.x >= per_job;
+  const uint32_t wg_in_job = second ? blockIdx.x - per_job : blockIdx.x;
+  const uint16_t* __restrict__ x = second ? jobs.j[1].x : jobs.j[0].x;
+  uint8_t* __restrict__ values = second ? jobs.j[1].values : jobs.j[0].values;
+  uint8_t* __restrict__ scales = second ? jobs.j[1].scales : jobs.j[0].scales;
+  float* __restrict__ amax_io = second ? jobs.j[1].amax_io : jobs.j[0].amax_io;
+  const float* __restrict__ parts = second ? jobs.j[1].parts : jobs.j[0].parts;
+  const unsigned long long* __restrict__ sink_parts = second ? jobs.j[1].sink_parts : jobs.j[0].sink_parts;
+  const uint32_t sink_epoch_base = second ? jobs.j[1].sink_epoch_base : jobs.j[0].sink_epoch_base;
+  const uint32_t* __restrict__ sink_epoch_offset = second ? jobs.j[1].sink_epoch_offset : jobs.j[0].sink_epoch_offset;
   __shared__ float s_red[kThreads / 64];
   __shared__ uint32_t s_scales[2][128];  // two staged 512-byte scale tiles in blocked order
   __shared__ ScaleEntry s_tab[128];
@@ -94,7 +116,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
     if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = m;
     __syncthreads();
     amax = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-    if (blockIdx.x == 0 && threadIdx.x == 0) amax_io[0] = amax;
+    if (wg_in_job == 0 && threadIdx.x == 0) amax_io[0] = amax;
   }
 
   // The fast path needs every block maximum to stay below amax (so block scales stay within e4m3 range: true by
@@ -124,7 +146,7 @@ __global__ __launch_bounds__(kThreads) void quantize_kernel(const uint16_t* __re
   // The grid is a multiple of 32 workgroups, so a workgroup's next tile is its current one plus the grid size:
   // the tile's row and column advance by constants, and no division is left in the loop.
   const uint32_t n_tiles = (uint32_t)total_tiles;
-  const uint32_t grid = gridDim.x, wg = blockIdx.x;
+  const uint32_t grid = per_job, wg = wg_in_job;
   const uint32_t first_tile = ((wg >> 5) * 8u + (wg & 7u)) * 4u + ((wg >> 3) & 3u);
   const uint32_t step_y = grid / tiles_x, step_x = grid - step_y * tiles_x;
 
@@ -256,46 +278,71 @@ static int resident_workgroups(int rule, bool generic, int64_t* out) {
   return LL_OK;
 }
 
-static int quantize_impl(const void* x, int64_t M, int64_t K, int64_t ldx, int rule, uint8_t* values, uint8_t* scales,
-                         float* amax, int amax_given, float* workspace, const ll_amax_sink* sink, void* stream) {
+// One host-side description per tensor of a launch.
+struct QuantRequest {
+  const void* x;
+  uint8_t* values;
+  uint8_t* scales;
+  float* amax;
+  float* workspace;
+  const ll_amax_sink* sink;
+};
+
+// n = 1 or 2 tensors of the same shape, leading dimension, rule and source of the amax, in one launch: the
+// resident workgroups are split evenly between them.
+static int quantize_impl(const QuantRequest* req, int n, int64_t M, int64_t K, int64_t ldx, int rule, int amax_given,
+                         void* stream) {
   using namespace ll;
-  LL_REQUIRE(x && values && scales && amax, "ll_nvfp4_quantize: null pointer");
+  LL_REQUIRE(n == 1 || n == 2, "ll_nvfp4_quantize: %d tensors in one launch (1 or 2)", n);
   LL_REQUIRE(M > 0 && K > 0 && ldx >= K, "ll_nvfp4_quantize: bad shape M=%lld K=%lld ldx=%lld", (long long)M,
              (long long)K, (long long)ldx);
   LL_REQUIRE(rule >= 0 && rule <= 4, "ll_nvfp4_quantize: unknown scale rule %d", rule);
-  LL_REQUIRE(amax_given || workspace || sink, "ll_nvfp4_quantize: workspace required to compute amax");
-  LL_REQUIRE(!sink || (sink->parts && sink_is_valid(sink)),
-             "ll_nvfp4_quantize_from_sink: amax sink needs an 8-byte aligned buffer and a non-zero epoch");
-  LL_REQUIRE((reinterpret_cast<uintptr_t>(values) & 7) == 0 && (reinterpret_cast<uintptr_t>(scales) & 3) == 0,
-             "ll_nvfp4_quantize: outputs must be 8-byte (values) / 4-byte (scales) aligned");
   const int64_t Mp = round_up(M, 128), Kp = round_up(K, 64);
   const int64_t total_tiles = (Kp / 64) * (Mp / 128);
   LL_REQUIRE(total_tiles < (1ll << 31), "ll_nvfp4_quantize: tensor too large for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const uint16_t* xp = static_cast<const uint16_t*>(x);
-  if (!amax_given && !sink) {
-    hipLaunchKernelGGL(amax_partial_kernel, dim3(kAmaxParts), dim3(kThreads), 0, s, xp, M, K, ldx, workspace);
-    LL_CHECK_LAUNCH("amax_partial_kernel");
+  QuantJobs jobs{};
+  jobs.n = n;
+  bool generic = (K % 64) != 0 || (ldx % 8) != 0;
+  for (int i = 0; i < n; ++i) {
+    const QuantRequest& r = req[i];
+    LL_REQUIRE(r.x && r.values && r.scales && r.amax, "ll_nvfp4_quantize: null pointer");
+    LL_REQUIRE(amax_given || r.workspace || r.sink, "ll_nvfp4_quantize: workspace required to compute amax");
+    LL_REQUIRE(!r.sink || (r.sink->parts && sink_is_valid(r.sink)),
+               "ll_nvfp4_quantize_from_sink: amax sink needs an 8-byte aligned buffer and a non-zero epoch");
+    LL_REQUIRE((reinterpret_cast<uintptr_t>(r.values) & 7) == 0 && (reinterpret_cast<uintptr_t>(r.scales) & 3) == 0,
+               "ll_nvfp4_quantize: outputs must be 8-byte (values) / 4-byte (scales) aligned");
+    generic = generic || (reinterpret_cast<uintptr_t>(r.x) & 15) != 0;
+    QuantJob& j = jobs.j[i];
+    j.x = static_cast<const uint16_t*>(r.x);
+    j.values = r.values;
+    j.scales = r.scales;
+    j.amax_io = r.amax;
+    j.parts = r.workspace;
+    j.sink_parts = r.sink ? reinterpret_cast<const unsigned long long*>(r.sink->parts) : nullptr;
+    j.sink_epoch_base = r.sink ? r.sink->epoch : 0u;
+    j.sink_epoch_offset = r.sink ? r.sink->epoch_offset : nullptr;
+    if (!amax_given && !r.sink) {
+      hipLaunchKernelGGL(amax_partial_kernel, dim3(kAmaxParts), dim3(kThreads), 0, s, j.x, M, K, ldx, r.workspace);
+      LL_CHECK_LAUNCH("amax_partial_kernel");
+    }
   }
-  const unsigned long long* sink_parts = sink ? reinterpret_cast<const unsigned long long*>(sink->parts) : nullptr;
-  const uint32_t sink_epoch = sink ? sink->epoch : 0u;
-  const uint32_t* sink_epoch_offset = sink ? sink->epoch_offset : nullptr;
-  const bool generic = (K % 64) != 0 || (ldx % 8) != 0 || (reinterpret_cast<uintptr_t>(x) & 15) != 0;
   // One workgroup per tile up to what the chip holds at once (the launch is persistent: every workgroup has to be
   // resident from the start, or the ones that wait would run after the others have finished).
   int64_t resident = 0;
   if (int rc = resident_workgroups(rule, generic, &resident)) return rc;
   const int64_t padded_tiles = (total_tiles + 31) & ~(int64_t)31;  // whole groups of 32 for the XCD-aware tile order
-  const int64_t resident32 = resident & ~(int64_t)31;
-  const dim3 grid((unsigned)(padded_tiles < resident32 ? padded_tiles : resident32));
+  int64_t share = (resident / n) & ~(int64_t)31;                  // workgroups per tensor
+  if (share < 32) share = 32;
+  const dim3 grid((unsigned)((padded_tiles < share ? padded_tiles : share) * n));
 #define LL_LAUNCH_Q(R)                                                                                                  \
   do {                                                                                                                  \
     if (generic)                                                                                                        \
-      hipLaunchKernelGGL((quantize_kernel<R, true>), grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales,    \
-                         amax, workspace, amax_given, total_tiles, sink_parts, sink_epoch, sink_epoch_offset);                            \
+      hipLaunchKernelGGL((quantize_kernel<R, true>), grid, dim3(kThreads), 0, s, jobs, M, K, ldx, Kp, amax_given,      \
+                         total_tiles);                                                                                  \
     else                                                                                                                \
-      hipLaunchKernelGGL((quantize_kernel<R, false>), grid, dim3(kThreads), 0, s, xp, M, K, ldx, Kp, values, scales,   \
-                         amax, workspace, amax_given, total_tiles, sink_parts, sink_epoch, sink_epoch_offset);                            \
+      hipLaunchKernelGGL((quantize_kernel<R, false>), grid, dim3(kThreads), 0, s, jobs, M, K, ldx, Kp, amax_given,     \
+                         total_tiles);                                                                                  \
   } while (0)
   switch (rule) {
     case LL_RULE_STATIC_6: LL_LAUNCH_Q(LL_RULE_STATIC_6); break;
@@ -311,7 +358,8 @@ static int quantize_impl(const void* x, int64_t M, int64_t K, int64_t ldx, int r
 
 extern "C" int ll_nvfp4_quantize(const void* x, int64_t M, int64_t K, int64_t ldx, int rule, uint8_t* values,
                                  uint8_t* scales, float* amax, int amax_given, float* workspace, void* stream) {
-  return quantize_impl(x, M, K, ldx, rule, values, scales, amax, amax_given, workspace, nullptr, stream);
+  const QuantRequest r{x, values, scales, amax, workspace, nullptr};
+  return quantize_impl(&r, 1, M, K, ldx, rule, amax_given, stream);
 }
 
 // One workgroup of kAmaxParts threads.  Every thread reads the word before anyone writes it, so all agree on
@@ -341,7 +389,22 @@ extern "C" int ll_nvfp4_quantize_from_sink(const void* x, int64_t M, int64_t K, 
                                            const ll_amax_sink* amax_sink, void* stream) {
   using namespace ll;
   LL_REQUIRE(amax_sink, "ll_nvfp4_quantize_from_sink: null amax sink");
-  return quantize_impl(x, M, K, ldx, rule, values, scales, amax, 0, nullptr, amax_sink, stream);
+  const QuantRequest r{x, values, scales, amax, nullptr, amax_sink};
+  return quantize_impl(&r, 1, M, K, ldx, rule, 0, stream);
+}
+
+extern "C" int ll_nvfp4_quantize_pair_from_sinks(const void* x0, const void* x1, int64_t M, int64_t K, int64_t ldx,
+                                                 int rule, uint8_t* values0, uint8_t* values1, uint8_t* scales0,
+                                                 uint8_t* scales1, float* amax0, float* amax1,
+                                                 const ll_amax_sink* amax_sink0, const ll_amax_sink* amax_sink1,
+                                                 void* stream) {
+  using namespace ll;
+  LL_REQUIRE(amax_sink0 && amax_sink1, "ll_nvfp4_quantize_pair_from_sinks: null amax sink");
+  LL_REQUIRE(values0 != values1 && scales0 != scales1 && amax0 != amax1,
+             "ll_nvfp4_quantize_pair_from_sinks: the two tensors need outputs of their own");
+  const QuantRequest r[2] = {{x0, values0, scales0, amax0, nullptr, amax_sink0},
+                             {x1, values1, scales1, amax1, nullptr, amax_sink1}};
+  return quantize_impl(r, 2, M, K, ldx, rule, 0, stream);
 }
 
 // ----------------------------------------------------------------------------- entry point that allocates nothing
@@ -394,5 +457,6 @@ extern "C" int ll_nvfp4_quantize_noalloc(const void* x, int64_t M, int64_t K, in
              (long long)M, (long long)K, (long long)LL_NOALLOC_MAX_ELEMENTS);
   float* ws = nullptr;
   if (int rc = scratch_address(&ws)) return rc;
-  return quantize_impl(x, M, K, ldx, rule, values, scales, amax, 0, ws, nullptr, stream);
+  const QuantRequest r{x, values, scales, amax, ws, nullptr};
+  return quantize_impl(&r, 1, M, K, ldx, rule, 0, stream);
 }

@@ -286,13 +286,19 @@ def apply_cache_update(cache: dict, current_end: int, local_end_index: int, info
         n_insert = (info["local_end_index"] - info["local_start_index"]) // blk
         rule = kv_quant_config.scale_rule.value
         for bi in range(n_insert):
+            blocks, slots, tickets = [], [], []
             for name, new in (("k", info["new_k"]), ("v", info["new_v"])):
-                slot: QuantizedTensor = cache[name][start_blk + bi]
-                block = new[0, bi * blk:(bi + 1) * blk].reshape(-1, new.shape[-1])
+                slots.append(cache[name][start_blk + bi])
+                blocks.append(new[0, bi * blk:(bi + 1) * blk].reshape(-1, new.shape[-1]))
                 # A chunk of one block is quantized as a whole: if its producer left the tensor maximum behind
                 # (an amax ticket of the layer's own sink), the quantization takes it from there.
-                ticket = info.get(f"new_{name}_amax") if n_insert == 1 and new.shape[1] == blk else None
-                _native.quantize(block, rule, amax=ticket, out=(slot.values, slot.scale_factors, slot.amax))
+                tickets.append(info.get(f"new_{name}_amax") if n_insert == 1 and new.shape[1] == blk else None)
+            outs = [(slot.values, slot.scale_factors, slot.amax) for slot in slots]
+            if tickets[0] is not None and tickets[1] is not None and blocks[0].shape == blocks[1].shape:
+                _native.quantize_pair(blocks[0], blocks[1], rule, tickets[0], tickets[1], outs[0], outs[1])  # one launch
+            else:
+                for block, ticket, out in zip(blocks, tickets, outs):
+                    _native.quantize(block, rule, amax=ticket, out=out)
     cache["global_end_index"].fill_(current_end)
     cache["local_end_index"].fill_(local_end_index)
     cache["_global_end"] = current_end

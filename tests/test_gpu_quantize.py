@@ -183,3 +183,27 @@ def test_four_over_six_choice_on_ties_and_near_ties(gpu, rule):
     tiny[0, 0] = 300.0  # tensor amax: the other blocks get scale byte 0 or subnormal scale bytes
     for x in (lattice, nudged, magn, two_level, tiny):
         _check(bits_of(torch.from_numpy(x).bfloat16()), rule, gpu)
+
+
+@pytest.mark.parametrize("rows,C,rule", [(300, 256, "mse"), (2640, 3072, "mse"), (130, 128, "static_6")])
+def test_two_tensors_in_one_launch_equal_the_oracle(gpu, rows, C, rule):
+    """The K and V of a chunk go into the cache as one launch (two tensors of one shape, each with the amax its
+    producer left in a sink of its own): bytes and amax of both equal the oracle's, i.e. those of two launches."""
+    g = torch.Generator().manual_seed(rows + C)
+    xs = [(torch.randn(rows, C, generator=g) * s).bfloat16().to(gpu) for s in (1.0, 7.0)]
+    sinks = [_native.PrivateAmaxSink(gpu), _native.PrivateAmaxSink(gpu)]
+    tickets = [s.ticket() for s in sinks]
+    ys = [_native.layer_norm(x, None, None, amax_out=t).reshape(-1, 128) for x, t in zip(xs, tickets)]
+    Mp, Kp = _native.padded_shape(tuple(ys[0].shape))
+    outs = [(torch.empty((Mp, Kp // 2), dtype=torch.uint8, device=gpu),
+             torch.empty(Mp * Kp // 16, dtype=torch.uint8, device=gpu),
+             torch.empty(1, dtype=torch.float32, device=gpu)) for _ in range(2)]
+    _native.quantize_pair(ys[0], ys[1], rule, tickets[0], tickets[1], outs[0], outs[1])
+    for y, (values, scales, amax) in zip(ys, outs):
+        v, s, a, _ = o.quantize_to_fp4(bits_of(y), rule)
+        assert float(amax.cpu()) == float(a)
+        assert np.array_equal(u8(scales), s) and np.array_equal(u8(values), v)
+    with pytest.raises(ValueError, match="two sink buffers"):
+        t = sinks[0].ticket()
+        _native.layer_norm(xs[0], None, None, amax_out=t)
+        _native.quantize_pair(ys[0], ys[1], rule, t, t, outs[0], outs[1])
