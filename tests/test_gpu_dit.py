@@ -706,9 +706,9 @@ def test_modulation_of_all_blocks_in_one_operation_is_what_each_block_would_form
 
 
 def test_block_forward_recorded_into_a_graph_replays_bit_for_bit(gpu):
-    """One DiT block forward over an FP4 cache slot recorded into a HIP graph (27 kernels of the library, seven amax
-    tickets) and replayed with new inputs.  A recorded launch runs again with the epoch it was recorded with, so
-    the tickets of the recording come from a ReplayableAmaxSink, whose first recorded launch moves every epoch of
+    """One DiT block forward over an FP4 cache slot recorded into a HIP graph (some twenty kernels of the library,
+    among them the one-launch normalize-and-quantize kernels, whose workgroups meet through the sink) and replayed
+    with new inputs.  A recorded launch runs again with the epoch it was recorded with, so the tickets of the recording come from a ReplayableAmaxSink, whose first recorded launch moves every epoch of
     the replay past those of the previous one.  Each of four replays - with eager forwards of the same block,
     which use the device's own sink, and synchronisations in between - must equal the eager result bit for bit;
     a replay that met stale maxima of an earlier replay would quantize against too large an amax."""
