@@ -151,3 +151,17 @@ def test_results_hold_while_another_stream_occupies_the_device(gpu):
     torch.cuda.synchronize()
     for i, got in enumerate(results):
         _same(got, want, f"launch {i} beside the side stream")
+
+
+def test_batches_of_two_with_strided_scale_and_shift(gpu):
+    """B = 2: scale / shift rows are picked by (batch, frame); they arrive as strided views of one [B, F, 6, C]
+    tensor, as the block passes them."""
+    B, L, C, frames = 2, 192, 512, 3
+    g = torch.Generator().manual_seed(61)
+    x = (torch.randn(B, L, C, generator=g) * 2).to(gpu).bfloat16()
+    e = (torch.randn(B, frames, 6, C, generator=g) * 0.5).to(gpu).bfloat16()
+    scale, shift = e[:, :, 4:5], e[:, :, 3:4]
+    t = _native.amax_ticket(gpu)
+    y = _native.adaln_modulate(x, scale, shift, L // frames, amax_out=t)
+    want = _native.quantize(y.reshape(-1, C), "mse", amax=t)
+    _same(_native.adaln_quantize(x, scale, shift, L // frames, "mse"), want, "B = 2")
