@@ -38,7 +38,7 @@ class StreamingGenerator:
                  skip_dead_cache_writes: bool = True, sampler: str = "euler", sample_shift: float = 5.0,
                  multi_shot_sink: bool = False, shot_clean_recache: bool = False,
                  use_relative_rope: bool = False, multi_shot_rope_offset: float = 0.0,
-                 guidance_scale: float = 1.0) -> None:
+                 guidance_scale: float = 1.0, skip_dead_recache_tail: bool = True) -> None:
         if sampler not in ("euler", "unipc"):
             raise ValueError(f"unknown sampler {sampler!r}")
         self.cfg, self.device = cfg, torch.device(device)
@@ -67,6 +67,9 @@ class StreamingGenerator:
             block.self_attn.use_relative_rope = use_relative_rope
         self.cache_text_kv = cache_text_kv
         self.skip_dead_cache_writes = skip_dead_cache_writes
+        # A pass that is run only to rewrite the cache (clean-context pass, context blocks of a continuation) has no
+        # reader for its prediction: the last block stops behind its K / V producers and the head is left out.
+        self.skip_dead_recache_tail = skip_dead_recache_tail
 
     def reset_cache(self, frame_seq_length: int) -> None:
         cfg = self.cfg
@@ -120,7 +123,8 @@ class StreamingGenerator:
             x = initial_latent[0, start:start + nb].transpose(0, 1).contiguous()
             out[0, start:start + nb] = initial_latent[0, start:start + nb]
             for cache, text in zip(caches, (first_text, negative_context)):
-                self.model(x, torch.zeros((1, nb), device=self.device), text, cache, start * fs, timestep_key=(0.0, nb))
+                self.model(x, torch.zeros((1, nb), device=self.device), text, cache, start * fs, timestep_key=(0.0, nb),
+                           cache_only=self.skip_dead_recache_tail)
         # projected text K / V per layer: one prompt per call, so they are computed by the first forward only
         xcache = [{"is_init": False} for _ in range(cfg.num_layers)] if self.cache_text_kv else None
         contexts = list(context) if isinstance(context, (list, tuple)) else None
@@ -182,7 +186,7 @@ class StreamingGenerator:
                 if is_scene_cut and self.shot_clean_recache:
                     kvc.zero_kv_data(cache, start * fs, self.global_sink_size * fs)
                 self.model(x, torch.zeros((1, f), device=self.device), text, cache, start * fs, crossattn_cache=xc,
-                           timestep_key=(0.0, f))
+                           timestep_key=(0.0, f), cache_only=self.skip_dead_recache_tail)
                 if is_scene_cut:
                     kvc.pin_current_chunk(cache, f * fs, cfg.sink_size * fs)
             if on_chunk is not None:

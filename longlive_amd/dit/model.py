@@ -145,8 +145,11 @@ class CausalSelfAttention(nn.Module):
         self.use_relative_rope = False  # set on the module by the pipeline (pipeline/causal_diffusion_inference.py:316)
 
     def forward(self, x, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size, *, input_amax=None,
-                residual=None, gate=None, gate_rows=0, global_sink_tokens=0, rope_fn=None, collect_kv_amax=True):
+                residual=None, gate=None, gate_rows=0, global_sink_tokens=0, rope_fn=None, collect_kv_amax=True,
+                keys_only=False):
         """``input_amax``: the amax ticket the producer of ``x`` was given, if any.
+        ``keys_only``: the caller reads the cache update only (the chunk's K and V), not the output: everything
+        behind the K / V producers is left out and the output is None.
         ``collect_kv_amax``: leave the maxima of the chunk's K and V behind for the cache write (a forward whose
         cache update will not be applied has no use for them, and they cost ~3 us).
         ``global_sink_tokens``: leading tokens of the stream that stay in the cache for good (multi-shot mode).
@@ -172,8 +175,11 @@ class CausalSelfAttention(nn.Module):
         if self.use_relative_rope:
             if rope_fn is None:
                 raise ValueError("use_relative_rope needs rope_fn")
-            q = self.norm_q(q).view(b, s, n, d)
             k = self.norm_k(k).view(b, s, n, d)
+            if keys_only:
+                return None, kvc.kv_cache_update_only(k, v, kv_cache, current_start, sink_tokens, max_attention_size,
+                                                      global_sink_tokens)
+            q = self.norm_q(q).view(b, s, n, d)
             out_amax = None
             out, update = kvc.kv_cache_attention_relative(q, k, v, kv_cache, current_start, sink_tokens, rope_fn,
                                                           max_attention_size=max_attention_size,
@@ -196,13 +202,19 @@ class CausalSelfAttention(nn.Module):
             roped_q = rope_apply(q[0], cos, sin).unsqueeze(0)
             roped_k = rope_apply(k[0], cos, sin).unsqueeze(0)
             smooth_k = None
-        out_amax = _native.amax_ticket(x.device) if isinstance(self.o, FourOverSixLinear) else None
-        out, update = kvc.kv_cache_attention(roped_q, roped_k, v, kv_cache, current_start, sink_tokens,
-                                             max_attention_size=max_attention_size, smoothed_key=smooth_k,
-                                             amax_out=out_amax, global_sink_tokens=global_sink_tokens)
+        if keys_only:
+            out, update = None, kvc.kv_cache_update_only(roped_k, v, kv_cache, current_start, sink_tokens,
+                                                         max_attention_size, global_sink_tokens)
+        else:
+            out_amax = _native.amax_ticket(x.device) if isinstance(self.o, FourOverSixLinear) else None
+            out, update = kvc.kv_cache_attention(roped_q, roped_k, v, kv_cache, current_start, sink_tokens,
+                                                 max_attention_size=max_attention_size, smoothed_key=smooth_k,
+                                                 amax_out=out_amax, global_sink_tokens=global_sink_tokens)
         if update[2] is not None:
             update[2]["new_k_amax"] = k_amax
             update[2]["new_v_amax"] = v_amax if v_amax_written else None
+        if keys_only:
+            return None, update
         return _project_out(self.o, out.flatten(2), out_amax, residual, gate, gate_rows), update
 
 
@@ -266,11 +278,14 @@ class DiTBlock(nn.Module):
         return _project_out(down, h, h_amax, residual, gate, gate_rows)
 
     def forward(self, x, e, cos, sin, context, kv_cache, current_start, sink_tokens, max_attention_size=None,
-                crossattn_cache=None, global_sink_tokens=0, rope_fn=None, collect_kv_amax=True, modulated=None):
+                crossattn_cache=None, global_sink_tokens=0, rope_fn=None, collect_kv_amax=True, modulated=None,
+                keys_only=False):
         """x [1, L, C]; e [1, F, 6, C]; returns (x, (current_end, local_end_index, cache_update_info)).
         The tensor amax that each activation quantization needs is produced by the kernel that writes the
         activation wherever that kernel is one of this package's.  ``modulated`` is ``self.modulation.unsqueeze(1)
-        + e`` when the caller has already formed it (the model does so for all its blocks in one operation)."""
+        + e`` when the caller has already formed it (the model does so for all its blocks in one operation).
+        ``keys_only``: the block's output has no reader (last block of a pass that only rewrites the cache):
+        the block stops behind the producers of the chunk's K and V and returns ``(None, update)``."""
         num_frames, frame_seqlen = e.shape[1], x.shape[1] // e.shape[1]
         e = (self.modulation.unsqueeze(1) + e if modulated is None else modulated).chunk(6, dim=2)
         gates = [g.reshape(-1, g.shape[-1]) for g in (e[2], e[5])]  # [B*F, C] views, one row per frame
@@ -279,7 +294,9 @@ class DiTBlock(nn.Module):
         x, update = self.self_attn(y, cos, sin, kv_cache, current_start, sink_tokens, max_attention_size,
                                    input_amax=y_amax, residual=x, gate=gates[0], gate_rows=frame_seqlen,
                                    global_sink_tokens=global_sink_tokens, rope_fn=rope_fn,
-                                   collect_kv_amax=collect_kv_amax)
+                                   collect_kv_amax=collect_kv_amax, keys_only=keys_only)
+        if keys_only:
+            return None, update
         y, y_amax = self._normalized_for([self.cross_attn.q], x, norm=self.norm3)
         x = self.cross_attn(y, context, crossattn_cache, residual=x, input_amax=y_amax)
         up = self.ffn[0]
@@ -438,12 +455,16 @@ class CausalDiT(nn.Module):
     @torch.no_grad()
     def forward(self, x: torch.Tensor, t: torch.Tensor, context: torch.Tensor, kv_cache: list[dict],
                 current_start: int, apply_cache_updates: bool = True,
-                crossattn_cache: list[dict] | None = None, timestep_key=None) -> torch.Tensor:
+                crossattn_cache: list[dict] | None = None, timestep_key=None, cache_only: bool = False):
         """x [C_in, F, H, W] latents of one chunk, t [1, F] timesteps, context [L, text_dim];
         returns the flow prediction [C_out, F, H, W] and updates the KV cache like the reference
         (all layers' updates applied after the last block).  ``crossattn_cache``: one dictionary per layer
         holding the projected text K / V of the current prompt (filled on first use).  ``timestep_key``: a
-        hashable naming the values of ``t``; the time conditioning is then computed once per key."""
+        hashable naming the values of ``t``; the time conditioning is then computed once per key.
+        ``cache_only``: the caller runs the pass for its cache update and does not read the prediction (the
+        clean-context pass of the chunk loop, pipeline/causal_diffusion_inference.py:639-647).  The last block then
+        stops behind its K / V producers and the head is left out - nothing that reaches the cache depends on them -
+        and the return value is None."""
         cfg = self.cfg
         x, (f, h, w) = self.patch_embed(x)
         frame_seqlen = h * w
@@ -463,10 +484,13 @@ class CausalDiT(nn.Module):
                            None if crossattn_cache is None else crossattn_cache[i],
                            global_sink_tokens=self.global_sink_size * frame_seqlen,
                            rope_fn=lambda frames, first: self._rope(frames, h, w, first, x.device),
-                           collect_kv_amax=apply_cache_updates, modulated=modulated[i])
+                           collect_kv_amax=apply_cache_updates, modulated=modulated[i],
+                           keys_only=cache_only and i == len(self.blocks) - 1)
             updates.append(upd)
         if apply_cache_updates:
             for i, (cur_end, loc_end, info) in enumerate(updates):
                 kvc.apply_cache_update(kv_cache[i], cur_end, loc_end, info, self.kv_quant_config)
+        if cache_only:
+            return None
         x = self.head(x, e.unsqueeze(2))
         return self.unpatchify(x[0].flatten(0, 1) if x.dim() == 4 else x[0], (f, h, w))

@@ -212,6 +212,17 @@ def kv_cache_attention(q: torch.Tensor, key_to_cache: torch.Tensor, v: torch.Ten
     return out.unsqueeze(0), (current_start + S, local_end, info)
 
 
+def kv_cache_update_only(key_to_cache: torch.Tensor, v: torch.Tensor, cache: dict, current_start: int, sink_tokens: int,
+                         max_attention_size: int | None = None, global_sink_tokens: int = 0):
+    """The ``(current_end, local_end_index, cache_update_info)`` that :func:`kv_cache_attention` (or the relative
+    variant) returns beside its output, without the attention: for a layer whose output nobody reads (the last
+    layer of a pass that is run only to rewrite the cache)."""
+    S = key_to_cache.shape[1]
+    _, info, local_end = plan_cache_step(cache, current_start, S, sink_tokens, max_attention_size, global_sink_tokens)
+    info["new_k"], info["new_v"] = key_to_cache, v
+    return current_start + S, local_end, info
+
+
 def kv_cache_attention_relative(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cache: dict, current_start: int,
                                 sink_tokens: int, rope_fn, softmax_scale: float | None = None,
                                 max_attention_size: int | None = None, global_sink_tokens: int = 0):

@@ -898,3 +898,28 @@ def test_normalizing_and_quantizing_in_one_launch_leaves_the_block_bit_identical
             outs.append((y.clone(), info["new_k"].clone(), info["new_v"].clone()))
     for a, b in zip(*outs):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("relative", [False, True])
+def test_leaving_out_the_unread_tail_of_the_clean_context_pass_changes_nothing(gpu, relative):
+    """The clean-context pass of a chunk (timestep 0, pipeline/causal_diffusion_inference.py:639-647) is run for its
+    cache writes; its prediction has no reader.  With the last block stopped behind its K / V producers and the head
+    left out, the latents and every byte of the cache are those of the full pass - for the plain run, with scene
+    cuts, a continuation from given latents, and relative RoPE (whose cache holds un-rotated keys)."""
+    cfg = DiTConfig(dim=256, ffn_dim=512, num_heads=2, num_layers=2, in_dim=8, out_dim=8, text_dim=64, text_len=16,
+                    num_frame_per_block=2, local_attn_size=8, sink_size=2)
+    g = torch.Generator().manual_seed(13)
+    noise = torch.randn(1, 12, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    first = torch.randn(1, 2, 8, 16, 16, generator=g).bfloat16().to(gpu)
+    ctx = torch.randn(10, 64, generator=g).bfloat16().to(gpu)
+    gens = [StreamingGenerator(cfg, gpu, seed=4, multi_shot_sink=not relative, use_relative_rope=relative,
+                               skip_dead_recache_tail=skip) for skip in (True, False)]
+    cuts = () if relative else (2, 4)
+    a, b = (gen.generate(noise, ctx, scene_cuts=cuts, initial_latent=first) for gen in gens)
+    assert torch.equal(a, b)
+    for la, lb in zip(gens[0].kv_cache, gens[1].kv_cache):
+        for key in ("_global_end", "_local_end", "_pinned_start", "_pinned_len"):
+            assert la[key] == lb[key], key
+        for sa, sb in zip(la["k"] + la["v"], lb["k"] + lb["v"]):
+            assert torch.equal(sa.values, sb.values) and torch.equal(sa.amax, sb.amax)
+            assert torch.equal(sa.scale_factors.view(torch.uint8), sb.scale_factors.view(torch.uint8))
