@@ -59,6 +59,49 @@ def measured_traffic_bytes():
             + keys["write_size_kib_per_launch"] * keys["write_scale"]) * 1024.0
 
 
+def live_traffic_bytes():
+    """The same figure measured now: four child runs of this file under `rocprofv3 --pmc` (FETCH_SIZE and WRITE_SIZE,
+    each for the linear set and for a device copy of known size that calibrates the counter), started before this
+    process touches the GPU.  Returns (bytes, details) or (None, reason)."""
+    import csv
+    import shutil
+    import subprocess
+    import tempfile
+
+    if shutil.which("rocprofv3") is None:
+        return None, "rocprofv3 not found"
+    out = tempfile.mkdtemp(prefix="ll_traffic_", dir=os.environ.get("TMPDIR", "/tmp"))
+    env = dict(os.environ, TMPDIR=os.environ.get("TMPDIR", "/tmp"))
+
+    def counter(name, workload, kernel):
+        d = os.path.join(out, f"{name}_{workload}")
+        cmd = ["rocprofv3", "--pmc", name, "--output-format", "csv", "-d", d, "-o", "p", "--", sys.executable,
+               os.path.abspath(__file__), "--no-cpu-baseline", "--no-extras", "--workload", workload, "--steps", "5", "--warmup", "2"]
+        subprocess.run(cmd, env=env, cwd=ROOT, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, timeout=150, check=True)
+        values = []
+        with open(os.path.join(d, "p_counter_collection.csv")) as f:
+            for row in csv.DictReader(f):
+                if row["Counter_Name"] == name and kernel(row):
+                    values.append(float(row["Counter_Value"]))
+        if not values:
+            raise RuntimeError(f"no {name} rows for {workload}")
+        return sum(values) / len(values)
+
+    ffn_up = lambda r: "gemm_w4a4_kernel<4, 2>" in r["Kernel_Name"] and r["Grid_Size"] == "315392"
+    copy = lambda r: "copyBuffer" in r["Kernel_Name"]
+    try:
+        fetch, write = counter("FETCH_SIZE", "linears", ffn_up), counter("WRITE_SIZE", "linears", ffn_up)
+        fetch_copy, write_copy = counter("FETCH_SIZE", "copy", copy), counter("WRITE_SIZE", "copy", copy)
+    except (OSError, subprocess.SubprocessError, RuntimeError, KeyError, ValueError) as e:
+        return None, f"{type(e).__name__}: {e}"
+    finally:
+        shutil.rmtree(out, ignore_errors=True)
+    copied_kib = 256.0 * 1024.0  # the copy workload moves 256 MiB each way
+    details = {"fetch_size_kib_per_launch": fetch, "fetch_scale": copied_kib / fetch_copy,
+               "write_size_kib_per_launch": write, "write_scale": copied_kib / write_copy}
+    return (fetch * details["fetch_scale"] + write * details["write_scale"]) * 1024.0, details
+
+
 def physical_cores() -> int:
     """Physical cores this process may use: distinct (package, core) pairs of /proc/cpuinfo among the CPUs of the
     affinity mask, capped by OMP_NUM_THREADS (the share of the machine a one-GPU job is given)."""
@@ -333,12 +376,16 @@ def main() -> None:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the attention / block / end-to-end figures")
     ap.add_argument("--workload", choices=["linears", "attention", "block", "block_release", "e2e", "copy", "quantize", "quantize_static"], default="linears")
+    ap.add_argument("--measure-traffic", action="store_true",
+                    help="measure roofline.traffic now (four child runs under rocprofv3 --pmc, about a minute) "
+                         "instead of reading the committed counter summary")
     ap.add_argument("--separate-norm-quantize", action="store_true",
                     help="block / e2e workloads: adaLN or LayerNorm and the quantization behind it as two launches "
                          "(for comparisons; the default is the one-launch kernel where it applies)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives are part of this path); use --gpus 1")
+    live_traffic = live_traffic_bytes() if args.measure_traffic else None  # child processes, before this one uses the GPU
 
     import torch
 
@@ -471,7 +518,11 @@ def main() -> None:
                                "dim 3072, ffn 14336, rule mse, seed 1", "flop_per_step": step_flops(),
                    "prewarm_s": PREWARM_SECONDS},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_F16_TFLOPS, "traffic": measured_traffic_bytes(),
+                     "frac": achieved / PEAK_F16_TFLOPS,
+                     "traffic": live_traffic[0] if live_traffic and live_traffic[0] else measured_traffic_bytes(),
+                     "traffic_source": ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in this run" if live_traffic and live_traffic[0]
+                                        else "profiles/gemm_w4a4_ffn_up_hbm_traffic.txt"
+                                        + (f" (live measurement failed: {live_traffic[1]})" if live_traffic else "")),
                      "kernel": "gemm_w4a4_kernel M=2640 N=14336 K=3072", "avg_ms": gemm_ms,
                      "frac_of_fp8_peak": achieved / PEAK_FP8_TFLOPS,
                      "note": "peak = dense f16 MFMA, the instruction the exact scheme runs on; frac_of_fp8_peak is the "
