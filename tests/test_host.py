@@ -45,6 +45,33 @@ def test_c_abi_rejects_bad_arguments_without_touching_the_gpu():
     assert lib.ll_amax_epoch_advance(None, 1, None, None) == -1 and b"epoch_offset" in lib.ll_last_error()
 
 
+def test_one_launch_entry_points_check_their_arguments_before_touching_the_gpu():
+    """ll_adaln_quantize / ll_layer_norm_quantize / ll_nvfp4_quantize_pair_from_sinks: null pointers, a missing amax
+    sink, and shapes the kernels do not take are answered on the host (LL_EINVAL = -1, LL_ENOSUP = -3)."""
+    import ctypes
+    lib = _native.load()
+    buf = (ctypes.c_uint8 * 4096)()                     # aligned host memory: only its address is looked at
+    ptr = ctypes.addressof(buf) + (-ctypes.addressof(buf)) % 256
+    sink = _native.AmaxSinkStruct(ptr, 1, None)
+    assert lib.ll_adaln_quantize(None, 1, 16, 64, None, None, 0, 0, 0, 0, 16, 1e-6, 1, 3, None, None, None, None, 64, None) == -1
+    assert b"null pointer" in lib.ll_last_error()
+    assert lib.ll_adaln_quantize(ptr, 1, 16, 64, ptr, ptr, 0, 0, 0, 0, 16, 1e-6, 1, 3, ptr, ptr, ptr, None, 64, None) == -1
+    assert b"amax sink" in lib.ll_last_error()
+    assert lib.ll_adaln_quantize(ptr, 1, 16, 64, ptr, ptr, 0, 0, 0, 0, 5, 1e-6, 1, 3, ptr, ptr, ptr, ctypes.byref(sink), 64, None) == -1
+    assert b"bad shape" in lib.ll_last_error()            # L is not a whole number of frames
+    assert lib.ll_adaln_quantize(ptr, 1, 16, 96, ptr, ptr, 0, 0, 0, 0, 16, 1e-6, 1, 3, ptr, ptr, ptr, ctypes.byref(sink), 64, None) == -3
+    assert b"multiple of 64" in lib.ll_last_error()
+    assert lib.ll_layer_norm_quantize(ptr, 16, 4096, None, None, 1e-6, 3, ptr, ptr, ptr, ctypes.byref(sink), 64, None) == -3
+    assert lib.ll_layer_norm_quantize(ptr, 16, 64, None, None, 1e-6, 9, ptr, ptr, ptr, ctypes.byref(sink), 64, None) == -1
+    assert b"scale rule" in lib.ll_last_error()
+    assert lib.ll_nvfp4_quantize_pair_from_sinks(ptr, ptr, 16, 64, 64, 3, ptr, ptr, ptr, ptr, ptr, ptr, ctypes.byref(sink),
+                                                 ctypes.byref(sink), None) == -1
+    assert b"outputs of their own" in lib.ll_last_error()
+    assert lib.ll_nvfp4_quantize_pair_from_sinks(ptr, ptr, 16, 64, 64, 3, ptr, ptr + 256, ptr, ptr + 256, ptr, ptr + 256,
+                                                 None, ctypes.byref(sink), None) == -1
+    assert b"null amax sink" in lib.ll_last_error()
+
+
 def test_noalloc_quantize_refuses_inputs_beyond_its_limit_before_touching_the_gpu():
     lib = _native.load()
     limit = lib.ll_nvfp4_quantize_noalloc_max_elements()
