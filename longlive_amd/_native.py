@@ -18,6 +18,8 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libll_nvfp4.so")
 HEADER_PATH = os.path.join(os.path.dirname(_HERE), "include", "ll_nvfp4.h")
 
 RULE_IDS = {"static_6": 0, "static_4": 1, "mae": 2, "mse": 3, "abs_max": 4}
+# looks (1-2 us each) a workgroup of a launch whose workgroups exchange their maxima waits for the others
+NORM_QUANTIZE_SPIN_LIMIT = 64
 DTYPE_CODES = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 ACTIVATION_IDS = {"gelu_tanh": 1}
 
@@ -720,9 +722,6 @@ def adaln_modulate(x, e_scale, e_shift, frame_seqlen, eps=1e-6, add_one_to_scale
                                              out.data_ptr(), ctypes.byref(sink), _stream())
     _check(code, "ll_adaln_modulate")
     return out
-
-
-NORM_QUANTIZE_SPIN_LIMIT = 64  # looks (1-2 us each) a workgroup of the one-launch normalize-and-quantize kernels waits for the others
 
 
 def _norm_quantize_outputs(M: int, C: int, device):

@@ -11,8 +11,9 @@
 // the grid to what the device holds), each publishes its maximum into its own slot of the caller's amax sink
 // under the launch's epoch, and each waits until all slots carry that epoch.  The wait is bounded: a workgroup that
 // has not seen every slot after `spin_limit` looks computes the maxima of the missing workgroups' rows itself,
-// which gives the same number, so the kernel finishes whatever the other workgroups do.
+// which gives the same number, so the kernel finishes whatever the other workgroups do (amax_exchange.h).
 #include "ll_common.h"
+#include "amax_exchange.h"
 #include "norm_rows.h"
 #include "quantize_block.h"
 
@@ -64,14 +65,10 @@ __device__ __forceinline__ uint32_t from_pair_lane(uint32_t v) {
 template <int RULE, int MODE, int R>
 __global__ __launch_bounds__(kNqThreads) __attribute__((amdgpu_waves_per_eu(R == 1 ? 3 : 2)))
 void norm_quantize_kernel(NormQuantParams p) {
-  __shared__ float s_red[kNqThreads / 64];
-  __shared__ float s_amax;
-  __shared__ int s_alone;
-  __shared__ unsigned long long s_missing[kAmaxParts / 64];
+  __shared__ AmaxExchangeSmem s_exchange;
   __shared__ ScaleEntry s_tab[128];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t G = gridDim.x;
-  const uint32_t epoch = amax_sink_epoch(p.sink.epoch, p.sink.epoch_offset);
 
   // ---- first half: the rows, kept as packed bf16, and their maximum
   uint4 kept[R][kNqChunks];
@@ -86,78 +83,20 @@ void norm_quantize_kernel(NormQuantParams p) {
       for (int i = 0; i < kNqChunks; ++i) kept[r][i] = make_uint4(0u, 0u, 0u, 0u);
     }
   }
-  wave_part = wave_max(wave_part);
-  if (lane == 0) s_red[wave] = wave_part;
-  __syncthreads();
-  if (threadIdx.x == 0)
-    amax_sink_update(p.sink, blockIdx.x, fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3])));
-
-  // ---- the other workgroups' maxima: wave 0 looks at the G slots until all carry this launch's epoch, at most
-  // spin_limit + 1 times; s_missing ends up with one bit per slot that did not
-  if (wave == 0) {
-    bool all_here = false;
-    float m = 0.0f;
-#pragma unroll 1
-    for (uint32_t look = 0;; ++look) {
-      unsigned long long any_missing = 0ull;
-      m = 0.0f;
-      for (uint32_t k = 0; k * 64 < G; ++k) {
-        const uint32_t s = lane + 64 * k;
-        bool here = s >= G;
-        if (s < G && !p.recompute) {
-          const unsigned long long v = __hip_atomic_load(p.sink.parts + s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          here = (uint32_t)(v >> 32) == epoch;
-          if (here) m = fmaxf(m, __uint_as_float((uint32_t)v));
-        }
-        const unsigned long long missing = __builtin_amdgcn_ballot_w64(!here);
-        if (lane == 0) s_missing[k] = missing;
-        any_missing |= missing;
-      }
-      if (any_missing == 0ull) {
-        all_here = true;
-        break;
-      }
-      if (p.recompute || look >= p.spin_limit) break;
-      __builtin_amdgcn_s_sleep(8);
-    }
-    m = wave_max(m);
-    if (lane == 0) {
-      s_amax = m;
-      s_alone = all_here ? 0 : 1;
-    }
-  }
-  __syncthreads();
-  float amax = s_amax;  // the maximum over the workgroups that have arrived
-  if (s_alone) {
-    // Uniform over the workgroup.  Some workgroups have not published (they may not even have started: another
-    // stream can hold compute units for milliseconds): their rows' maxima are computed here, wave w taking the
-    // row their wave w has.  Whatever they publish later is the same number.
+  // ---- the maximum of the whole tensor: exchanged with the other workgroups through the sink; a missing
+  // workgroup's rows are normalized here, wave w taking the row its wave w has
+  const float amax = exchange_amax(p.sink, G, blockIdx.x, wave_part, p.spin_limit, p.recompute != 0, s_exchange, [&](uint32_t s) {
     float part = 0.0f;
 #pragma unroll 1
-    for (uint32_t k = 0; k * 64 < G; ++k) {
-      const unsigned long long word = s_missing[k];
-      uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)word), hi = __builtin_amdgcn_readfirstlane((uint32_t)(word >> 32));
-#pragma unroll 1
-      while ((lo | hi) != 0u) {
-        const uint32_t bit = lo != 0u ? (uint32_t)__builtin_ctz(lo) : 32u + (uint32_t)__builtin_ctz(hi);
-        if (lo != 0u) lo &= lo - 1u; else hi &= hi - 1u;
-        const uint32_t s = 64 * k + bit;
-#pragma unroll 1
-        for (int r = 0; r < R; ++r) {
-          const int64_t row = ((int64_t)r * G + s) * 4 + wave;
-          if (row < p.M) {
-            uint4 unused[kNqChunks];
-            part = fmaxf(part, norm_row<MODE>(p, row, lane, unused));
-          }
-        }
+    for (int r = 0; r < R; ++r) {
+      const int64_t row = ((int64_t)r * G + s) * 4 + wave;
+      if (row < p.M) {
+        uint4 unused[kNqChunks];
+        part = fmaxf(part, norm_row<MODE>(p, row, lane, unused));
       }
     }
-    part = wave_max(part);
-    __syncthreads();  // s_red was read by thread 0 above
-    if (lane == 0) s_red[wave] = part;
-    __syncthreads();
-    amax = fmaxf(amax, fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3])));
-  }
+    return part;
+  });
   if (blockIdx.x == 0 && threadIdx.x == 0) p.amax_out[0] = amax;
 
   // ---- second half: quantize the kept rows (same constants and paths as quantize_kernel)
