@@ -87,7 +87,7 @@ def live_traffic_bytes():
             raise RuntimeError(f"no {name} rows for {workload}")
         return sum(values) / len(values)
 
-    ffn_up = lambda r: "gemm_w4a4_kernel<4, 2>" in r["Kernel_Name"] and r["Grid_Size"] == "315392"
+    ffn_up = lambda r: "gemm_w4a4_asm_kernel<4, 2>" in r["Kernel_Name"] and r["Grid_Size"] == "315392"
     copy = lambda r: "copyBuffer" in r["Kernel_Name"]
     try:
         fetch, write = counter("FETCH_SIZE", "linears", ffn_up), counter("WRITE_SIZE", "linears", ffn_up)
@@ -382,6 +382,8 @@ def main() -> None:
     ap.add_argument("--separate-norm-quantize", action="store_true",
                     help="block / e2e workloads: adaLN or LayerNorm and the quantization behind it as two launches "
                          "(for comparisons; the default is the one-launch kernel where it applies)")
+    ap.add_argument("--gemm-schedule", choices=["auto", "tiles", "tiles_compiled", "persistent"], default="auto",
+                    help="which kernel the GEMM entry points run (for comparisons; the default is the library's choice)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU only (no collectives are part of this path); use --gpus 1")
@@ -399,6 +401,9 @@ def main() -> None:
     if args.separate_norm_quantize:
         from longlive_amd.dit import DiTBlock
         DiTBlock.fuse_norm_quantize = False
+    if args.gemm_schedule != "auto":
+        from longlive_amd import _native
+        _native.gemm_schedule(args.gemm_schedule).__enter__()  # for the whole run
     if args.workload == "copy":
         # plain device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE counters are scaled by
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
@@ -516,14 +521,16 @@ def main() -> None:
         "data": "synthetic",
         "config": {"workload": "configs[1]: 10 W4A4 linears of one Wan2.2-TI2V-5B block, M=2640 (512 for cross k/v), "
                                "dim 3072, ffn 14336, rule mse, seed 1", "flop_per_step": step_flops(),
-                   "prewarm_s": PREWARM_SECONDS},
+                   "prewarm_s": PREWARM_SECONDS, **({} if args.gemm_schedule == "auto" else {"gemm_schedule": args.gemm_schedule})},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / PEAK_F16_TFLOPS,
                      "traffic": live_traffic[0] if live_traffic and live_traffic[0] else measured_traffic_bytes(),
                      "traffic_source": ("rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE in this run" if live_traffic and live_traffic[0]
                                         else "profiles/gemm_w4a4_ffn_up_hbm_traffic.txt"
                                         + (f" (live measurement failed: {live_traffic[1]})" if live_traffic else "")),
-                     "kernel": "gemm_w4a4_kernel M=2640 N=14336 K=3072", "avg_ms": gemm_ms,
+                     "kernel": ("gemm_w4a4_asm_kernel<4, 2>" if args.gemm_schedule in ("auto", "tiles") else
+                                "gemm_w4a4_kernel<4, 2>" if args.gemm_schedule == "tiles_compiled" else
+                                "gemm_w4a4_persistent_kernel") + " M=2640 N=14336 K=3072", "avg_ms": gemm_ms,
                      "frac_of_fp8_peak": achieved / PEAK_FP8_TFLOPS,
                      "note": "peak = dense f16 MFMA, the instruction the exact scheme runs on; frac_of_fp8_peak is the "
                              "same rate against the 5 PFLOP/s dense FP8 figure"},

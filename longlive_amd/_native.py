@@ -492,7 +492,7 @@ def gemm_grouped(a_values, a_scales, amax_a, denom_a: float, M: int, N: int, pro
     return outs
 
 
-GEMM_SCHEDULES = {"auto": -1, "tiles": 0, "persistent": 1}
+GEMM_SCHEDULES = {"auto": -1, "tiles": 0, "persistent": 1, "tiles_compiled": 2}
 
 
 def gemm_plan(M: int, N: int, Kp: int, n_products: int = 1, compute_units: int = 256, schedule: str = "auto") -> dict:
@@ -513,8 +513,9 @@ def gemm_reserve(M: int, N: int, Kp: int, n_products: int = 1, device=None) -> N
 
 class gemm_schedule:
     """``with gemm_schedule("tiles"): ...`` - which kernel the GEMM entry points run ("auto", "tiles": one workgroup
-    per output tile, "persistent": one workgroup per compute unit wherever the shapes allow; process-wide,
-    restored on exit)."""
+    per output tile, its large tiles with the hand-scheduled main loop, "tiles_compiled": the same with the compiled
+    loop everywhere, "persistent": one workgroup per compute unit wherever the shapes allow; process-wide, restored
+    on exit)."""
 
     def __init__(self, name: str):
         if name not in GEMM_SCHEDULES:

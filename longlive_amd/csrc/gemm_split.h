@@ -97,7 +97,7 @@ struct PersistentPlan {
 };
 inline PersistentPlan plan_persistent(int64_t M, int64_t N, int64_t Kp, int n_products, int cus, int schedule) {
   PersistentPlan plan{};
-  if (schedule == 0 /* LL_GEMM_TILES */ || Kp % 128 != 0 || cus < 1) return plan;
+  if (schedule == 0 /* LL_GEMM_TILES */ || schedule == 2 /* LL_GEMM_TILES_COMPILED */ || Kp % 128 != 0 || cus < 1) return plan;
   const int64_t tiles_m = (M + kPTileM - 1) / kPTileM, tiles_n_each = (N + kPTileN - 1) / kPTileN;
   const int64_t tiles = tiles_m * tiles_n_each * n_products, nk = Kp / 128;
   if (tiles >= (1ll << 30) || tiles * nk < cus) return plan;

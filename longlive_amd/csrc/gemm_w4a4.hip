@@ -726,6 +726,163 @@ __global__ __launch_bounds__(256) void gemm_w4a4_persistent_kernel(PersistentPar
 #undef LL_V10
 
 
+// ============================================================================ tile kernel, hand-scheduled loop
+// gemm_w4a4_kernel<FA, FB> with its main loop replaced by a generated instruction sequence
+// (gemm_tile_loop_gen.py): the same workgroup -> tile map, the same arithmetic in the same order (the accumulators
+// receive the same MFMAs in the same sequence, so the results are bit-identical), the same epilogue.  Needs Kp to be a
+// multiple of 128.  Tiles 256 x 128 and 128 x 256: the 128 x 128 tile, with 8 decode instructions per MFMA against 6, is
+// bound by the issue of those whatever their order (measured: 53.5 us against the compiler's 52.6 on 2640 x 3072 x 3072).
+template <int FA, int FB>
+struct AsmTile {
+  static constexpr int BM = 64 * FA, BN = 64 * FB;
+  static constexpr int kAScales = (BM + BN) * 64;                      // LDS offsets inside a stage, as in the generator
+  static constexpr int kBScales = kAScales + 1024 * (BM / 128);
+  static constexpr int kStage = kBScales + 1024 * (BN / 128);
+  static constexpr int kScaleBlocks = BM / 128 + BN / 128;
+};
+
+#define LL_V10(a) "v" #a "0", "v" #a "1", "v" #a "2", "v" #a "3", "v" #a "4", "v" #a "5", "v" #a "6", "v" #a "7", "v" #a "8", "v" #a "9"
+#define LL_ASM_TILE_INPUTS                                                                                              \
+  "s"(nsteps), "v"(lane_voff), "v"(lane_soff), "v"(ard), "v"(brd), "v"(sard), "v"(sbrd), "v"(sh), "s"(sA), "s"(sB), "s"(sS),    \
+      "s"(rb16), "s"(adst), "s"(bdst), "s"(sdst), "s"(idle)
+#define LL_ASM_TILE_SGPRS                                                                                               \
+  "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73",  \
+      "s74", "s75", "s76", "s77", "s78", "s79", "s80", "s81", "s82", "s83", "s84", "s85", "s86", "s87"
+
+template <int FA, int FB>
+__global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_asm_kernel(
+    const uint8_t* __restrict__ Av, const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bv0,
+    const uint8_t* __restrict__ Bs0, const float* __restrict__ alpha_ptr0, const float* __restrict__ amax_a,
+    const float* __restrict__ amax_b0, float inv_denom_a, float inv_denom_b0, int M, int N, int Mp, int Np, int Kp,
+    uint16_t* __restrict__ D0, int64_t ldd0, int tiles_m, int tiles_n, GemmEpilogue epi, GemmGroups groups) {
+  using T = AsmTile<FA, FB>;
+  constexpr int BM = T::BM, BN = T::BN;
+  const uint8_t* __restrict__ Bv = Bv0;
+  const uint8_t* __restrict__ Bs = Bs0;
+  const float* __restrict__ alpha_ptr = alpha_ptr0;
+  const float* __restrict__ amax_b = amax_b0;
+  float inv_denom_b = inv_denom_b0;
+  uint16_t* __restrict__ D = D0;
+  int64_t ldd = ldd0;
+  const uint16_t* __restrict__ bias = epi.bias;
+  const int act = epi.act;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  // Workgroup -> tile, as in gemm_w4a4_kernel.
+  int wg = blockIdx.x;
+  {
+    const int total = tiles_m * tiles_n;
+    const int per_xcd = (total + 7) / 8;
+    const int xcd = wg & 7, idx = wg >> 3;
+    const int remapped = xcd * per_xcd + idx;
+    if (total % 8 == 0) wg = remapped;
+  }
+  int tile_n = wg / tiles_m, tile_m = wg - tile_n * tiles_m;
+  {
+    constexpr int kBandRows = 8;
+    const int total = tiles_m * tiles_n, per_xcd = total / 8;
+    const int panels = per_xcd / tiles_m;
+    if (total % 8 == 0 && panels * tiles_m == per_xcd) {
+      const int xcd = wg / per_xcd, idx = wg - xcd * per_xcd;
+      const int band = min(idx / (kBandRows * panels), tiles_m / kBandRows);
+      const int rows_in_band = min(kBandRows, tiles_m - band * kBandRows);
+      const int in_band = idx - band * kBandRows * panels;
+      const int c = in_band / rows_in_band;
+      tile_m = band * kBandRows + (in_band - c * rows_in_band);
+      tile_n = xcd * panels + c;
+    }
+  }
+  if (groups.n > 1) {
+    const int g = tile_n / groups.tiles_n_each;
+    tile_n -= g * groups.tiles_n_each;
+    if (g > 0) {
+      const GemmGroup& gg = groups.more[g - 1];
+      Bv = gg.Bv;
+      Bs = gg.Bs;
+      alpha_ptr = gg.alpha;
+      amax_b = gg.amax_b;
+      inv_denom_b = gg.inv_denom_b;
+      D = gg.D;
+      ldd = gg.ldd;
+      bias = gg.bias;
+      epi.sink = gg.sink;
+    }
+  }
+  const int row0 = tile_m * BM, col0 = tile_n * BN;
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave & 1, wn = wave >> 1;
+
+  // What the loop needs from here (gemm_tile_loop_gen.py): the wave's quarter of the A and B rows of the tile to load
+  // (rows beyond the padded matrix are replaced by the last rows: their outputs are masked), its scale block, the
+  // lane's offsets in a load of 16 rows, its read addresses in LDS, the shift that picks its pair of scale bytes.
+  const uint32_t row_bytes = (uint32_t)Kp >> 1;
+  const uint32_t swz = (l32 >> 2) & 3;
+  const uint32_t lane_voff = (uint32_t)(lane >> 2) * row_bytes + 16u * ((lane & 3) ^ ((lane >> 4) & 3));
+  const uint32_t lane_soff = (uint32_t)lane * 16u;
+  const uint32_t lane_rd = (uint32_t)l32 * 64u + 16u * ((lh ^ (swz & 1)) | (swz & 2));
+  const uint32_t ard = (uint32_t)(32 * FA * wm) * 64u + lane_rd;
+  const uint32_t brd = (uint32_t)(BM * 64) + (uint32_t)(32 * FB * wn) * 64u + lane_rd;
+  // a wave with four fragments of an operand owns a whole 128-row group of its scales, one with two owns half of one
+  const uint32_t sard = T::kAScales + (uint32_t)l32 * 16u + (FA == 4 ? 1024u : 8u) * wm;
+  const uint32_t sbrd = T::kBScales + (uint32_t)l32 * 16u + (FB == 4 ? 1024u : 8u) * wn;
+  const uint32_t sh = 16u * lh;
+  const int a_rows = min(row0 + (BM / 4) * wave, Mp - BM / 4), b_rows = min(col0 + (BN / 4) * wave, Np - BN / 4);
+  const uint8_t* sA = Av + (size_t)a_rows * row_bytes;
+  const uint8_t* sB = Bv + (size_t)b_rows * row_bytes;
+  // scale blocks of a K step (1 KB per 128 rows): those of A, then those of B; wave w loads block w (the last waves
+  // the last block again)
+  const int block = min(wave, T::kScaleBlocks - 1);
+  const uint8_t* sS = block < BM / 128 ? As + (size_t)min((row0 >> 7) + block, (Mp >> 7) - 1) * (size_t)(Kp >> 6) * 512
+                                       : Bs + (size_t)min((col0 >> 7) + block - BM / 128, (Np >> 7) - 1) * (size_t)(Kp >> 6) * 512;
+  const uint32_t adst = (uint32_t)wave * (BM / 4) * 64u, bdst = (uint32_t)(BM * 64) + (uint32_t)wave * (BN / 4) * 64u;
+  const uint32_t sdst = T::kAScales + 1024u * (uint32_t)block;
+  const uint32_t nsteps = (uint32_t)Kp >> 7, rb16 = 16u * row_bytes;
+  // A wave whose rows (or columns) all lie beyond M (N) only helps with the staging.
+  const uint32_t idle = __builtin_amdgcn_readfirstlane(row0 + wm * 32 * FA < M && col0 + wn * 32 * FB < N ? 0 : 1);
+
+  float16v acc[FB][FA];
+#pragma unroll
+  for (int g = 0; g < FB; ++g)
+#pragma unroll
+    for (int f = 0; f < FA; ++f)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[g][f][i] = 0.0f;
+  if constexpr (FA == 4 && FB == 2) {
+    asm volatile(
+#include "gemm_tile_loop_42_gfx950.inc"
+        : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[0][2]), "+a"(acc[0][3]), "+a"(acc[1][0]), "+a"(acc[1][1]), "+a"(acc[1][2]),
+          "+a"(acc[1][3])
+        : LL_ASM_TILE_INPUTS
+        : "memory", "scc", "vcc", "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", LL_V10(1), LL_V10(2), LL_V10(3),
+          LL_V10(4), LL_V10(5), LL_V10(6), LL_V10(7), LL_V10(8), LL_V10(9), "v100", "v101", LL_ASM_TILE_SGPRS);
+  } else {
+    static_assert(FA == 2 && FB == 4, "generated loops exist for the 256 x 128 and the 128 x 256 tile");
+    asm volatile(
+#include "gemm_tile_loop_24_gfx950.inc"
+        : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[1][0]), "+a"(acc[1][1]), "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[3][0]),
+          "+a"(acc[3][1])
+        : LL_ASM_TILE_INPUTS
+        : "memory", "scc", "vcc", "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", LL_V10(1), LL_V10(2), LL_V10(3),
+          LL_V10(4), LL_V10(5), LL_V10(6), LL_V10(7), LL_V10(8), LL_V10(9), "v100", "v101", LL_ASM_TILE_SGPRS);
+  }
+  __syncthreads();  // every wave has left the stages: the epilogue reuses them
+
+  float alpha;
+  if (alpha_ptr) {
+    alpha = alpha_ptr[0];
+  } else {
+    alpha = (amax_a[0] * amax_b[0]) * (inv_denom_a * inv_denom_b);
+  }
+  gemm_epilogue<FA, FB>(acc, alpha, smem, wave, lane, row0 + wm * 32 * FA, col0 + wn * 32 * FB, M, N, D, ldd, bias, act, epi,
+                        (uint32_t)blockIdx.x * 4 + wave);
+}
+#undef LL_ASM_TILE_SGPRS
+#undef LL_ASM_TILE_INPUTS
+#undef LL_V10
+
+static std::atomic<int> g_gemm_schedule{LL_GEMM_AUTO};
+
 template <int FA, int FB>
 int launch_gemm(const uint8_t* Av, const uint8_t* As, const uint8_t* Bv, const uint8_t* Bs, const float* alpha,
                 const float* amax_a, const float* amax_b, float denom_a, float denom_b, int M, int N, int Mp, int Np,
@@ -733,6 +890,21 @@ int launch_gemm(const uint8_t* Av, const uint8_t* As, const uint8_t* Bv, const u
   using S = GemmSmem<FA, FB>;
   groups.tiles_n_each = (N + S::BN - 1) / S::BN;
   const int tiles_m = (M + S::BM - 1) / S::BM, tiles_n = groups.tiles_n_each * groups.n;
+  if constexpr (FA + FB == 6) {
+    if (Kp % 128 == 0 && g_gemm_schedule.load(std::memory_order_relaxed) != LL_GEMM_TILES_COMPILED) {
+      // the same kernel with its main loop as a hand-scheduled instruction sequence
+      using T = AsmTile<FA, FB>;
+      static_assert(2 * T::kStage >= 4 * 32 * (64 * FB + 16), "the epilogue's patches fit the stages");
+      const size_t smem = 2 * T::kStage;
+      static std::atomic<uint64_t> lds_allowed{0};
+      if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_w4a4_asm_kernel<FA, FB>), smem, lds_allowed, "ll_nvfp4_gemm_tnt")) return rc;
+      hipLaunchKernelGGL((gemm_w4a4_asm_kernel<FA, FB>), dim3((unsigned)(tiles_m * tiles_n)), dim3(kGemmThreads), smem, stream, Av,
+                         As, Bv, Bs, alpha, amax_a, amax_b, 1.0f / denom_a, 1.0f / denom_b, M, N, Mp, Np, Kp,
+                         static_cast<uint16_t*>(D), ldd, tiles_m, tiles_n, epi, groups);
+      LL_CHECK_LAUNCH("gemm_w4a4_asm_kernel");
+      return LL_OK;
+    }
+  }
   const size_t smem = 2 * S::kStage;
   static std::atomic<uint64_t> lds_allowed{0};  // one per tile configuration
   if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_w4a4_kernel<FA, FB>), smem, lds_allowed, "ll_nvfp4_gemm_tnt")) return rc;
@@ -823,7 +995,6 @@ extern "C" int ll_nvfp4_gemm_tnt_fused(const uint8_t* A_values, const uint8_t* A
 }
 
 namespace ll {
-static std::atomic<int> g_gemm_schedule{LL_GEMM_AUTO};
 
 inline size_t persistent_record_bytes(const GemmDivision& d) { return (size_t)2 * d.G * kPRecordFloats * sizeof(float); }
 
@@ -834,7 +1005,7 @@ static int try_persistent(const uint8_t* A_values, const uint8_t* A_scales, cons
                           const GemmGroups& groups, hipStream_t stream, bool* launched) {
   *launched = false;
   const int schedule = g_gemm_schedule.load(std::memory_order_relaxed);
-  if (schedule == LL_GEMM_TILES || Kp % 128 != 0) return LL_OK;
+  if (schedule == LL_GEMM_TILES || schedule == LL_GEMM_TILES_COMPILED || Kp % 128 != 0) return LL_OK;
   int dev = 0, cus = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     set_error("ll_nvfp4_gemm_tnt: hipGetDevice failed");
@@ -972,7 +1143,7 @@ extern "C" int ll_nvfp4_gemm_tnt_grouped(const uint8_t* A_values, const uint8_t*
 }
 
 extern "C" int ll_nvfp4_gemm_set_schedule(int schedule) {
-  LL_REQUIRE(schedule >= LL_GEMM_AUTO && schedule <= LL_GEMM_PERSISTENT, "ll_nvfp4_gemm_set_schedule: unknown schedule %d", schedule);
+  LL_REQUIRE(schedule >= LL_GEMM_AUTO && schedule <= LL_GEMM_TILES_COMPILED, "ll_nvfp4_gemm_set_schedule: unknown schedule %d", schedule);
   ll::g_gemm_schedule.store(schedule);
   return LL_OK;
 }

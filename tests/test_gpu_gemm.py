@@ -548,3 +548,42 @@ def test_persistent_schedule_on_a_capturing_stream(gpu):
             fp4_matmul(xq, wq)
         with torch.cuda.stream(side2):
             _native.release_stream_memory()
+
+
+@pytest.mark.parametrize("M,N,K,groups", [
+    (2640, 14336, 3072, 1),   # 256 x 128 tiles: FFN-up
+    (2688, 4096, 128, 1),     # one K step
+    (513, 14336, 256, 1),     # ragged M, two steps
+    (2640, 3072, 3072, 1),    # 128 x 128 tiles: the projections
+    (2600, 14300, 1152, 1),   # 256 x 128 tiles, ragged M and N, an odd number of steps
+    (12763, 379, 384, 1),     # 128 x 256 tiles, ragged M and N
+    (2640, 3072, 3072, 3),    # 128 x 256 tiles: q, k, v in one launch
+    (300, 1100, 1152, 2),     # two products, ragged
+])
+def test_hand_scheduled_main_loop_is_bit_identical_to_the_compiled_one(gpu, M, N, K, groups):
+    """The one-workgroup-per-tile kernels with tiles of 256 x 128 and 128 x 256 run their main loop as a generated
+    instruction sequence wherever K is a multiple of 128; every accumulator receives the same products in the same
+    order as in the compiler's loop, so outputs and the amax left in the sinks are equal bit for bit.  (The shapes
+    that take 128 x 128 tiles run the compiler's loop under either setting.)"""
+    cfg = QuantizationConfig(scale_rule="mse")
+    xq = quantize_to_fp4(activations((M, K), 5).to(gpu), cfg)
+    ws = [quantize_to_fp4((weights((N, K), 6 + i) * (1 + i)).to(gpu), cfg) for i in range(groups)]
+    bias = (torch.randn(N, generator=torch.Generator().manual_seed(7)) * 0.1).to(gpu).bfloat16()
+    out = {}
+    for sched in ("tiles_compiled", "tiles"):
+        with _native.gemm_schedule(sched):
+            if groups == 1:
+                t = _native.amax_ticket(gpu)
+                y = [fp4_matmul(xq, ws[0], bias=bias, activation="gelu_tanh", amax_out=t)]
+                amax = [float(quantize_to_fp4(y[0], cfg, amax=t).amax)]
+            else:
+                sinks = [_native.PrivateAmaxSink(gpu) for _ in range(groups)]
+                products = [dict(values=w.values, scales=w.scale_factors, amax=w.amax, denom=1536.0, bias=bias if i != 1 else None,
+                                 amax_out=s.ticket()) for i, (w, s) in enumerate(zip(ws, sinks))]
+                y = _native.gemm_grouped(xq.values, xq.scale_factors, xq.amax, 1536.0, M, N, products)
+                amax = [float(quantize_to_fp4(yi, cfg, amax=pr["amax_out"]).amax) for yi, pr in zip(y, products)]
+        out[sched] = (y, amax)
+    for got, want in zip(out["tiles"][0], out["tiles_compiled"][0]):
+        assert torch.equal(got, want)
+    assert out["tiles"][1] == out["tiles_compiled"][1]
+    assert out["tiles"][1] == [float(yi.float().abs().max()) for yi in out["tiles"][0]]
