@@ -29,7 +29,7 @@ import sys
 
 
 class Plan:
-    def __init__(self, fa, fb):
+    def __init__(self, fa, fb, waves=4):
         self.fa, self.fb, self.nf = fa, fb, fa + fb
         nf = self.nf
         self.a_bytes = 64 * fa * 64                      # A tile of a stage
@@ -48,8 +48,8 @@ class Plan:
         self.n_vgprs = self.addr0 + 9
         # loads of a wave per K step: its quarter of the A tile and of the B tile (16 rows = 1 KB per load) and one
         # 1 KB scale block
-        self.a_loads = (64 * fa) // 16 // 4
-        self.b_loads = (64 * fb) // 16 // 4
+        self.a_loads = (64 * fa) // 16 // waves
+        self.b_loads = (64 * fb) // 16 // waves
 
     # ---- registers
     def O(self, b, frag, q=None):
@@ -297,16 +297,213 @@ def gen(fa, fb):
     return P, out
 
 
-def main(fa, fb, path):
-    P, lines = gen(fa, fb)
+# ---------------------------------------------------------------------------------------------------------------------
+# Eight waves per workgroup, the K range of every step split between two groups of four (gemm_w4a4_asm8_kernel).
+#
+# One workgroup per compute unit computes a (64 FA) x (64 FB) tile; waves 0-3 and 4-7 hold the same 2 x 2 arrangement of
+# wave tiles, the first group multiplies the first 64 K elements of every K step, the second group the other 64, and
+# the kernel adds the two partial tiles through LDS behind the loop.  A wave therefore walks four sub-steps per K
+# step (dwords 0-3 of ONE 16-byte piece per lane and fragment; which piece, and which half of the scales, is in the
+# addresses the kernel passes).  The stages form a ring of NSTAGE: their offset is kept in registers, not in the
+# instructions, so the loop is not unrolled.  The barrier of step t sits behind sub-step 1, when the wave has issued
+# its last read of stage t and has waited for its loads of step t + 1; behind it the wave requests step t + NSTAGE
+# into the stage it just left and reads the first dwords and the scales of step t + 1.
+SPLIT_INPUTS = ["N", "VOFF", "SOFF", "ARD", "BRD", "SARD", "SBRD", "SH", "SA", "SB", "SS", "RB16", "ADST", "BDST", "SDST", "IDLE",
+                "HASSC"]
+# HASSC: not zero for the waves that load a block of scales (one more load per K step than the others).
+
+
+def gen_split(fa, fb, nstage=3):
+    P = Plan(fa, fb, waves=8)
+    nacc, n_mfma = fa * fb, fa * fb
+    OP = {name: "%%%d" % (nacc + i) for i, name in enumerate(SPLIT_INPUTS)}
+    A_RD, B_RD, SA_RD, SB_RD, SH, VOFF, SOFF = (P.addr(i) for i in range(7))
+    S_A = ["s[%d:%d]" % (58 + 2 * i, 59 + 2 * i) for i in range(P.a_loads)]
+    S_B = ["s[%d:%d]" % (58 + 2 * (P.a_loads + i), 59 + 2 * (P.a_loads + i)) for i in range(P.b_loads)]
+    assert 58 + 2 * (P.a_loads + P.b_loads) <= 76
+    S_RS, S_WS, S_DELTA, S_TMP, S_HASSC = "s76", "s77", "s78", "s79", "s85"
+    ring = nstage * P.stage
+    labels = iter(range(10, 100))
+
+    def mfma(j, g, f):
+        acc = "%%%d" % (fa * g + f)
+        return "v_mfma_f32_32x32x16_f16 %s, %s, %s, %s" % (acc, P.O(j & 1, fa + g), P.O(j & 1, f), acc)
+
+    def decode(j, frag):
+        """Eight instructions: dword j of the lane's piece of fragment `frag`, scaled, into operand buffer j % 2."""
+        out = []
+        for q in range(4):
+            sel = " op_sel:[%d,%d,0]" % (q & 1, q >> 1) if q else ""
+            out.append("v_cvt_scalef32_pk_f16_fp4 %s, %s, 1.0%s" % (P.T, P.R(j >> 1, frag, j & 1), sel))
+            if j < 2:   # the piece's first 16 elements: low half of the pair of block scales
+                out.append("v_pk_mul_f16 %s, %s, %s op_sel_hi:[0,1]" % (P.O(j & 1, frag, q), P.S(0, frag), P.T))
+            else:
+                out.append("v_pk_mul_f16 %s, %s, %s op_sel:[1,0] op_sel_hi:[1,1]" % (P.O(j & 1, frag, q), P.S(0, frag), P.T))
+        return out
+
+    order = [0, fa] + list(range(1, fa)) + list(range(fa + 1, fa + fb))
+
+    def decode_all(j):
+        return [i for frag in order for i in decode(j, frag)]
+
+    def quarter_reads(quarter):
+        """Dwords 2 quarter, 2 quarter + 1 of the lane's pieces in the stage the address registers point at."""
+        out = ["ds_read_b64 %s, %s offset:%d" % (P.R(quarter, f), A_RD, 8 * quarter + 2048 * f) for f in range(fa)]
+        out += ["ds_read_b64 %s, %s offset:%d" % (P.R(quarter, fa + g), B_RD, 8 * quarter + 2048 * g) for g in range(fb)]
+        return out
+
+    def scale_reads():
+        def read(x, n, addr):
+            base = P.sr0 + 4 * x
+            return ("ds_read_b128 %s, %s" % (P.SR(x), addr)) if n == 4 else ("ds_read_b64 v[%d:%d], %s" % (base, base + 1, addr))
+        return [read(0, fa, SA_RD), read(1, fb, SB_RD)]
+
+    def scale_conversion():
+        out = []
+        for f in range(fa):
+            out += ["v_lshrrev_b32 %s, %s, %s" % (P.T, SH, P.SR(0, f)), "v_cvt_scalef32_pk_f16_fp8 %s, %s, 1.0" % (P.S(0, f), P.T)]
+        for g in range(fb):
+            out += ["v_lshrrev_b32 %s, %s, %s" % (P.T, SH, P.SR(1, g)), "v_cvt_scalef32_pk_f16_fp8 %s, %s, 1.0" % (P.S(0, fa + g), P.T)]
+        return out
+
+    def request():
+        """The wave's loads of one K step into the stage at S_WS, then the offsets of the next step."""
+        out = []
+        for i in range(P.a_loads):
+            out += ["s_add_u32 m0, %s, %s" % (S_ADST, S_WS)] + (["s_add_u32 m0, m0, %d" % (1024 * i)] if i else []) + \
+                   ["s_nop 0", "global_load_lds_dwordx4 %s, %s" % (VOFF, S_A[i])]
+        for i in range(P.b_loads):
+            out += ["s_add_u32 m0, %s, %s" % (S_BDST, S_WS)] + (["s_add_u32 m0, m0, %d" % (1024 * i)] if i else []) + \
+                   ["s_nop 0", "global_load_lds_dwordx4 %s, %s" % (VOFF, S_B[i])]
+        skip = next(labels)
+        out += ["s_cmp_eq_u32 %s, 0" % S_HASSC, "s_cbranch_scc1 %df" % skip,
+                "s_add_u32 m0, %s, %s" % (S_SDST, S_WS), "s_nop 0", "global_load_lds_dwordx4 %s, %s" % (SOFF, S_SC), "%d:" % skip]
+        out += ["s_sub_u32 %s, %s, 1" % (S_LEFT, S_LEFT), "v_add_u32 %s, 64, %s" % (VOFF, VOFF), "v_add_u32 %s, 0x400, %s" % (SOFF, SOFF)]
+        return out
+
+    def request_if_left():
+        skip = next(labels)
+        return ["s_cmp_eq_u32 %s, 0" % S_LEFT, "s_cbranch_scc1 %df" % skip] + request() + ["%d:" % skip]
+
+    def rotate(with_addresses):
+        """The stage just read becomes the one to refill; the address registers move on to the next stage."""
+        out = ["s_mov_b32 %s, %s" % (S_WS, S_RS),
+               "s_add_u32 %s, %s, %d" % (S_TMP, S_RS, P.stage),
+               "s_cmp_eq_u32 %s, %d" % (S_TMP, ring),
+               "s_cselect_b32 %s, 0, %s" % (S_TMP, S_TMP),
+               "s_sub_u32 %s, %s, %s" % (S_DELTA, S_TMP, S_RS),
+               "s_mov_b32 %s, %s" % (S_RS, S_TMP)]
+        if with_addresses:
+            out += ["v_add_u32 %s, %s, %s" % (r, S_DELTA, r) for r in (A_RD, B_RD, SA_RD, SB_RD)]
+        return out
+
+    def wait_and_barrier():
+        """The wave's loads of step t + 1 have landed (those of step t + 2, if it exists, may still be under way)."""
+        l0, l4, lb = next(labels), next(labels), next(labels)
+        per_wave = P.a_loads + P.b_loads
+        return ["s_cmp_le_u32 %s, 2" % S_N, "s_cbranch_scc1 %df" % l0,
+                "s_cmp_lg_u32 %s, 0" % S_HASSC, "s_cbranch_scc1 %df" % l4,
+                "s_waitcnt vmcnt(%d)" % per_wave, "s_branch %df" % lb,
+                "%d:" % l4, "s_waitcnt vmcnt(%d)" % (per_wave + 1), "s_branch %df" % lb,
+                "%d:" % l0, "s_waitcnt vmcnt(0)",
+                "%d:" % lb, "s_barrier"]
+
+    def k_step():
+        out = []
+        for j in range(4):
+            fill = decode_all((j + 1) & 3)
+            per = len(fill) // n_mfma
+            assert per * n_mfma == len(fill)
+            extra = {m: [] for m in range(n_mfma)}
+            head = []
+            if j == 0:      # dwords 2, 3: the last reads of this stage
+                for i, ins in enumerate(quarter_reads(1)):
+                    extra[i % n_mfma].append(ins)
+            elif j == 1:
+                head.append("s_waitcnt lgkmcnt(0)")
+                extra[0] += rotate(True)
+                extra[n_mfma - 1] += wait_and_barrier()
+            elif j == 2:    # refill the stage just left; first dwords and scales of the next step
+                extra[0] += request_if_left()
+                for i, ins in enumerate(quarter_reads(0) + scale_reads()):
+                    extra[1 + i % (n_mfma - 1)].append(ins)
+            else:
+                head.append("s_waitcnt lgkmcnt(0)")
+                head += scale_conversion()
+            out += head
+            for m in range(n_mfma):
+                out.append(mfma(j, m // fa, m % fa))
+                out += fill[per * m:per * (m + 1)]
+                out += extra[m]
+        return out
+
+    def prologue():
+        out = ["s_mov_b32 %s, %s" % (S_N, OP["N"]),
+               "s_mov_b32 %s, %s" % (S_LEFT, OP["N"]),
+               "s_mov_b32 %s, %s" % (S_HASSC, OP["HASSC"]),
+               "s_mov_b32 %s, 0" % S_RS,
+               "s_mov_b32 %s, 0" % S_WS,
+               "v_mov_b32 %s, %s" % (VOFF, OP["VOFF"]),
+               "v_mov_b32 %s, %s" % (SOFF, OP["SOFF"]),
+               "v_mov_b32 %s, %s" % (A_RD, OP["ARD"]),
+               "v_mov_b32 %s, %s" % (B_RD, OP["BRD"]),
+               "v_mov_b32 %s, %s" % (SA_RD, OP["SARD"]),
+               "v_mov_b32 %s, %s" % (SB_RD, OP["SBRD"]),
+               "v_mov_b32 %s, %s" % (SH, OP["SH"]),
+               "s_mov_b32 %s, %s" % (S_ADST, OP["ADST"]),
+               "s_mov_b32 %s, %s" % (S_BDST, OP["BDST"]),
+               "s_mov_b32 %s, %s" % (S_SDST, OP["SDST"]),
+               "s_mov_b64 %s, %s" % (S_A[0], OP["SA"])]
+        regs = [58 + 2 * i for i in range(P.a_loads + P.b_loads)]
+        for i in range(1, P.a_loads):
+            out += ["s_add_u32 s%d, s%d, %s" % (regs[i], regs[i - 1], OP["RB16"]), "s_addc_u32 s%d, s%d, 0" % (regs[i] + 1, regs[i - 1] + 1)]
+        out.append("s_mov_b64 %s, %s" % (S_B[0], OP["SB"]))
+        for i in range(P.a_loads + 1, P.a_loads + P.b_loads):
+            out += ["s_add_u32 s%d, s%d, %s" % (regs[i], regs[i - 1], OP["RB16"]), "s_addc_u32 s%d, s%d, 0" % (regs[i] + 1, regs[i - 1] + 1)]
+        out += ["s_mov_b64 %s, %s" % (S_SC, OP["SS"]), "s_nop 4"]
+        out += request()
+        for stage in range(1, nstage):
+            out.append("s_mov_b32 %s, %d" % (S_WS, stage * P.stage))
+            out += request_if_left()
+        out += ["s_waitcnt vmcnt(0)", "s_barrier", "s_cmp_lg_u32 %s, 0" % OP["IDLE"], "s_cbranch_scc1 3f"]
+        out += quarter_reads(0) + scale_reads()
+        out.append("s_waitcnt lgkmcnt(0)")
+        out += scale_conversion()
+        out += decode_all(0)
+        out.append("s_nop 1")
+        return out
+
+    out = prologue()
+    out.append("1:")
+    out += k_step()
+    out += ["s_sub_u32 %s, %s, 1" % (S_N, S_N), "s_cmp_lg_u32 %s, 0" % S_N, "s_cbranch_scc1 1b"]
+    out.append("2:")
+    out += ["s_nop 7", "s_nop 7", "s_nop 7", "s_waitcnt vmcnt(0) lgkmcnt(0)", "s_branch 4f"]
+    out.append("3:")    # a wave without outputs: the barrier, the rotation, its loads
+    out += wait_and_barrier() + rotate(False) + request_if_left()
+    out += ["s_sub_u32 %s, %s, 1" % (S_N, S_N), "s_cmp_lg_u32 %s, 0" % S_N, "s_cbranch_scc1 3b", "s_branch 2b"]
+    out.append("4:")
+    return P, out
+
+
+def main(fa, fb, path, waves=4):
+    P, lines = gen(fa, fb) if waves == 4 else gen_split(fa, fb)
+    inputs = INPUTS if waves == 4 else SPLIT_INPUTS
     with open(path, "w") as f:
-        f.write("// Generated by gemm_tile_loop_gen.py %d %d - do not edit.  %d instructions, VGPRs v0-v%d, LDS stage %d bytes;\n"
+        f.write("// Generated by gemm_tile_loop_gen.py %d %d%s - do not edit.  %d instructions, VGPRs v0-v%d, LDS stage %d bytes;\n"
                 "// operands: %%0-%%%d accumulators, then %s.\n"
-                % (fa, fb, sum(1 for l in lines if not l.endswith(":")), P.n_vgprs - 1, P.stage, fa * fb - 1, ", ".join(INPUTS)))
+                % (fa, fb, "" if waves == 4 else " --waves 8", sum(1 for l in lines if not l.endswith(":")), P.n_vgprs - 1, P.stage,
+                   fa * fb - 1, ", ".join(inputs)))
         for l in lines:
             f.write('"%s\\n"\n' % l)
 
 
 if __name__ == "__main__":
-    fa, fb = int(sys.argv[1]), int(sys.argv[2])
-    main(fa, fb, sys.argv[3] if len(sys.argv) > 3 else "gemm_tile_loop_%d%d_gfx950.inc" % (fa, fb))
+    # usage: gemm_tile_loop_gen.py FA FB out.inc [--waves 8]
+    args = sys.argv[1:]
+    waves = 4
+    if "--waves" in args:
+        i = args.index("--waves")
+        waves = int(args[i + 1])
+        del args[i:i + 2]
+    main(int(args[0]), int(args[1]), args[2], waves)

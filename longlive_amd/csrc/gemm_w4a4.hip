@@ -877,6 +877,150 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_asm_kernel(
   gemm_epilogue<FA, FB>(acc, alpha, smem, wave, lane, row0 + wm * 32 * FA, col0 + wn * 32 * FB, M, N, D, ldd, bias, act, epi,
                         (uint32_t)blockIdx.x * 4 + wave);
 }
+// ============================================================================ one workgroup per compute unit, K split inside it
+// A 128 x 256 tile by eight waves: waves 0-3 and 4-7 hold the same 2 x 2 arrangement of 64 x 128 wave tiles; of every K
+// step of 128 the first group multiplies the first 64 elements, the second group the other 64 (generated loop,
+// gemm_tile_loop_gen.py --waves 8: three LDS stages in a ring, the loads of a step shared by all eight waves).  Behind
+// the loop the partners exchange half of their partial tiles through LDS - wave w keeps its first 32 rows and
+// receives the partner's, wave w + 4 the other 32 - and every wave runs the epilogue on the 32 x 128 sums it holds.
+// fp32 addition is commutative, so the result does not depend on which side adds; it differs from the kernels above
+// by the order of the fp32 additions only (two halves of K summed separately).  For shapes that give at most one
+// 128 x 256 tile per compute unit: two waves per SIMD with 6 decode instructions per MFMA, where 128 x 128 tiles in
+// pairs need 8.  Kp is a multiple of 128.
+constexpr int kSplitThreads = 512;
+constexpr int kSplitStages = 3;
+constexpr int kSplitSmem = 8 * 64 * 64 * 4;  // the exchange: 64 accumulator registers of 8 waves; the ring needs less
+
+__global__ __launch_bounds__(kSplitThreads) void gemm_w4a4_asm8_kernel(
+    const uint8_t* __restrict__ Av, const uint8_t* __restrict__ As, const uint8_t* __restrict__ Bv0,
+    const uint8_t* __restrict__ Bs0, const float* __restrict__ alpha_ptr0, const float* __restrict__ amax_a,
+    const float* __restrict__ amax_b0, float inv_denom_a, float inv_denom_b0, int M, int N, int Mp, int Np, int Kp,
+    uint16_t* __restrict__ D0, int64_t ldd0, int tiles_m, int tiles_n, GemmEpilogue epi, GemmGroups groups) {
+  constexpr int FA = 2, FB = 4;
+  using T = AsmTile<FA, FB>;
+  constexpr int BM = T::BM, BN = T::BN;
+  static_assert(kSplitStages * T::kStage <= kSplitSmem && 8 * 32 * (64 * FB + 16) <= kSplitSmem, "ring and epilogue patches fit");
+  const uint8_t* __restrict__ Bv = Bv0;
+  const uint8_t* __restrict__ Bs = Bs0;
+  const float* __restrict__ alpha_ptr = alpha_ptr0;
+  const float* __restrict__ amax_b = amax_b0;
+  float inv_denom_b = inv_denom_b0;
+  uint16_t* __restrict__ D = D0;
+  int64_t ldd = ldd0;
+  const uint16_t* __restrict__ bias = epi.bias;
+  const int act = epi.act;
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+
+  // Workgroup -> tile.  The grid is the number of tiles rounded up to a multiple of 8; workgroup b runs on XCD b % 8,
+  // and every XCD takes a run of consecutive tiles (whole column panels first), so that its L2 holds the A rows once
+  // and few B panels.
+  const int total = tiles_m * tiles_n;
+  const int per_xcd = (int)gridDim.x >> 3;
+  const int tile = ((int)blockIdx.x & 7) * per_xcd + ((int)blockIdx.x >> 3);
+  if (tile >= total) return;
+  int tile_n = tile / tiles_m;
+  const int tile_m = tile - tile_n * tiles_m;
+  if (groups.n > 1) {
+    const int g = tile_n / groups.tiles_n_each;
+    tile_n -= g * groups.tiles_n_each;
+    if (g > 0) {
+      const GemmGroup& gg = groups.more[g - 1];
+      Bv = gg.Bv;
+      Bs = gg.Bs;
+      alpha_ptr = gg.alpha;
+      amax_b = gg.amax_b;
+      inv_denom_b = gg.inv_denom_b;
+      D = gg.D;
+      ldd = gg.ldd;
+      bias = gg.bias;
+      epi.sink = gg.sink;
+    }
+  }
+  const int row0 = tile_m * BM, col0 = tile_n * BN;
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, lh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = wave >> 2, wm = wave & 1, wn = (wave >> 1) & 1;
+
+  const uint32_t row_bytes = (uint32_t)Kp >> 1;
+  const uint32_t swz = (l32 >> 2) & 3;
+  const uint32_t lane_voff = (uint32_t)(lane >> 2) * row_bytes + 16u * ((lane & 3) ^ ((lane >> 4) & 3));
+  const uint32_t lane_soff = (uint32_t)lane * 16u;
+  // the lane's 16-byte piece of this wave's half of a K step: piece 2 half + lane / 32, stored at piece ^ swz
+  const uint32_t lane_rd = ((uint32_t)l32 * 64u + 16u * ((lh ^ (swz & 1)) | (swz & 2))) ^ (32u * half);
+  const uint32_t ard = (uint32_t)(32 * FA * wm) * 64u + lane_rd;
+  const uint32_t brd = (uint32_t)(BM * 64) + (uint32_t)(32 * FB * wn) * 64u + lane_rd;
+  // scales of a K step and a 128-row group: two halves of 512 bytes, 16 bytes per row of 32 and half
+  const uint32_t sard = T::kAScales + 512u * half + (uint32_t)l32 * 16u + 8u * wm;
+  const uint32_t sbrd = T::kBScales + 512u * half + 1024u * wn + (uint32_t)l32 * 16u;
+  const uint32_t sh = 16u * lh;
+  // loads of a K step: wave w brings 16 rows of A, 32 rows of B, and (waves 0-2) one 1 KB block of scales
+  const int a_rows = min(row0 + 16 * wave, Mp - 16), b_rows = min(col0 + 32 * wave, Np - 32);
+  const uint8_t* sA = Av + (size_t)a_rows * row_bytes;
+  const uint8_t* sB = Bv + (size_t)b_rows * row_bytes;
+  const int block = min(wave, T::kScaleBlocks - 1);
+  const uint8_t* sS = block < BM / 128 ? As + (size_t)min((row0 >> 7) + block, (Mp >> 7) - 1) * (size_t)(Kp >> 6) * 512
+                                       : Bs + (size_t)min((col0 >> 7) + block - BM / 128, (Np >> 7) - 1) * (size_t)(Kp >> 6) * 512;
+  const uint32_t adst = (uint32_t)wave * 1024u, bdst = (uint32_t)(BM * 64) + (uint32_t)wave * 2048u;
+  const uint32_t sdst = T::kAScales + 1024u * (uint32_t)block;
+  const uint32_t hassc = __builtin_amdgcn_readfirstlane(wave < T::kScaleBlocks ? 1 : 0);
+  const uint32_t nsteps = (uint32_t)Kp >> 7, rb16 = 16u * row_bytes;
+  const uint32_t idle = __builtin_amdgcn_readfirstlane(row0 + wm * 32 * FA < M && col0 + wn * 32 * FB < N ? 0 : 1);
+
+  float16v acc[FB][FA];
+#pragma unroll
+  for (int g = 0; g < FB; ++g)
+#pragma unroll
+    for (int f = 0; f < FA; ++f)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[g][f][i] = 0.0f;
+  asm volatile(
+#include "gemm_tile_loop_24w8_gfx950.inc"
+      : "+a"(acc[0][0]), "+a"(acc[0][1]), "+a"(acc[1][0]), "+a"(acc[1][1]), "+a"(acc[2][0]), "+a"(acc[2][1]), "+a"(acc[3][0]),
+        "+a"(acc[3][1])
+      : LL_ASM_TILE_INPUTS, "s"(hassc)
+      : "memory", "scc", "vcc", "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", LL_V10(1), LL_V10(2), LL_V10(3),
+        LL_V10(4), LL_V10(5), LL_V10(6), LL_V10(7), LL_V10(8), LL_V10(9), "v100", "v101", LL_ASM_TILE_SGPRS);
+  __syncthreads();  // every wave has left the ring
+
+  // Exchange: 16 KB per receiving wave, [register / 4][lane][4 floats].  Waves 0-3 keep their first 32 rows, waves 4-7
+  // their second 32 (selects instead of two code paths: the choice is uniform and made once per tile).
+  float* out = reinterpret_cast<float*>(smem) + (size_t)(wave ^ 4) * 4096 + lane * 4;
+  const float* in = reinterpret_cast<const float*>(smem) + (size_t)wave * 4096 + lane * 4;
+  float16v kept[FB][1];
+#pragma unroll
+  for (int g = 0; g < FB; ++g)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      float send[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float first = acc[g][0][4 * q + i], second = acc[g][1][4 * q + i];
+        send[i] = half ? first : second;
+        kept[g][0][4 * q + i] = half ? second : first;
+      }
+      *reinterpret_cast<float4*>(out + (4 * g + q) * 256) = make_float4(send[0], send[1], send[2], send[3]);
+    }
+  __syncthreads();
+#pragma unroll
+  for (int g = 0; g < FB; ++g)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const float4 v = *reinterpret_cast<const float4*>(in + (4 * g + q) * 256);
+      kept[g][0][4 * q] += v.x;
+      kept[g][0][4 * q + 1] += v.y;
+      kept[g][0][4 * q + 2] += v.z;
+      kept[g][0][4 * q + 3] += v.w;
+    }
+  __syncthreads();  // the patches of the epilogue overlap the exchange
+  float alpha;
+  if (alpha_ptr) {
+    alpha = alpha_ptr[0];
+  } else {
+    alpha = (amax_a[0] * amax_b[0]) * (inv_denom_a * inv_denom_b);
+  }
+  gemm_epilogue<1, FB>(kept, alpha, smem, wave, lane, row0 + wm * 32 * FA + 32 * half, col0 + wn * 32 * FB, M, N, D, ldd, bias, act,
+                       epi, (uint32_t)blockIdx.x * 8 + wave);
+}
 #undef LL_ASM_TILE_SGPRS
 #undef LL_ASM_TILE_INPUTS
 #undef LL_V10
@@ -1055,6 +1199,29 @@ int dispatch_gemm(const uint8_t* A_values, const uint8_t* A_scales, const uint8_
     if (int rc = try_persistent(A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, M, N, Np, Kp, D, ldd,
                                 epi, groups, s, &launched)) return rc;
     if (launched) return LL_OK;
+  }
+  // At most one 128 x 256 tile per compute unit, and more than half of the units busy: one workgroup of eight waves
+  // per tile, the K range of every step split between its two halves.
+  if (Kp % 128 == 0 && Kp >= 512 && g_gemm_schedule.load(std::memory_order_relaxed) != LL_GEMM_TILES_COMPILED) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) != hipSuccess) {
+      set_error("ll_nvfp4_gemm_tnt: hipGetDevice failed");
+      return LL_ELAUNCH;
+    }
+    if (int rc = compute_units_of(dev, cus, "ll_nvfp4_gemm_tnt")) return rc;
+    GemmGroups gr = groups;
+    gr.tiles_n_each = (int)((N + 255) / 256);
+    const int tiles_m = (int)((M + 127) / 128), tiles_n = gr.tiles_n_each * gr.n;
+    const int64_t tiles = (int64_t)tiles_m * tiles_n;
+    if (tiles <= cus && 2 * tiles > cus) {
+      static std::atomic<uint64_t> lds_allowed{0};
+      if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_w4a4_asm8_kernel), kSplitSmem, lds_allowed, "ll_nvfp4_gemm_tnt")) return rc;
+      hipLaunchKernelGGL(gemm_w4a4_asm8_kernel, dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(kSplitThreads), kSplitSmem, s, A_values,
+                         A_scales, B_values, B_scales, alpha, amax_a, amax_b, 1.0f / denom_a, 1.0f / denom_b, (int)M, (int)N, (int)Mp,
+                         (int)Np, (int)Kp, static_cast<uint16_t*>(D), ldd, tiles_m, tiles_n, epi, gr);
+      LL_CHECK_LAUNCH("gemm_w4a4_asm8_kernel");
+      return LL_OK;
+    }
   }
   const int64_t n_all = N * groups.n;
   // Tile choice.  Two workgroups are resident per CU (512 slots on 256 CUs).  The 256x128 / 128x256

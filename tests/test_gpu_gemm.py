@@ -446,6 +446,58 @@ def _ulp_close(a, b, frac=1e-3):
     assert float((diff != 0).float().mean()) <= frac
 
 
+@pytest.mark.parametrize("M,N,K,groups", [
+    (2640, 3072, 3072, 1),    # the projections of the DiT block: 252 tiles of 128 x 256
+    (2640, 3072, 14336, 1),   # FFN-down
+    (1300, 5000, 640, 1),     # ragged M and N (waves without output rows), five K steps
+    (2100, 2100, 512, 1),     # waves without output columns, four K steps
+    (880, 3072, 1024, 3),     # three products in one launch
+])
+def test_one_workgroup_per_unit_with_k_split_between_its_halves(gpu, M, N, K, groups):
+    """Shapes that give at most one 128 x 256 tile per compute unit (and fill more than half of the units) run as
+    one workgroup of eight waves per tile, the two halves of every K step summed separately and added through LDS:
+    the same exact products as the other tile kernels added in another order.  Against the compiled kernel within
+    one bf16 ulp of the fp32 sum, twice for identical bits, against the oracle (1e-3 relative Frobenius) where it
+    finishes in seconds; bias, GELU, gated residual and the amax sinks go through the same epilogue."""
+    cfg = QuantizationConfig(scale_rule="mse")
+    xq = quantize_to_fp4(activations((M, K), 15).to(gpu), cfg)
+    ws = [quantize_to_fp4((weights((N, K), 16 + i) * (1 + i)).to(gpu), cfg) for i in range(groups)]
+    gen = torch.Generator().manual_seed(17)
+    bias = (torch.randn(N, generator=gen) * 0.1).to(gpu).bfloat16()
+    frame = M // 4 if M % 4 == 0 else M
+    residual = torch.randn(M, N, generator=gen).bfloat16().to(gpu)
+    gate = torch.randn(M // frame, 6, N, generator=gen).bfloat16().to(gpu)[:, 2]
+    out = {}
+    for sched in ("tiles_compiled", "tiles", "tiles"):
+        with _native.gemm_schedule(sched):
+            if groups == 1:
+                t = _native.amax_ticket(gpu)
+                y = [fp4_matmul(xq, ws[0], bias=bias, activation="gelu_tanh", amax_out=t)]
+                amax = [float(quantize_to_fp4(y[0], cfg, amax=t).amax)]
+                if N % 8 == 0:
+                    y.append(fp4_matmul(xq, ws[0], bias=bias, residual=residual, gate=gate, gate_rows=frame))
+                y.append(fp4_matmul(xq, ws[0]))
+            else:
+                sinks = [_native.PrivateAmaxSink(gpu) for _ in range(groups)]
+                products = [dict(values=w.values, scales=w.scale_factors, amax=w.amax, denom=1536.0, bias=bias if i != 1 else None,
+                                 amax_out=s.ticket()) for i, (w, s) in enumerate(zip(ws, sinks))]
+                y = list(_native.gemm_grouped(xq.values, xq.scale_factors, xq.amax, 1536.0, M, N, products))
+                amax = [float(quantize_to_fp4(yi, cfg, amax=pr["amax_out"]).amax) for yi, pr in zip(y, products)]
+        out.setdefault(sched, []).append((y, amax))
+    (want, _), = out["tiles_compiled"]
+    (got, amax), (again, amax_again) = out["tiles"]
+    for a, b in zip(got, again):
+        assert torch.equal(a, b)
+    assert amax == amax_again
+    for a, b in zip(got, want):
+        _ulp_close(a, b, frac=5e-3)
+    n_sinks = 1 if groups == 1 else groups
+    assert amax == [float(yi.float().abs().max()) for yi in got[:n_sinks]]
+    if M * N * K <= 3e10 and groups == 1:
+        ref = o.fp4_matmul(_as_oracle(xq), _as_oracle(ws[0]))
+        assert _rel(got[-1].float().cpu().numpy(), ref) <= TOL
+
+
 @pytest.mark.parametrize("M,N,K", [(300, 1100, 5120), (2640, 3072, 3072), (130, 513, 12800), (1000, 2048, 14336)])
 def test_persistent_schedule_against_the_oracle_and_the_tile_schedule(gpu, M, N, K):
     """The persistent launch (one workgroup per compute unit, 128 x 512 tiles, the K range of the tiles behind the
