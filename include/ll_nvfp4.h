@@ -216,8 +216,12 @@ int ll_nvfp4_gemm_tnt_grouped(const uint8_t* A_values, const uint8_t* A_scales, 
 /*
  * The GEMM entry points can run one of two kernels.  LL_GEMM_TILES: one workgroup per output tile, two workgroups
  * per compute unit; where Kp is a multiple of 128, the tiles of 256 x 128 and 128 x 256 run their main loop as a
- * hand-scheduled instruction sequence (same arithmetic in the same order as the compiled loop: identical bits;
- * LL_GEMM_TILES_COMPILED takes the compiled loop everywhere, for comparisons).  LL_GEMM_PERSISTENT (wherever Kp is a multiple of 128 and there is at least one K step per
+ * hand-scheduled instruction sequence (same arithmetic in the same order as the compiled loop: identical bits), and
+ * a shape that gives at most one 128 x 256 tile per compute unit (and fills more than half of them) runs as one
+ * workgroup of eight waves per tile, which sums the two halves of every K step of 128 separately and adds them at
+ * the end (deterministic; differs from the other kernels by the order of the fp32 additions).
+ * LL_GEMM_TILES_COMPILED takes the compiled loop and one workgroup of four waves per tile everywhere, for
+ * comparisons.  LL_GEMM_PERSISTENT (wherever Kp is a multiple of 128 and there is at least one K step per
  * compute unit): one workgroup per compute unit, output tiles of 128 x 512, whole rounds of tiles first and the
  * (tile, K step) pairs of the tiles behind them cut into equal shares, so that no compute unit waits for another
  * (the reference's kernel is a persistent tile scheduler too, csrc/fp4_gemm.cu:67-92).  A tile whose K range is

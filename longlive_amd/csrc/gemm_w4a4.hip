@@ -982,10 +982,14 @@ __global__ __launch_bounds__(kSplitThreads) void gemm_w4a4_asm8_kernel(
         LL_V10(4), LL_V10(5), LL_V10(6), LL_V10(7), LL_V10(8), LL_V10(9), "v100", "v101", LL_ASM_TILE_SGPRS);
   __syncthreads();  // every wave has left the ring
 
+  // Everything behind the loop is computed from this copy of the lane number: the loop leaves the compiler 26
+  // registers, and what it would otherwise prepare for the epilogue ahead of the loop does not fit them.
+  int lane_after = lane;
+  asm volatile("" : "+v"(lane_after));
   // Exchange: 16 KB per receiving wave, [register / 4][lane][4 floats].  Waves 0-3 keep their first 32 rows, waves 4-7
   // their second 32 (selects instead of two code paths: the choice is uniform and made once per tile).
-  float* out = reinterpret_cast<float*>(smem) + (size_t)(wave ^ 4) * 4096 + lane * 4;
-  const float* in = reinterpret_cast<const float*>(smem) + (size_t)wave * 4096 + lane * 4;
+  float* out = reinterpret_cast<float*>(smem) + (size_t)(wave ^ 4) * 4096 + lane_after * 4;
+  const float* in = reinterpret_cast<const float*>(smem) + (size_t)wave * 4096 + lane_after * 4;
   float16v kept[FB][1];
 #pragma unroll
   for (int g = 0; g < FB; ++g)
@@ -1018,7 +1022,7 @@ __global__ __launch_bounds__(kSplitThreads) void gemm_w4a4_asm8_kernel(
   } else {
     alpha = (amax_a[0] * amax_b[0]) * (inv_denom_a * inv_denom_b);
   }
-  gemm_epilogue<1, FB>(kept, alpha, smem, wave, lane, row0 + wm * 32 * FA + 32 * half, col0 + wn * 32 * FB, M, N, D, ldd, bias, act,
+  gemm_epilogue<1, FB>(kept, alpha, smem, wave, lane_after, row0 + wm * 32 * FA + 32 * half, col0 + wn * 32 * FB, M, N, D, ldd, bias, act,
                        epi, (uint32_t)blockIdx.x * 8 + wave);
 }
 #undef LL_ASM_TILE_SGPRS
