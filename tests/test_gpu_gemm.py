@@ -498,6 +498,30 @@ def test_one_workgroup_per_unit_with_k_split_between_its_halves(gpu, M, N, K, gr
         assert _rel(got[-1].float().cpu().numpy(), ref) <= TOL
 
 
+def test_eight_wave_kernel_recorded_into_a_graph(gpu):
+    """The eight-wave kernel allocates nothing and waits for no other workgroup: recorded into a graph it replays
+    with fresh operands, every replay equal to the eager result bit for bit."""
+    cfg = QuantizationConfig(scale_rule="mse")
+    M, N, K = 2640, 3072, 1024
+    x = activations((M, K), 61).to(gpu)
+    wq = quantize_to_fp4(weights((N, K), 62).to(gpu), cfg)
+    xq = quantize_to_fp4(x, cfg)
+    fp4_matmul(xq, wq)  # first use outside the recording
+    side = torch.cuda.Stream(device=gpu)
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        out = fp4_matmul(xq, wq)
+    for seed in (63, 64, 65):
+        fresh = quantize_to_fp4(activations((M, K), seed).to(gpu), cfg)
+        xq.values.copy_(fresh.values), xq.scale_factors.copy_(fresh.scale_factors), xq.amax.copy_(fresh.amax)
+        torch.cuda.synchronize()
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, fp4_matmul(xq, wq))
+
+
 @pytest.mark.parametrize("M,N,K", [(300, 1100, 5120), (2640, 3072, 3072), (130, 513, 12800), (1000, 2048, 14336)])
 def test_persistent_schedule_against_the_oracle_and_the_tile_schedule(gpu, M, N, K):
     """The persistent launch (one workgroup per compute unit, 128 x 512 tiles, the K range of the tiles behind the
@@ -606,7 +630,7 @@ def test_persistent_schedule_on_a_capturing_stream(gpu):
     (2640, 14336, 3072, 1),   # 256 x 128 tiles: FFN-up
     (2688, 4096, 128, 1),     # one K step
     (513, 14336, 256, 1),     # ragged M, two steps
-    (2640, 3072, 3072, 1),    # 128 x 128 tiles: the projections
+    (7040, 3072, 1024, 1),    # the projections at the released chunk size
     (2600, 14300, 1152, 1),   # 256 x 128 tiles, ragged M and N, an odd number of steps
     (12763, 379, 384, 1),     # 128 x 256 tiles, ragged M and N
     (2640, 3072, 3072, 3),    # 128 x 256 tiles: q, k, v in one launch
@@ -615,8 +639,8 @@ def test_persistent_schedule_on_a_capturing_stream(gpu):
 def test_hand_scheduled_main_loop_is_bit_identical_to_the_compiled_one(gpu, M, N, K, groups):
     """The one-workgroup-per-tile kernels with tiles of 256 x 128 and 128 x 256 run their main loop as a generated
     instruction sequence wherever K is a multiple of 128; every accumulator receives the same products in the same
-    order as in the compiler's loop, so outputs and the amax left in the sinks are equal bit for bit.  (The shapes
-    that take 128 x 128 tiles run the compiler's loop under either setting.)"""
+    order as in the compiler's loop, so outputs and the amax left in the sinks are equal bit for bit.  (Shapes that
+    take the eight-wave kernel, whose sums are formed in another order, have a test of their own.)"""
     cfg = QuantizationConfig(scale_rule="mse")
     xq = quantize_to_fp4(activations((M, K), 5).to(gpu), cfg)
     ws = [quantize_to_fp4((weights((N, K), 6 + i) * (1 + i)).to(gpu), cfg) for i in range(groups)]
