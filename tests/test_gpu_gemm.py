@@ -282,8 +282,15 @@ def test_amax_sink_of_the_epilogue_feeds_the_next_quantization(gpu):
 def test_products_that_share_their_input_in_one_launch_equal_the_separate_launches(gpu, M, N, K, n):
     """ll_nvfp4_gemm_tnt_grouped (the q / k / v projections of one activation): every product - own weight, tensor
     scale, bias and amax sink - is bit for bit what the single call computes, at ragged and at full sizes; the
-    quantized linear layers take that path through forward_quantized_together."""
+    quantized linear layers take that path through forward_quantized_together.  (With one summation order for every
+    shape: a single 2640 x 3072 product would otherwise take the kernel that sums the halves of K separately,
+    three of them in one launch the large tiles.)"""
     from longlive_amd import _native
+    with _native.gemm_schedule("tiles_compiled"):
+        _grouped_equals_separate(gpu, M, N, K, n)
+
+
+def _grouped_equals_separate(gpu, M, N, K, n):
     cfg = QuantizationConfig(scale_rule="mse")
     xq = quantize_to_fp4(activations((M, K), 61).to(gpu), cfg)
     ws = [quantize_to_fp4((weights((N, K), 62 + i) * (1 + i)).to(gpu), cfg) for i in range(n)]
