@@ -766,7 +766,7 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_asm_kernel(
   int64_t ldd = ldd0;
   const uint16_t* __restrict__ bias = epi.bias;
   const int act = epi.act;
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // the loop forms addresses by xor: whole pieces of 64 bytes
 
   // Workgroup -> tile, as in gemm_w4a4_kernel.
   int wg = blockIdx.x;
@@ -820,12 +820,13 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_asm_kernel(
   const uint32_t swz = (l32 >> 2) & 3;
   const uint32_t lane_voff = (uint32_t)(lane >> 2) * row_bytes + 16u * ((lane & 3) ^ ((lane >> 4) & 3));
   const uint32_t lane_soff = (uint32_t)lane * 16u;
-  const uint32_t lane_rd = (uint32_t)l32 * 64u + 16u * ((lh ^ (swz & 1)) | (swz & 2));
+  const uint32_t lds0 = lds_address(smem);  // the loop addresses LDS with plain offsets: they start where smem does
+  const uint32_t lane_rd = lds0 + (uint32_t)l32 * 64u + 16u * ((lh ^ (swz & 1)) | (swz & 2));
   const uint32_t ard = (uint32_t)(32 * FA * wm) * 64u + lane_rd;
   const uint32_t brd = (uint32_t)(BM * 64) + (uint32_t)(32 * FB * wn) * 64u + lane_rd;
   // a wave with four fragments of an operand owns a whole 128-row group of its scales, one with two owns half of one
-  const uint32_t sard = T::kAScales + (uint32_t)l32 * 16u + (FA == 4 ? 1024u : 8u) * wm;
-  const uint32_t sbrd = T::kBScales + (uint32_t)l32 * 16u + (FB == 4 ? 1024u : 8u) * wn;
+  const uint32_t sard = lds0 + T::kAScales + (uint32_t)l32 * 16u + (FA == 4 ? 1024u : 8u) * wm;
+  const uint32_t sbrd = lds0 + T::kBScales + (uint32_t)l32 * 16u + (FB == 4 ? 1024u : 8u) * wn;
   const uint32_t sh = 16u * lh;
   const int a_rows = min(row0 + (BM / 4) * wave, Mp - BM / 4), b_rows = min(col0 + (BN / 4) * wave, Np - BN / 4);
   const uint8_t* sA = Av + (size_t)a_rows * row_bytes;
@@ -835,8 +836,8 @@ __global__ __launch_bounds__(kGemmThreads, 2) void gemm_w4a4_asm_kernel(
   const int block = min(wave, T::kScaleBlocks - 1);
   const uint8_t* sS = block < BM / 128 ? As + (size_t)min((row0 >> 7) + block, (Mp >> 7) - 1) * (size_t)(Kp >> 6) * 512
                                        : Bs + (size_t)min((col0 >> 7) + block - BM / 128, (Np >> 7) - 1) * (size_t)(Kp >> 6) * 512;
-  const uint32_t adst = (uint32_t)wave * (BM / 4) * 64u, bdst = (uint32_t)(BM * 64) + (uint32_t)wave * (BN / 4) * 64u;
-  const uint32_t sdst = T::kAScales + 1024u * (uint32_t)block;
+  const uint32_t adst = lds0 + (uint32_t)wave * (BM / 4) * 64u, bdst = lds0 + (uint32_t)(BM * 64) + (uint32_t)wave * (BN / 4) * 64u;
+  const uint32_t sdst = lds0 + T::kAScales + 1024u * (uint32_t)block;
   const uint32_t nsteps = (uint32_t)Kp >> 7, rb16 = 16u * row_bytes;
   // A wave whose rows (or columns) all lie beyond M (N) only helps with the staging.
   const uint32_t idle = __builtin_amdgcn_readfirstlane(row0 + wm * 32 * FA < M && col0 + wn * 32 * FB < N ? 0 : 1);
@@ -909,7 +910,7 @@ __global__ __launch_bounds__(kSplitThreads) void gemm_w4a4_asm8_kernel(
   int64_t ldd = ldd0;
   const uint16_t* __restrict__ bias = epi.bias;
   const int act = epi.act;
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];  // the loop forms addresses by xor: whole pieces of 64 bytes
 
   // Workgroup -> tile.  The grid is the number of tiles rounded up to a multiple of 8; workgroup b runs on XCD b % 8,
   // and every XCD takes a run of consecutive tiles (whole column panels first), so that its L2 holds the A rows once
@@ -946,12 +947,13 @@ __global__ __launch_bounds__(kSplitThreads) void gemm_w4a4_asm8_kernel(
   const uint32_t lane_voff = (uint32_t)(lane >> 2) * row_bytes + 16u * ((lane & 3) ^ ((lane >> 4) & 3));
   const uint32_t lane_soff = (uint32_t)lane * 16u;
   // the lane's 16-byte piece of this wave's half of a K step: piece 2 half + lane / 32, stored at piece ^ swz
-  const uint32_t lane_rd = ((uint32_t)l32 * 64u + 16u * ((lh ^ (swz & 1)) | (swz & 2))) ^ (32u * half);
+  const uint32_t lds0 = lds_address(smem);  // the loop addresses LDS with plain offsets: they start where smem does
+  const uint32_t lane_rd = lds0 + (((uint32_t)l32 * 64u + 16u * ((lh ^ (swz & 1)) | (swz & 2))) ^ (32u * half));
   const uint32_t ard = (uint32_t)(32 * FA * wm) * 64u + lane_rd;
   const uint32_t brd = (uint32_t)(BM * 64) + (uint32_t)(32 * FB * wn) * 64u + lane_rd;
   // scales of a K step and a 128-row group: two halves of 512 bytes, 16 bytes per row of 32 and half
-  const uint32_t sard = T::kAScales + 512u * half + (uint32_t)l32 * 16u + 8u * wm;
-  const uint32_t sbrd = T::kBScales + 512u * half + 1024u * wn + (uint32_t)l32 * 16u;
+  const uint32_t sard = lds0 + T::kAScales + 512u * half + (uint32_t)l32 * 16u + 8u * wm;
+  const uint32_t sbrd = lds0 + T::kBScales + 512u * half + 1024u * wn + (uint32_t)l32 * 16u;
   const uint32_t sh = 16u * lh;
   // loads of a K step: wave w brings 16 rows of A, 32 rows of B, and (waves 0-2) one 1 KB block of scales
   const int a_rows = min(row0 + 16 * wave, Mp - 16), b_rows = min(col0 + 32 * wave, Np - 32);
@@ -960,8 +962,8 @@ __global__ __launch_bounds__(kSplitThreads) void gemm_w4a4_asm8_kernel(
   const int block = min(wave, T::kScaleBlocks - 1);
   const uint8_t* sS = block < BM / 128 ? As + (size_t)min((row0 >> 7) + block, (Mp >> 7) - 1) * (size_t)(Kp >> 6) * 512
                                        : Bs + (size_t)min((col0 >> 7) + block - BM / 128, (Np >> 7) - 1) * (size_t)(Kp >> 6) * 512;
-  const uint32_t adst = (uint32_t)wave * 1024u, bdst = (uint32_t)(BM * 64) + (uint32_t)wave * 2048u;
-  const uint32_t sdst = T::kAScales + 1024u * (uint32_t)block;
+  const uint32_t adst = lds0 + (uint32_t)wave * 1024u, bdst = lds0 + (uint32_t)(BM * 64) + (uint32_t)wave * 2048u;
+  const uint32_t sdst = lds0 + T::kAScales + 1024u * (uint32_t)block;
   const uint32_t hassc = __builtin_amdgcn_readfirstlane(wave < T::kScaleBlocks ? 1 : 0);
   const uint32_t nsteps = (uint32_t)Kp >> 7, rb16 = 16u * row_bytes;
   const uint32_t idle = __builtin_amdgcn_readfirstlane(row0 + wm * 32 * FA < M && col0 + wn * 32 * FB < N ? 0 : 1);
