@@ -451,3 +451,21 @@ def test_persistent_gemm_plan_for_the_benchmark_shapes():
     assert not _native.gemm_plan(2640, 3072, 14336, schedule="tiles")["persistent"]
     assert not _native.gemm_plan(2640, 3072, 14336 + 64, schedule="persistent")["persistent"]
     assert not _native.gemm_plan(64, 64, 128, schedule="persistent")["persistent"]
+
+
+def test_generated_gemm_loops_in_the_tree_are_what_their_generators_write(tmp_path):
+    """The hand-scheduled main loops are generated text kept in the tree; a generator edited without regenerating
+    (or a generated file edited by hand) would build a library that no longer matches its source."""
+    import os
+    import subprocess
+    import sys
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "longlive_amd", "csrc")
+    cases = [("gemm_loop_gfx950.inc", ["gemm_loop_gen.py", "{out}"]),
+             ("gemm_tile_loop_42_gfx950.inc", ["gemm_tile_loop_gen.py", "4", "2", "{out}"]),
+             ("gemm_tile_loop_24_gfx950.inc", ["gemm_tile_loop_gen.py", "2", "4", "{out}"]),
+             ("gemm_tile_loop_24w8_gfx950.inc", ["gemm_tile_loop_gen.py", "2", "4", "{out}", "--waves", "8"])]
+    for name, cmd in cases:
+        out = str(tmp_path / name)
+        subprocess.run([sys.executable, os.path.join(csrc, cmd[0])] + [a.format(out=out) for a in cmd[1:]], check=True, cwd=csrc)
+        with open(out) as got, open(os.path.join(csrc, name)) as kept:
+            assert got.read() == kept.read(), name
