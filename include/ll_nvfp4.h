@@ -245,6 +245,19 @@ int ll_nvfp4_gemm_reserve(int64_t M, int64_t N, int64_t Kp, int n_products, void
  * Output pointers may be NULL. */
 int ll_nvfp4_gemm_plan(int64_t M, int64_t N, int64_t Kp, int n_products, int compute_units, int schedule,
                        int* persistent, uint32_t* workgroups, uint32_t* tiles, uint32_t* k_steps);
+/* Which kernel a launch of these sizes runs on a device with `compute_units` CUs under `schedule` (host arithmetic
+ * only; a persistent launch on a capturing stream without memory falls back to the tile kernels, which this does not
+ * see): *kernel = one of the codes below, *hand_scheduled = 1 if its main loop is the generated instruction sequence.
+ * The four-wave tile kernels add the K steps in order; LL_GEMM_KERNEL_EIGHT_WAVES and LL_GEMM_KERNEL_PERSISTENT form
+ * partial sums over parts of K.  Output pointers may be NULL.  No counterpart in the reference. */
+#define LL_GEMM_KERNEL_64X64 0       /* four waves per tile, two workgroups per compute unit */
+#define LL_GEMM_KERNEL_128X128 1
+#define LL_GEMM_KERNEL_128X256 2
+#define LL_GEMM_KERNEL_256X128 3
+#define LL_GEMM_KERNEL_EIGHT_WAVES 4 /* 128 x 256 tiles, eight waves per tile, one workgroup per compute unit */
+#define LL_GEMM_KERNEL_PERSISTENT 5  /* 128 x 512 tiles, one workgroup per compute unit over several tiles */
+int ll_nvfp4_gemm_kernel(int64_t M, int64_t N, int64_t Kp, int n_products, int compute_units, int schedule, int* kernel,
+                         int* hand_scheduled);
 
 /*
  * Replaces torch.ops.longlive_kernels.dequantize_kv_cache_fp4 (utils/kernel/kv_dequant.cpp:14,

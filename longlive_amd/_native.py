@@ -87,6 +87,7 @@ _SIGNATURES = {
     "ll_nvfp4_gemm_get_schedule": (c_int, []),
     "ll_nvfp4_gemm_reserve": (c_int, [c_int64, c_int64, c_int64, c_int, c_void_p]),
     "ll_nvfp4_gemm_plan": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ll_nvfp4_gemm_kernel": (c_int, [c_int64, c_int64, c_int64, c_int, c_int, c_int, c_void_p, c_void_p]),
     "ll_kv_attention_reserve": (c_int, [c_int64, c_int, c_int64, c_void_p]),
     "ll_kv_attention_release": (c_int, [c_void_p]),
     "ll_nvfp4_quantize_noalloc_max_elements": (c_int64, []),
@@ -502,6 +503,18 @@ def gemm_plan(M: int, N: int, Kp: int, n_products: int = 1, compute_units: int =
     _check(load().ll_nvfp4_gemm_plan(M, N, Kp, n_products, compute_units, GEMM_SCHEDULES[schedule], ctypes.byref(persistent),
                                      ctypes.byref(groups), ctypes.byref(tiles), ctypes.byref(steps)), "ll_nvfp4_gemm_plan")
     return {"persistent": bool(persistent.value), "workgroups": groups.value, "tiles": tiles.value, "k_steps": steps.value}
+
+
+GEMM_KERNELS = ("64x64", "128x128", "128x256", "256x128", "eight_waves", "persistent")
+
+
+def gemm_kernel(M: int, N: int, Kp: int, n_products: int = 1, compute_units: int = 256, schedule: str = "auto") -> dict:
+    """Which kernel a GEMM launch of these sizes runs on a device with ``compute_units`` CUs (host arithmetic only):
+    one of GEMM_KERNELS, and whether its main loop is the hand-scheduled one."""
+    kernel, generated = c_int(), c_int()
+    _check(load().ll_nvfp4_gemm_kernel(M, N, Kp, n_products, compute_units, GEMM_SCHEDULES[schedule], ctypes.byref(kernel),
+                                       ctypes.byref(generated)), "ll_nvfp4_gemm_kernel")
+    return {"kernel": GEMM_KERNELS[kernel.value], "hand_scheduled": bool(generated.value)}
 
 
 def gemm_reserve(M: int, N: int, Kp: int, n_products: int = 1, device=None) -> None:

@@ -101,14 +101,12 @@ inline PersistentPlan plan_persistent(int64_t M, int64_t N, int64_t Kp, int n_pr
   const int64_t tiles_m = (M + kPTileM - 1) / kPTileM, tiles_n_each = (N + kPTileN - 1) / kPTileN;
   const int64_t tiles = tiles_m * tiles_n_each * n_products, nk = Kp / 128;
   if (tiles >= (1ll << 30) || tiles * nk < cus) return plan;
-  // The automatic choice never takes the persistent launch.  Its main loop does more MFMAs per cycle and per joule
-  // (sustained, K = 14336: 0.53 - 0.58 of the f16 peak against 0.47 - 0.53), but one wave per SIMD has nobody to hide
-  // a tile's first loads and its epilogue behind, and the tiles behind the whole rounds pay for their partial tiles:
-  // inside the DiT block, with bias, GELU or the gated residual in the epilogue, every product measured slower
-  // (FFN-down 243 against 221 us, FFN-up 300 against 224 us).  Alone, the launch wins where K is long and every
-  // workgroup has at least a whole tile (7040 x 3072 x 14336: 505 against 542 us; 4096 x 4096 x 14336: 355 against
-  // 385 us); an automatic choice that takes it for exactly those shapes left the block of 7040 tokens where it was
-  // (4.55 - 4.57 against 4.54 - 4.55 ms), so it is not made.
+  // The automatic choice never takes the persistent launch.  One wave per SIMD has nobody to hide a tile's first
+  // loads and its epilogue behind, and the tiles behind the whole rounds pay for their partial tiles: inside the DiT
+  // block, with bias, GELU or the gated residual in the epilogue, every product measured slower (FFN-down 243 against
+  // 221 us, FFN-up 300 against 224 us), and where it used to win alone (long K, at least a whole tile per workgroup:
+  // 7040 x 3072 x 14336 in 505 us, 4096 x 4096 x 14336 in 355 us) the hand-scheduled tile kernels have caught up
+  // (483 and 359 us).
   if (schedule == -1 /* LL_GEMM_AUTO */) return plan;
   int64_t rounds = tiles / cus;
   // A few left-over tiles would be cut into many thin parts each (or leave workgroups without a single K step, and
@@ -119,6 +117,48 @@ inline PersistentPlan plan_persistent(int64_t M, int64_t N, int64_t Kp, int n_pr
   plan.tiles_m = (int)tiles_m;
   plan.tiles_n_each = (int)tiles_n_each;
   return plan;
+}
+
+// ---- which one-workgroup-per-tile kernel a launch takes (host arithmetic; the values are the header's
+// LL_GEMM_KERNEL_* codes)
+struct TileKernelChoice {
+  int kernel;           // 0: 64 x 64, 1: 128 x 128, 2: 128 x 256, 3: 256 x 128 (four waves); 4: 128 x 256, eight waves
+  bool hand_scheduled;  // the generated main loop
+};
+inline TileKernelChoice choose_tile_kernel(int64_t M, int64_t N, int64_t Kp, int n_products, int cus, int schedule) {
+  const bool generated_ok = Kp % 128 == 0 && schedule != 2 /* LL_GEMM_TILES_COMPILED */;
+  // At most one 128 x 256 tile per compute unit, and more than half of the units busy: one workgroup of eight waves
+  // per tile, the K range of every step split between its two halves.
+  if (generated_ok && Kp >= 512) {
+    const int64_t tiles = ((M + 127) / 128) * ((N + 255) / 256) * n_products;
+    if (tiles <= cus && 2 * tiles > cus) return {4, true};
+  }
+  // Small problems: when even 128 x 128 tiles would occupy at most half of the compute units, 64 x 64 tiles (more
+  // decode work per MFMA, but four times the workgroups) finish sooner.
+  if (((M + 127) / 128) * ((N * n_products + 127) / 128) <= cus / 2) return {0, false};
+  // Two workgroups of four waves are resident per compute unit.  The 256 x 128 / 128 x 256 tiles need 6 decode
+  // instructions per MFMA, the 128 x 128 tile 8, so the larger tiles win unless they fill the slots much worse.  A last
+  // round of at most one workgroup per unit is cheap: alone on its unit a workgroup runs in 0.56 of the time it takes
+  // next to another (measured: 252 tiles of 128 x 256 alone, 59 us, against 504 of 128 x 128 in pairs, 55 us).
+  const int64_t slots = 2 * (int64_t)cus;
+  auto rounds_eff = [&](int bm, int bn) {
+    const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * n_products;
+    const int64_t whole = tiles / slots, rest = tiles % slots;
+    const double time = (double)whole + (rest == 0 ? 0.0 : (rest <= cus ? 0.564 : 1.0));
+    return ((double)tiles / (double)slots) / time;
+  };
+  struct Cfg { int kernel, bm, bn; double bonus; };
+  const Cfg cfgs[3] = {{3, 256, 128, 1.00}, {2, 128, 256, 1.00}, {1, 128, 128, 0.90}};
+  int best = 3;
+  double best_score = -1.0;
+  for (const Cfg& c : cfgs) {
+    const double sc = rounds_eff(c.bm, c.bn) * c.bonus;
+    if (sc > best_score) {
+      best_score = sc;
+      best = c.kernel;
+    }
+  }
+  return {best, generated_ok && best >= 2};
 }
 
 }  // namespace ll

@@ -1206,61 +1206,32 @@ int dispatch_gemm(const uint8_t* A_values, const uint8_t* A_scales, const uint8_
                                 epi, groups, s, &launched)) return rc;
     if (launched) return LL_OK;
   }
-  // At most one 128 x 256 tile per compute unit, and more than half of the units busy: one workgroup of eight waves
-  // per tile, the K range of every step split between its two halves.
-  if (Kp % 128 == 0 && Kp >= 512 && g_gemm_schedule.load(std::memory_order_relaxed) != LL_GEMM_TILES_COMPILED) {
-    int dev = 0, cus = 0;
-    if (hipGetDevice(&dev) != hipSuccess) {
-      set_error("ll_nvfp4_gemm_tnt: hipGetDevice failed");
-      return LL_ELAUNCH;
-    }
-    if (int rc = compute_units_of(dev, cus, "ll_nvfp4_gemm_tnt")) return rc;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    set_error("ll_nvfp4_gemm_tnt: hipGetDevice failed");
+    return LL_ELAUNCH;
+  }
+  if (int rc = compute_units_of(dev, cus, "ll_nvfp4_gemm_tnt")) return rc;
+  const TileKernelChoice choice = choose_tile_kernel(M, N, Kp, groups.n, cus, g_gemm_schedule.load(std::memory_order_relaxed));
+  if (choice.kernel == LL_GEMM_KERNEL_EIGHT_WAVES) {
     GemmGroups gr = groups;
     gr.tiles_n_each = (int)((N + 255) / 256);
     const int tiles_m = (int)((M + 127) / 128), tiles_n = gr.tiles_n_each * gr.n;
     const int64_t tiles = (int64_t)tiles_m * tiles_n;
-    if (tiles <= cus && 2 * tiles > cus) {
-      static std::atomic<uint64_t> lds_allowed{0};
-      if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_w4a4_asm8_kernel), kSplitSmem, lds_allowed, "ll_nvfp4_gemm_tnt")) return rc;
-      hipLaunchKernelGGL(gemm_w4a4_asm8_kernel, dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(kSplitThreads), kSplitSmem, s, A_values,
-                         A_scales, B_values, B_scales, alpha, amax_a, amax_b, 1.0f / denom_a, 1.0f / denom_b, (int)M, (int)N, (int)Mp,
-                         (int)Np, (int)Kp, static_cast<uint16_t*>(D), ldd, tiles_m, tiles_n, epi, gr);
-      LL_CHECK_LAUNCH("gemm_w4a4_asm8_kernel");
-      return LL_OK;
-    }
+    static std::atomic<uint64_t> lds_allowed{0};
+    if (int rc = allow_dynamic_lds(reinterpret_cast<const void*>(&gemm_w4a4_asm8_kernel), kSplitSmem, lds_allowed, "ll_nvfp4_gemm_tnt")) return rc;
+    hipLaunchKernelGGL(gemm_w4a4_asm8_kernel, dim3((unsigned)((tiles + 7) / 8 * 8)), dim3(kSplitThreads), kSplitSmem, s, A_values,
+                       A_scales, B_values, B_scales, alpha, amax_a, amax_b, 1.0f / denom_a, 1.0f / denom_b, (int)M, (int)N, (int)Mp,
+                       (int)Np, (int)Kp, static_cast<uint16_t*>(D), ldd, tiles_m, tiles_n, epi, gr);
+    LL_CHECK_LAUNCH("gemm_w4a4_asm8_kernel");
+    return LL_OK;
   }
-  const int64_t n_all = N * groups.n;
-  // Tile choice.  Two workgroups are resident per CU (512 slots on 256 CUs).  The 256x128 / 128x256
-  // tiles need 6 decode instructions per MFMA, the 128x128 tile 8, so the larger tiles win unless
-  // they fill the slots much worse.  A last round of at most one workgroup per CU is cheap: alone on its CU a
-  // workgroup runs in 0.56 of the time it takes next to another (measured: 252 tiles of 128x256 alone, 59 us,
-  // against 504 of 128x128 in pairs, 55 us).
-  auto rounds_eff = [&](int bm, int bn) {
-    const int64_t tiles = ((M + bm - 1) / bm) * ((N + bn - 1) / bn) * groups.n;
-    const int64_t whole = tiles / 512, rest = tiles % 512;
-    const double time = (double)whole + (rest == 0 ? 0.0 : (rest <= 256 ? 0.564 : 1.0));
-    return ((double)tiles / 512.0) / time;
-  };
-  struct Cfg { int fa, fb; double bonus; };
-  const Cfg cfgs[3] = {{4, 2, 1.00}, {2, 4, 1.00}, {2, 2, 0.90}};
-  int best = 0;
-  double best_score = -1.0;
-  for (int i = 0; i < 3; ++i) {
-    const double sc = rounds_eff(64 * cfgs[i].fa, 64 * cfgs[i].fb) * cfgs[i].bonus;
-    if (sc > best_score) {
-      best_score = sc;
-      best = i;
-    }
-  }
-  // Small problems: when even 128x128 tiles would occupy at most half of the CUs, 64x64 tiles (more decode
-  // work per MFMA, but four times the workgroups) finish sooner.
-  if (((M + 127) / 128) * ((n_all + 127) / 128) <= 128) best = 4;
 #define LL_GEMM_ARGS A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, (int)M, (int)N, \
                      (int)Mp, (int)Np, (int)Kp, D, ldd, epi, groups, s
-  switch (best) {
-    case 0: return launch_gemm<4, 2>(LL_GEMM_ARGS);
-    case 1: return launch_gemm<2, 4>(LL_GEMM_ARGS);
-    case 2: return launch_gemm<2, 2>(LL_GEMM_ARGS);
+  switch (choice.kernel) {
+    case LL_GEMM_KERNEL_256X128: return launch_gemm<4, 2>(LL_GEMM_ARGS);
+    case LL_GEMM_KERNEL_128X256: return launch_gemm<2, 4>(LL_GEMM_ARGS);
+    case LL_GEMM_KERNEL_128X128: return launch_gemm<2, 2>(LL_GEMM_ARGS);
     default: return launch_gemm<1, 1>(LL_GEMM_ARGS);
   }
 #undef LL_GEMM_ARGS
@@ -1328,12 +1299,29 @@ extern "C" int ll_nvfp4_gemm_plan(int64_t M, int64_t N, int64_t Kp, int n_produc
   LL_REQUIRE(M > 0 && N > 0 && Kp > 0 && Kp % 64 == 0 && n_products >= 1 && n_products <= ll::kMaxGemmGroups && compute_units > 0 &&
                  M < (1 << 30) && N < (1 << 30) && Kp < (1 << 30),
              "ll_nvfp4_gemm_plan: bad sizes");
-  LL_REQUIRE(schedule >= LL_GEMM_AUTO && schedule <= LL_GEMM_PERSISTENT, "ll_nvfp4_gemm_plan: unknown schedule %d", schedule);
+  LL_REQUIRE(schedule >= LL_GEMM_AUTO && schedule <= LL_GEMM_TILES_COMPILED, "ll_nvfp4_gemm_plan: unknown schedule %d", schedule);
   const ll::PersistentPlan plan = ll::plan_persistent(M, N, Kp, n_products, compute_units, schedule);
   if (persistent) *persistent = plan.use ? 1 : 0;
   if (workgroups) *workgroups = plan.d.G;
   if (tiles) *tiles = plan.d.tiles;
   if (k_steps) *k_steps = plan.d.nk;
+  return LL_OK;
+}
+
+extern "C" int ll_nvfp4_gemm_kernel(int64_t M, int64_t N, int64_t Kp, int n_products, int compute_units, int schedule,
+                                    int* kernel, int* hand_scheduled) {
+  LL_REQUIRE(M > 0 && N > 0 && Kp > 0 && Kp % 64 == 0 && n_products >= 1 && n_products <= ll::kMaxGemmGroups && compute_units > 0 &&
+                 M < (1 << 30) && N < (1 << 30) && Kp < (1 << 30),
+             "ll_nvfp4_gemm_kernel: bad sizes");
+  LL_REQUIRE(schedule >= LL_GEMM_AUTO && schedule <= LL_GEMM_TILES_COMPILED, "ll_nvfp4_gemm_kernel: unknown schedule %d", schedule);
+  if (ll::plan_persistent(M, N, Kp, n_products, compute_units, schedule).use) {
+    if (kernel) *kernel = LL_GEMM_KERNEL_PERSISTENT;
+    if (hand_scheduled) *hand_scheduled = 1;
+    return LL_OK;
+  }
+  const ll::TileKernelChoice c = ll::choose_tile_kernel(M, N, Kp, n_products, compute_units, schedule);
+  if (kernel) *kernel = c.kernel;
+  if (hand_scheduled) *hand_scheduled = c.hand_scheduled ? 1 : 0;
   return LL_OK;
 }
 

@@ -469,3 +469,27 @@ def test_generated_gemm_loops_in_the_tree_are_what_their_generators_write(tmp_pa
         subprocess.run([sys.executable, os.path.join(csrc, cmd[0])] + [a.format(out=out) for a in cmd[1:]], check=True, cwd=csrc)
         with open(out) as got, open(os.path.join(csrc, name)) as kept:
             assert got.read() == kept.read(), name
+
+
+def test_which_gemm_kernel_the_shapes_of_the_block_take():
+    """ll_nvfp4_gemm_kernel (host arithmetic): on 256 compute units FFN-up takes the 256 x 128 tile and the grouped
+    q / k / v launch the 128 x 256 tile, both with the hand-scheduled loop; the 2640 x 3072 products take the
+    eight-wave kernel; the M = 512 text projections 64 x 64 tiles; a K that is not a multiple of 128, or the schedule
+    that asks for it, the compiled loops; the persistent schedule only when asked for."""
+    k = _native.gemm_kernel
+    assert k(2640, 14336, 3072) == {"kernel": "256x128", "hand_scheduled": True}
+    assert k(2640, 3072, 3072, n_products=3) == {"kernel": "128x256", "hand_scheduled": True}
+    for K in (3072, 14336):
+        assert k(2640, 3072, K) == {"kernel": "eight_waves", "hand_scheduled": True}
+    assert k(1760, 3072, 3072)["kernel"] == "eight_waves" and k(880, 3072, 3072, n_products=3)["kernel"] == "eight_waves"
+    assert k(880, 3072, 3072)["kernel"] != "eight_waves"          # 84 tiles: less than half of the units
+    assert k(7040, 3072, 3072)["kernel"] == "256x128"             # 660 tiles of 128 x 256: more than one per unit
+    assert k(512, 3072, 3072) == {"kernel": "64x64", "hand_scheduled": False}
+    assert k(2640, 3072, 3072 + 64) == {"kernel": "128x128", "hand_scheduled": False}
+    assert k(2640, 3072, 384)["kernel"] == "128x128"              # fewer than four K steps
+    assert k(2640, 3072, 3072, schedule="tiles_compiled") == {"kernel": "128x128", "hand_scheduled": False}
+    assert k(2640, 14336, 3072, schedule="tiles_compiled") == {"kernel": "256x128", "hand_scheduled": False}
+    assert k(2640, 14336, 3072, schedule="persistent") == {"kernel": "persistent", "hand_scheduled": True}
+    assert k(2640, 3072, 3072, compute_units=128)["kernel"] != "eight_waves"   # 252 tiles on 128 units
+    with pytest.raises(Exception):
+        k(0, 3072, 3072)
