@@ -97,7 +97,7 @@ struct PersistentPlan {
 };
 inline PersistentPlan plan_persistent(int64_t M, int64_t N, int64_t Kp, int n_products, int cus, int schedule) {
   PersistentPlan plan{};
-  if (schedule == 0 /* LL_GEMM_TILES */ || schedule == 2 /* LL_GEMM_TILES_COMPILED */ || Kp % 128 != 0 || cus < 1) return plan;
+  if (schedule == 0 /* LL_GEMM_TILES */ || schedule == 2 /* LL_GEMM_TILES_COMPILED */ || Kp % 128 != 0 || Kp >= (1 << 28) || cus < 1) return plan;
   const int64_t tiles_m = (M + kPTileM - 1) / kPTileM, tiles_n_each = (N + kPTileN - 1) / kPTileN;
   const int64_t tiles = tiles_m * tiles_n_each * n_products, nk = Kp / 128;
   if (tiles >= (1ll << 30) || tiles * nk < cus) return plan;
@@ -126,7 +126,8 @@ struct TileKernelChoice {
   bool hand_scheduled;  // the generated main loop
 };
 inline TileKernelChoice choose_tile_kernel(int64_t M, int64_t N, int64_t Kp, int n_products, int cus, int schedule) {
-  const bool generated_ok = Kp % 128 == 0 && schedule != 2 /* LL_GEMM_TILES_COMPILED */;
+  // the generated loops address a row band with 32-bit offsets: 16 rows of Kp / 2 bytes
+  const bool generated_ok = Kp % 128 == 0 && Kp < (1 << 28) && schedule != 2 /* LL_GEMM_TILES_COMPILED */;
   // At most one 128 x 256 tile per compute unit, and more than half of the units busy: one workgroup of eight waves
   // per tile, the K range of every step split between its two halves.
   if (generated_ok && Kp >= 512) {

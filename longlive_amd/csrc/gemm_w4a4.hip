@@ -1036,12 +1036,13 @@ static std::atomic<int> g_gemm_schedule{LL_GEMM_AUTO};
 template <int FA, int FB>
 int launch_gemm(const uint8_t* Av, const uint8_t* As, const uint8_t* Bv, const uint8_t* Bs, const float* alpha,
                 const float* amax_a, const float* amax_b, float denom_a, float denom_b, int M, int N, int Mp, int Np,
-                int Kp, void* D, int64_t ldd, const GemmEpilogue& epi, GemmGroups groups, hipStream_t stream) {
+                int Kp, void* D, int64_t ldd, const GemmEpilogue& epi, GemmGroups groups, hipStream_t stream,
+                bool hand_scheduled) {
   using S = GemmSmem<FA, FB>;
   groups.tiles_n_each = (N + S::BN - 1) / S::BN;
   const int tiles_m = (M + S::BM - 1) / S::BM, tiles_n = groups.tiles_n_each * groups.n;
   if constexpr (FA + FB == 6) {
-    if (Kp % 128 == 0 && g_gemm_schedule.load(std::memory_order_relaxed) != LL_GEMM_TILES_COMPILED) {
+    if (hand_scheduled) {
       // the same kernel with its main loop as a hand-scheduled instruction sequence
       using T = AsmTile<FA, FB>;
       static_assert(2 * T::kStage >= 4 * 32 * (64 * FB + 16), "the epilogue's patches fit the stages");
@@ -1227,7 +1228,7 @@ int dispatch_gemm(const uint8_t* A_values, const uint8_t* A_scales, const uint8_
     return LL_OK;
   }
 #define LL_GEMM_ARGS A_values, A_scales, B_values, B_scales, alpha, amax_a, amax_b, denom_a, denom_b, (int)M, (int)N, \
-                     (int)Mp, (int)Np, (int)Kp, D, ldd, epi, groups, s
+                     (int)Mp, (int)Np, (int)Kp, D, ldd, epi, groups, s, choice.hand_scheduled
   switch (choice.kernel) {
     case LL_GEMM_KERNEL_256X128: return launch_gemm<4, 2>(LL_GEMM_ARGS);
     case LL_GEMM_KERNEL_128X256: return launch_gemm<2, 4>(LL_GEMM_ARGS);
